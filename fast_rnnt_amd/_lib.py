@@ -1,0 +1,82 @@
+"""ctypes binding of libfast_rnnt_amd.so (the gfx950 C-ABI library).
+
+The library is built in-tree by ``make -C fast_rnnt_amd/csrc`` (or
+``__graft_entry__.build()``).  There is no fallback: if it is missing, loading
+raises, and every operator of this package needs it.
+"""
+import ctypes
+import os
+import re
+
+import torch  # noqa: F401  (loads the HIP runtime the library binds to)
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libfast_rnnt_amd.so")
+HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "fast_rnnt_amd.h")
+
+_lib = None
+
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+_F = ctypes.c_float
+_D = ctypes.c_double
+
+# argument lists of the entry points, in header order
+_SIGNATURES = {
+    "frnnt_version": ([], _I),
+    "frnnt_last_error": ([], ctypes.c_char_p),
+    "frnnt_mi_forward_f32": ([_P, _P, _P, _P, _P, _I, _I, _I, _I, _P], _I),
+    "frnnt_mi_forward_f64": ([_P, _P, _P, _P, _P, _I, _I, _I, _I, _P], _I),
+    "frnnt_mi_backward_f32": ([_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P], _I),
+    "frnnt_mi_backward_f64": ([_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P], _I),
+}
+
+
+def declared_symbols():
+    """Names of every function the public header declares."""
+    with open(HEADER_PATH) as f:
+        text = re.sub(r"/\*.*?\*/", "", f.read(), flags=re.S)
+    return sorted(set(re.findall(r"\b(frnnt_[a-z0-9_]+)\s*\(", text)))
+
+
+def load():
+    """Return the loaded library; raises RuntimeError if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `make -C fast_rnnt_amd/csrc` "
+                "(hipcc, gfx950). fast_rnnt_amd has no CPU or eager fallback."
+            )
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (argtypes, restype) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = restype
+        _lib = lib
+    return _lib
+
+
+def call(name, *args):
+    """Invoke an int-returning entry point; raise RuntimeError on a non-zero code."""
+    lib = load()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        raise RuntimeError(f"{name} failed ({rc}): {lib.frnnt_last_error().decode()}")
+
+
+def stream_of(t: "torch.Tensor"):
+    """hipStream_t (as an int) torch is currently using on the tensor's device."""
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def suffix(dtype) -> str:
+    if dtype == torch.float32:
+        return "f32"
+    if dtype == torch.float64:
+        return "f64"
+    raise RuntimeError(f"fast_rnnt_amd supports float32 and float64 tensors, got {dtype}")
+
+
+def ptr(t):
+    return None if t is None else t.data_ptr()

@@ -1,0 +1,82 @@
+// Shared device/host helpers for the gfx950 kernels (wave64, CDNA4).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <limits>
+
+#include "../../include/fast_rnnt_amd.h"
+
+namespace frnnt {
+
+constexpr int kWave = 64;
+
+// ---- host side: thread-local error text --------------------------------------
+char *error_buffer();
+int fail(int code, const char *fmt, ...);
+int check_launch(const char *what);
+
+// ---- device side -----------------------------------------------------------------
+template <typename R>
+struct Num;
+
+template <>
+struct Num<float> {
+  static __device__ __forceinline__ float neg_inf() { return -__builtin_huge_valf(); }
+  // v_exp_f32 / v_log_f32 based; absolute error of log1p(exp(d)) stays below
+  // 1e-7 for d <= 0, far under one ulp of lattice scores of magnitude >= 1.
+  static __device__ __forceinline__ float exp_(float x) { return __expf(x); }
+  static __device__ __forceinline__ float log1p_(float x) { return __logf(1.0f + x); }
+};
+
+template <>
+struct Num<double> {
+  static __device__ __forceinline__ double neg_inf() { return -__builtin_huge_val(); }
+  static __device__ __forceinline__ double exp_(double x) { return exp(x); }
+  static __device__ __forceinline__ double log1p_(double x) { return log1p(x); }
+};
+
+// log(exp(a) + exp(b)) with the reference's handling of non-finite operands
+// (fast_rnnt/csrc/mutual_information.h:36-65): the larger operand is returned
+// untouched when the difference is not a finite number.
+template <typename R>
+__device__ __forceinline__ R log_add(R a, R b) {
+  const bool lt = a < b;
+  const R hi = lt ? b : a;
+  const R gap = lt ? (a - b) : (b - a);
+  if (gap - gap != 0) return hi;
+  return hi + Num<R>::log1p_(Num<R>::exp_(gap));
+}
+
+// Value held by lane-1 (whole-wave shift right by one); lane 0 receives `fill`.
+// DPP wave_shr:1 is a full-rate VALU modifier on gfx9-family parts, no LDS trip.
+__device__ __forceinline__ float from_lane_below(float v, float fill) {
+  const int r = __builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(v), 0x138, 0xf,
+                                            0xf, false);
+  return __int_as_float(r);
+}
+__device__ __forceinline__ double from_lane_below(double v, double fill) {
+  const long long vi = __double_as_longlong(v), fi = __double_as_longlong(fill);
+  const int lo = __builtin_amdgcn_update_dpp((int)(fi & 0xffffffffLL), (int)(vi & 0xffffffffLL),
+                                             0x138, 0xf, 0xf, false);
+  const int hi = __builtin_amdgcn_update_dpp((int)(fi >> 32), (int)(vi >> 32), 0x138, 0xf, 0xf,
+                                             false);
+  return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+
+// Broadcast of lane `src`'s value (src wave-uniform).
+__device__ __forceinline__ float lane_value(float v, int src) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src));
+}
+__device__ __forceinline__ double lane_value(double v, int src) {
+  const long long vi = __double_as_longlong(v);
+  const int lo = __builtin_amdgcn_readlane((int)(vi & 0xffffffffLL), src);
+  const int hi = __builtin_amdgcn_readlane((int)(vi >> 32), src);
+  return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+
+}  // namespace frnnt

@@ -1,0 +1,91 @@
+/*
+ * fast_rnnt_amd -- C ABI of the MI355X (gfx950) library for the fast_rnnt loss
+ * hot path.  Shared library: fast_rnnt_amd/csrc/libfast_rnnt_amd.so.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer to a dense, row-major (last axis
+ *     fastest) buffer unless stated otherwise; the caller owns and allocates
+ *     every buffer, outputs included;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); work
+ *     is only enqueued, nothing here synchronises or allocates;
+ *   - the device the pointers live on must be current when calling;
+ *   - return value 0 = enqueued; a negative value is an FRNNT_E* code and
+ *     frnnt_last_error() then describes the failure (thread-local text);
+ *   - B batch, S symbols, T frames, C vocabulary size; `modified` = 1 when px has
+ *     T columns (the "modified"/"constrained" lattices), 0 when it has T+1;
+ *   - `boundary` is int64 [B][4] = (s_begin, t_begin, s_end, t_end) or NULL for
+ *     (0, 0, S, T) on every row.  A row that violates
+ *     0 <= s_begin <= s_end <= S or 0 <= t_begin <= t_end <= T is skipped and its
+ *     `ans` is set to NaN (its gradients to 0); nothing is read out of bounds.
+ *   - suffix _f32 / _f64 = element type of the floating-point buffers.
+ */
+#ifndef FAST_RNNT_AMD_H_
+#define FAST_RNNT_AMD_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FRNNT_OK 0
+#define FRNNT_EINVAL (-1)  /* bad argument (null pointer, negative size, ...) */
+#define FRNNT_ELAUNCH (-2) /* the HIP runtime refused the launch             */
+#define FRNNT_ELIMIT (-3)  /* a size exceeds what the kernels support        */
+
+/* Library version, major*100 + minor. */
+int frnnt_version(void);
+
+/* Text of the last error raised on the calling thread ("" if none). */
+const char *frnnt_last_error(void);
+
+/*
+ * Lattice recursion, forward.  Replaces
+ *   _fast_rnnt.mutual_information_forward
+ *     (fast_rnnt/python/csrc/mutual_information.cu:27-45), i.e.
+ *   MutualInformationCpu / MutualInformationCuda
+ *     (fast_rnnt/csrc/mutual_information.h:116-126,
+ *      fast_rnnt/csrc/mutual_information_cpu.cu:50-124).
+ *   px  [B][S][T+1] (modified: [B][S][T])      in
+ *   py  [B][S+1][T]                            in
+ *   p   [B][S+1][T+1]                          out: only the boundary window of
+ *                                              each row is written
+ *   ans [B]                                    out: p[b][s_end][t_end]
+ */
+int frnnt_mi_forward_f32(const float *px, const float *py, const int64_t *boundary,
+                         float *p, float *ans, int B, int S, int T, int modified,
+                         void *stream);
+int frnnt_mi_forward_f64(const double *px, const double *py, const int64_t *boundary,
+                         double *p, double *ans, int B, int S, int T, int modified,
+                         void *stream);
+
+/*
+ * Lattice recursion, backward.  Replaces
+ *   _fast_rnnt.mutual_information_backward
+ *     (fast_rnnt/python/csrc/mutual_information.cu:47-67), i.e.
+ *   MutualInformationBackwardCpu / ...Cuda
+ *     (fast_rnnt/csrc/mutual_information.h:136-143,
+ *      fast_rnnt/csrc/mutual_information_cpu.cu:128-256).
+ *   p        [B][S+1][T+1]   in: the table frnnt_mi_forward_* produced
+ *   ans_grad [B]             in; if overwrite_ans_grad != 0 it is overwritten
+ *                            with the gradient that reaches (s_begin, t_begin),
+ *                            which equals the input when the sweep is consistent
+ *                            (mutual_information_cuda.cu:667-669)
+ *   px_grad  same shape as px, py_grad same shape as py: out.  Every element is
+ *            written: the window gets the gradients, the rest exact zeros.
+ * The split of a cell's gradient follows the CPU reference: d1 = exp(term1 - p),
+ * d2 = 1 - d1, both 0 when d1 is not finite.
+ */
+int frnnt_mi_backward_f32(const float *px, const float *py, const int64_t *boundary,
+                          const float *p, float *ans_grad, float *px_grad,
+                          float *py_grad, int B, int S, int T, int modified,
+                          int overwrite_ans_grad, void *stream);
+int frnnt_mi_backward_f64(const double *px, const double *py, const int64_t *boundary,
+                          const double *p, double *ans_grad, double *px_grad,
+                          double *py_grad, int B, int S, int T, int modified,
+                          int overwrite_ans_grad, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FAST_RNNT_AMD_H_ */
