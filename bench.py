@@ -1,0 +1,203 @@
+#!/usr/bin/env python3
+"""Benchmark of the fast_rnnt loss hot path on one MI355X.
+
+One step = one ``rnnt_loss_simple(..., reduction="sum", return_grad=True)`` call
+plus ``loss.backward()`` on the synthetic ASR-shaped batch c2
+(B=32, T=250, S=80, C=500, fp32; inputs already resident in HBM).  Prints ONE
+JSON line: whole-call throughput, the roofline figure of the dominant kernel
+(timed live with events on the launch stream) and the CPU baseline (the oracle
+restatement of the reference path, timed on this host's cores).
+
+    python bench.py [--gpus 1] [--steps 200] [--warmup 20] [--workload c2]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+FP32_MFMA_PEAK_TFLOPS = 157.3
+
+
+def _parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c4"])
+    ap.add_argument("--cpu-seconds", type=float, default=12.0,
+                    help="budget of the CPU-baseline leg (0 disables it)")
+    ap.add_argument("--kernel-reps", type=int, default=50)
+    return ap.parse_args()
+
+
+def _event_time_ms(fn, reps):
+    """Average duration of fn() over `reps` back-to-back launches, measured with
+    events recorded on the stream the kernels are enqueued on."""
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(reps):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / reps
+
+
+def _recursion_bytes(boundary, S, T, B, backward):
+    """Algorithmic HBM bytes of one recursion launch (fp32): every input cell of
+    the boundary window read once, every output cell written once."""
+    Sb = boundary[:, 2] - boundary[:, 0]
+    Tb = boundary[:, 3] - boundary[:, 1]
+    win = (Sb * (Tb + 1) + (Sb + 1) * Tb + (Sb + 1) * (Tb + 1)).sum().item()
+    if not backward:
+        return 4 * win + 4 * B + 32 * B
+    # backward reads the px/py/p windows, writes the full gradient arrays
+    return 4 * win + 4 * (B * S * (T + 1) + B * (S + 1) * T) + 4 * B + 32 * B
+
+
+def main():
+    args = _parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the loss path has no multi-GPU part "
+              "(each rank would run this same kernel on its own shard); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+
+    import fast_rnnt_amd
+    from fast_rnnt_amd import _fast_rnnt, _lib, workloads
+    from fast_rnnt_amd.rnnt_loss import _SimpleLogprobs
+
+    _lib.load()
+    dev = torch.device("cuda", 0)
+    w = workloads.make(args.workload)
+    am = w.am.to(dev).requires_grad_(True)
+    lm = w.lm.to(dev).requires_grad_(True)
+    sym = w.symbols.to(dev)
+    bnd = w.boundary.to(dev)
+
+    def step():
+        am.grad = None
+        lm.grad = None
+        loss, (gx, gy) = fast_rnnt_amd.rnnt_loss_simple(
+            lm, am, sym, w.termination_symbol, boundary=bnd, reduction="sum", return_grad=True)
+        loss.backward()
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = 1e3 * elapsed / args.steps
+    calls_per_sec = args.steps / elapsed
+
+    # ---- per-stage kernel timings (events on the launch stream) -------------------
+    with torch.no_grad():
+        px, py = fast_rnnt_amd.get_rnnt_logprobs(lm, am, sym, 0, boundary=bnd)
+        B, S, T = w.B, w.S, w.T
+        p = torch.empty(B, S + 1, T + 1, device=dev)
+        ones = torch.ones(B, device=dev)
+        t_fwd = _event_time_ms(lambda: _fast_rnnt.mutual_information_forward(px, py, bnd, p),
+                               args.kernel_reps)
+        t_bwd = _event_time_ms(
+            lambda: _fast_rnnt.mutual_information_backward(px, py, bnd, p, ones),
+            args.kernel_reps)
+        t_logp = _event_time_ms(
+            lambda: fast_rnnt_amd.get_rnnt_logprobs(lm, am, sym, 0, boundary=bnd),
+            args.kernel_reps)
+    stages = {"mi_forward_ms": t_fwd, "mi_backward_ms": t_bwd, "logprobs_fwd_ms": t_logp}
+
+    fwd_bytes = _recursion_bytes(w.boundary, S, T, B, backward=False)
+    achieved = fwd_bytes / (t_fwd * 1e-3) / 1e9
+    roofline = {
+        "kernel": "mi_forward_kernel<float,false,256>",
+        "bound": "hbm",
+        "achieved": round(achieved, 2),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 5),
+        "traffic": None,
+        "algorithmic_bytes": fwd_bytes,
+        "avg_launch_us": round(1e3 * t_fwd, 2),
+    }
+
+    # ---- CPU baseline: the oracle restatement of the reference path ------------------
+    cpu = None
+    if args.cpu_seconds > 0:
+        from oracle import losses as O
+
+        cores = os.cpu_count() or 1
+        torch.set_num_threads(min(cores, 16))
+        a = w.am.clone().requires_grad_(True)
+        l = w.lm.clone().requires_grad_(True)
+
+        def cpu_step():
+            a.grad = None
+            l.grad = None
+            loss, _ = O.loss_simple(l, a, w.symbols, 0, boundary=w.boundary, reduction="sum",
+                                    return_grad=True)
+            loss.backward()
+            return loss
+
+        cpu_step()
+        cpu_step()
+        n, t_start = 0, time.perf_counter()
+        while True:
+            cpu_loss = cpu_step()
+            n += 1
+            spent = time.perf_counter() - t_start
+            if spent > args.cpu_seconds or n >= 200:
+                break
+        gpu_loss = step().item()
+        cpu = {
+            "value": round(n / spent, 3),
+            "unit": "fwd+bwd loss calls/sec",
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"{n} full {w.name} calls in {spent:.1f} s (torch-CPU tensor algebra on "
+                      f"{torch.get_num_threads()} threads + single-thread C recursion)",
+            "loss_rel_diff_vs_gpu": abs(gpu_loss - cpu_loss.item()) / abs(cpu_loss.item()),
+        }
+
+    out = {
+        "metric": "fwd+bwd loss calls/sec (B=32,T=250,S=80,C=500) + achieved HBM GB/s",
+        "value": round(calls_per_sec, 2),
+        "unit": "calls/sec",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"{w.name}: rnnt_loss_simple fwd+bwd, B={w.B} T={w.T} S={w.S} "
+                               f"C={w.C}, ragged boundary, reduction=sum, return_grad=True",
+                   "call_bytes": workloads.simple_call_bytes(w)},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "stages": {k: round(v, 4) for k, v in stages.items()},
+        "whole_call_hbm_GBs": round(workloads.simple_call_bytes(w) / elapsed * args.steps / 1e9, 2),
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -6,3 +6,6 @@ from ._fast_rnnt import with_cuda
 
 from .mutual_information import mutual_information_recursion
 from .mutual_information import joint_mutual_information_recursion
+
+from .rnnt_loss import get_rnnt_logprobs
+from .rnnt_loss import rnnt_loss_simple

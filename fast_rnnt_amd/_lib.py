@@ -29,6 +29,10 @@ _SIGNATURES = {
     "frnnt_mi_forward_f64": ([_P, _P, _P, _P, _P, _I, _I, _I, _I, _P], _I),
     "frnnt_mi_backward_f32": ([_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P], _I),
     "frnnt_mi_backward_f64": ([_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P], _I),
+    "frnnt_simple_logprobs_fwd_f32": ([_P] * 9 + [_I] * 6 + [_P], _I),
+    "frnnt_simple_logprobs_fwd_f64": ([_P] * 9 + [_I] * 6 + [_P], _I),
+    "frnnt_simple_logprobs_bwd_f32": ([_P] * 15 + [_I] * 6 + [_P], _I),
+    "frnnt_simple_logprobs_bwd_f64": ([_P] * 15 + [_I] * 6 + [_P], _I),
 }
 
 

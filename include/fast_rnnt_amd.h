@@ -85,6 +85,52 @@ int frnnt_mi_backward_f64(const double *px, const double *py, const int64_t *bou
                           double *py_grad, int B, int S, int T, int modified,
                           int overwrite_ans_grad, void *stream);
 
+/*
+ * px / py of the simple (additive-joiner) RNN-T loss.  Replaces the tensor
+ * algebra of get_rnnt_logprobs (fast_rnnt/python/fast_rnnt/rnnt_loss.py:66-227):
+ * row maxima, the exp(lm) exp(am)^T contraction (fp32 / fp64 MFMA with the
+ * exponentials fused into the operand loads), log, and the px / py assembly
+ * including the -inf column(s) of the regular lattice and the constrained
+ * "px += py[:, 1:]" step.
+ *   lm [B][S+1][C], am [B][T][C], symbols int64 [B][S]              in
+ *   boundary int64 [B][4] or NULL: only boundary[b][3] is used (regular lattice)
+ *   px [B][S][T+1] (rnnt_type 0) or [B][S][T] (1, 2); py [B][S+1][T]   out
+ *   lm_max [B][S+1], am_max [B][T]                                  out (row maxima)
+ *   norm_raw [B][S+1][T] or NULL  out: log(sum_c exp(lm-lm_max) exp(am-am_max) + tiny),
+ *                                 needed by the backward entry point
+ *   rnnt_type: 0 regular, 1 modified, 2 constrained
+ */
+int frnnt_simple_logprobs_fwd_f32(const float *lm, const float *am, const int64_t *symbols,
+                                  const int64_t *boundary, float *px, float *py, float *lm_max,
+                                  float *am_max, float *norm_raw, int B, int S, int T, int C,
+                                  int termination_symbol, int rnnt_type, void *stream);
+int frnnt_simple_logprobs_fwd_f64(const double *lm, const double *am, const int64_t *symbols,
+                                  const int64_t *boundary, double *px, double *py, double *lm_max,
+                                  double *am_max, double *norm_raw, int B, int S, int T, int C,
+                                  int termination_symbol, int rnnt_type, void *stream);
+
+/*
+ * Backward of the above: what autograd derives for rnnt_loss.py:174-225, as one
+ * elementwise pass plus two MFMA GEMMs.
+ *   px_grad, py_grad: dL/dpx, dL/dpy (shapes of px, py)                    in
+ *   dmat [B][S+1][T], row_x [B][S+1], row_y [B][S+1], col_y [B][T]         scratch
+ *   lm_grad [B][S+1][C], am_grad [B][T][C]: out; either may be NULL to skip it
+ */
+int frnnt_simple_logprobs_bwd_f32(const float *lm, const float *am, const int64_t *symbols,
+                                  const int64_t *boundary, const float *lm_max,
+                                  const float *am_max, const float *norm_raw, const float *px_grad,
+                                  const float *py_grad, float *dmat, float *row_x, float *row_y,
+                                  float *col_y, float *lm_grad, float *am_grad, int B, int S,
+                                  int T, int C, int termination_symbol, int rnnt_type,
+                                  void *stream);
+int frnnt_simple_logprobs_bwd_f64(const double *lm, const double *am, const int64_t *symbols,
+                                  const int64_t *boundary, const double *lm_max,
+                                  const double *am_max, const double *norm_raw,
+                                  const double *px_grad, const double *py_grad, double *dmat,
+                                  double *row_x, double *row_y, double *col_y, double *lm_grad,
+                                  double *am_grad, int B, int S, int T, int C,
+                                  int termination_symbol, int rnnt_type, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

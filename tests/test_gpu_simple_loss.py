@@ -1,0 +1,144 @@
+"""rnnt_loss_simple / get_rnnt_logprobs on the GPU against the CPU oracle.
+
+Tolerances (float32): loss 1e-5 relative, px_grad / py_grad 1e-4 absolute,
+am.grad / lm.grad 1e-4 absolute; float64: 1e-9.
+"""
+import sys
+
+import pytest
+import torch
+
+import fast_rnnt_amd
+from fast_rnnt_amd import rnnt_loss as R
+from fast_rnnt_amd import workloads
+from oracle import losses as O
+
+pytestmark = pytest.mark.gpu
+KINDS = ["regular", "modified", "constrained"]
+
+
+def _say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def _case(seed, B, S, T, C, dtype, kind, with_boundary=True):
+    g = torch.Generator().manual_seed(seed)
+    am = torch.randn(B, T, C, generator=g, dtype=dtype)
+    lm = torch.randn(B, S + 1, C, generator=g, dtype=dtype)
+    sym = torch.randint(0, C, (B, S), generator=g)
+    bnd = None
+    if with_boundary:
+        Sb = torch.randint(1, S + 1, (B,), generator=g)
+        lo = 1 if kind == "regular" else S
+        Tb = torch.randint(lo, T + 1, (B,), generator=g)
+        z = torch.zeros(B, dtype=torch.int64)
+        bnd = torch.stack([z, z, Sb, Tb], 1)
+    return am, lm, sym, bnd
+
+
+def _close(a, b, atol, rtol=0.0):
+    a, b = a.detach().cpu(), b.detach().cpu()
+    same_inf = torch.isinf(a) & (a == b)
+    return bool((same_inf | ((a - b).abs() <= atol + rtol * b.abs())).all())
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_logprobs_match_oracle(gpu_device, dtype, kind):
+    shapes = [(1, 3, 4, 3), (3, 5, 9, 8), (2, 70, 65, 33), (2, 17, 130, 100), (3, 64, 64, 64)]
+    for n, (B, S, T, C) in enumerate(shapes):
+        if kind != "regular" and T < S:
+            continue
+        for with_boundary in (False, True):
+            _say(f"logprobs {kind} {dtype} shape{n} B={B} S={S} T={T} C={C} bnd={with_boundary}")
+            am, lm, sym, bnd = _case(40 + n, B, S, T, C, dtype, kind, with_boundary)
+            term = C - 1
+            wx, wy = O.lattice_logprobs_simple(lm, am, sym, term, rnnt_type=kind, boundary=bnd)
+            dev = gpu_device
+            gx, gy = fast_rnnt_amd.get_rnnt_logprobs(
+                lm.to(dev), am.to(dev), sym.to(dev), term, rnnt_type=kind,
+                boundary=bnd.to(dev) if bnd is not None else None)
+            tol = 2e-5 if dtype == torch.float32 else 1e-11
+            assert gx.shape == wx.shape and gy.shape == wy.shape
+            assert _close(gx, wx, tol, tol), (gx.cpu() - wx).abs().max()
+            assert _close(gy, wy, tol, tol)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_loss_and_all_gradients(gpu_device, dtype, kind):
+    dev = gpu_device
+    for n, (B, S, T, C) in enumerate([(3, 5, 9, 8), (4, 20, 75, 50), (2, 66, 140, 70)]):
+        for reduction in ("sum", "mean", "none"):
+            _say(f"loss {kind} {dtype} shape{n} reduction={reduction}")
+            am, lm, sym, bnd = _case(60 + n, B, S, T, C, dtype, kind)
+            a = am.clone().requires_grad_(True)
+            l = lm.clone().requires_grad_(True)
+            want, (wx, wy) = O.loss_simple(l, a, sym, 0, boundary=bnd, rnnt_type=kind,
+                                           reduction=reduction, return_grad=True)
+            wx0, wy0 = wx.clone(), wy.clone()
+            want.sum().backward()
+
+            da = am.to(dev).requires_grad_(True)
+            dl = lm.to(dev).requires_grad_(True)
+            got, (gx, gy) = fast_rnnt_amd.rnnt_loss_simple(
+                dl, da, sym.to(dev), 0, boundary=bnd.to(dev), rnnt_type=kind,
+                reduction=reduction, return_grad=True)
+            gx0, gy0 = gx.clone(), gy.clone()
+            got.sum().backward()
+            f32 = dtype == torch.float32
+            assert _close(got, want, 0.0, 1e-5 if f32 else 1e-12)
+            gtol = 1e-4 if f32 else 1e-9
+            assert _close(gx0, wx0, gtol) and _close(gy0, wy0, gtol)
+            assert _close(da.grad, a.grad, gtol, 1e-4 if f32 else 1e-9), \
+                (da.grad.cpu() - a.grad).abs().max()
+            assert _close(dl.grad, l.grad, gtol, 1e-4 if f32 else 1e-9), \
+                (dl.grad.cpu() - l.grad).abs().max()
+            # the tensors handed out by return_grad were scaled in place by backward
+            assert _close(gx, wx, gtol) and _close(gy, wy, gtol)
+
+
+def test_delay_penalty_and_only_one_input_needs_grad(gpu_device):
+    dev = gpu_device
+    am, lm, sym, bnd = _case(77, 3, 9, 30, 21, torch.float32, "regular")
+    l = lm.clone().requires_grad_(True)
+    want = O.loss_simple(l, am, sym, 0, boundary=bnd, delay_penalty=0.02, reduction="sum")
+    want.backward()
+    dl = lm.to(dev).requires_grad_(True)
+    got = fast_rnnt_amd.rnnt_loss_simple(dl, am.to(dev), sym.to(dev), 0, boundary=bnd.to(dev),
+                                         delay_penalty=0.02, reduction="sum")
+    got.backward()
+    assert _close(got, want, 0.0, 1e-5)
+    assert _close(dl.grad, l.grad, 1e-4, 1e-4)
+    with pytest.raises(ValueError):
+        fast_rnnt_amd.rnnt_loss_simple(dl, am.to(dev), sym.to(dev), 0, reduction="bogus")
+
+
+@pytest.mark.parametrize("name", ["c1", "c2"])
+def test_baseline_configs(gpu_device, name):
+    dev = gpu_device
+    w = workloads.make(name)
+    _say(f"workload {name}: B={w.B} T={w.T} S={w.S} C={w.C}")
+    a = w.am.clone().requires_grad_(True)
+    l = w.lm.clone().requires_grad_(True)
+    want, (wx, wy) = O.loss_simple(l, a, w.symbols, 0, boundary=w.boundary, reduction="sum",
+                                   return_grad=True)
+    wx0, wy0 = wx.clone(), wy.clone()
+    want.backward()
+    da = w.am.to(dev).requires_grad_(True)
+    dl = w.lm.to(dev).requires_grad_(True)
+    got, (gx, gy) = fast_rnnt_amd.rnnt_loss_simple(
+        dl, da, w.symbols.to(dev), 0, boundary=w.boundary.to(dev), reduction="sum",
+        return_grad=True)
+    gx0, gy0 = gx.clone(), gy.clone()
+    got.backward()
+    rel = abs(got.item() - want.item()) / abs(want.item())
+    _say(f"  loss gpu={got.item():.6f} cpu={want.item():.6f} rel={rel:.2e} "
+         f"px_grad maxdiff={(gx0.cpu() - wx0).abs().max().item():.2e} "
+         f"py_grad maxdiff={(gy0.cpu() - wy0).abs().max().item():.2e} "
+         f"am.grad maxdiff={(da.grad.cpu() - a.grad).abs().max().item():.2e} "
+         f"lm.grad maxdiff={(dl.grad.cpu() - l.grad).abs().max().item():.2e}")
+    assert rel <= 1e-5
+    assert _close(gx0, wx0, 1e-4) and _close(gy0, wy0, 1e-4)
+    assert _close(da.grad, a.grad, 1e-4, 1e-4) and _close(dl.grad, l.grad, 1e-4, 1e-4)
