@@ -8,6 +8,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <limits>
+#include <type_traits>
 
 #include "../../include/fast_rnnt_amd.h"
 
@@ -65,6 +66,19 @@ __device__ __forceinline__ double from_lane_below(double v, double fill) {
                                              0x138, 0xf, 0xf, false);
   const int hi = __builtin_amdgcn_update_dpp((int)(fi >> 32), (int)(vi >> 32), 0x138, 0xf, 0xf,
                                              false);
+  return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+
+// Same shift with lane 0 receiving 0: in this form the compiler can fold the
+// shift into the consuming VALU instruction.
+__device__ __forceinline__ float from_lane_below_zero(float v) {
+  return __int_as_float(
+      __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x138, 0xf, 0xf, true));
+}
+__device__ __forceinline__ double from_lane_below_zero(double v) {
+  const long long vi = __double_as_longlong(v);
+  const int lo = __builtin_amdgcn_update_dpp(0, (int)(vi & 0xffffffffLL), 0x138, 0xf, 0xf, true);
+  const int hi = __builtin_amdgcn_update_dpp(0, (int)(vi >> 32), 0x138, 0xf, 0xf, true);
   return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
 }
 

@@ -1,28 +1,42 @@
 // Lattice ("mutual information") recursion, forward and backward, for gfx950.
 //
-// Mapping: one workgroup per utterance, one lane per lattice row.  A wave owns
-// 64 consecutive rows and sweeps the lattice along anti-diagonals: at local
-// step e lane L works on column e - L, so the "up" neighbour is what lane L-1
-// produced one step earlier (regular lattice) or two steps earlier (modified
-// lattice) and arrives through a DPP wave shift, and the "left" neighbour is the
-// lane's own previous result.  Rows beyond 64 go to further waves of the same
-// workgroup; wave w+1 consumes the last row of wave w through an LDS seam row
-// guarded by a monotone progress counter, so waves run skewed by a chunk or two
-// instead of meeting at a barrier every step.  Lattices taller than the
-// workgroup are swept band after band with the same seam mechanism.
+// Mapping.  One workgroup per utterance, one lane per lattice row.  A *sweep
+// wave* owns 64 consecutive rows and walks the lattice along anti-diagonals: at
+// local step e lane L works on column e - L, so the neighbour in the previous
+// row is what lane L-1 produced one step earlier (regular lattice) or two steps
+// earlier (modified lattice) and arrives through a DPP wave shift, and the
+// neighbour in the same row is the lane's own previous result.  Nothing but this
+// dependent chain runs on a sweep wave: all HBM traffic is done by *staging
+// waves* of the same workgroup, which fetch px/py (forward) or p/px (backward)
+// with coalesced row loads, turn them into diagonal ("sheared") 64-row x 32-step
+// tiles in LDS, and -- for the backward sweep -- also evaluate the exp() of the
+// gradient split and write the finished gradient tiles back to HBM.  Tiles are
+// double buffered; sweep and staging waves meet only through monotone LDS
+// counters (acquire/release, bounded spinning), never at a barrier.
+//
+// Rows beyond 64 go to further sweep waves; wave w+1 consumes the last row of
+// wave w through an LDS seam row guarded by a progress counter and simply runs a
+// few steps behind.  Lattices taller than the workgroup's sweep waves are
+// processed band after band with the same seam mechanism.
 //
 // The arithmetic follows the CPU reference operation for operation
 // (fast_rnnt/csrc/mutual_information_cpu.cu:89-121 forward, :179-252 backward,
-// log-add from fast_rnnt/csrc/mutual_information.h:36-65); only exp/log1p come
+// log-add from fast_rnnt/csrc/mutual_information.h:36-65); only exp/log come
 // from the GPU's own units.
 #include "common.hip.h"
 
 namespace frnnt {
 namespace {
 
-constexpr int kMaxWaves = 16;  // 1024 threads
-constexpr int kChunk = 8;      // steps per prefetch / seam hand-over chunk
-constexpr int kSpinLimit = 1 << 24;
+constexpr int kMaxSweep = 4;           // sweep waves per workgroup
+constexpr int kChunk = 8;              // steps per seam hand-over
+constexpr int kTileSteps = 32;         // steps per staged tile
+constexpr int kTilePitch = kTileSteps + 1;
+constexpr int kTileElems = kWave * kTilePitch;
+constexpr int kFwdStagers = 2;         // staging waves per sweep wave
+constexpr int kStageBatch = 8;         // rows a staging lane fetches before it writes LDS
+constexpr int kBwdStagers = 3;
+constexpr int kSpinLimit = 1 << 22;
 
 struct Window {
   int s0, t0, ns, nt;  // origin and extent (ns = s_end - s_begin, ...)
@@ -43,8 +57,8 @@ __device__ __forceinline__ Window load_window(const int64_t *boundary, int b, in
   return w;
 }
 
-// Blocks until the producer's counter reaches `target`; gives up (returns false)
-// after a bounded number of polls so that no wave can spin forever.
+// Blocks until the counter reaches `target`; gives up (returns false) after a
+// bounded number of polls so that no wave can spin forever.
 __device__ __forceinline__ bool wait_for(const int *counter, int target) {
   int spins = 0;
   while (__hip_atomic_load(counter, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < target) {
@@ -53,22 +67,64 @@ __device__ __forceinline__ bool wait_for(const int *counter, int target) {
   }
   return true;
 }
+__device__ __forceinline__ void publish(int *counter, int value) {
+  __hip_atomic_store(counter, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
 
-template <typename R, bool kModified, int kBlock>
-__global__ void __launch_bounds__(kBlock)
+// log(exp(a) + exp(c)) on the serial chain: same operation order as log_add(),
+// written so that the only fix-up is the NaN that (-inf) - (-inf) produces.
+__device__ __forceinline__ float chain_log_add(float a, float c) {
+  const float d = a - c;
+  const float hi = (a > c) ? a : c;
+  // -|d| * log2(e) is <= 0 or NaN ((-inf) - (-inf)); fminf maps the NaN to 0, and
+  // the result is then hi + log(2) = hi, because hi is infinite in that case --
+  // exactly the "return the larger operand" rule of the reference, without a branch.
+  const float t = fminf(-fabsf(d) * 1.44269504088896341f, 0.0f);
+  const float e = __builtin_amdgcn_exp2f(t);
+  const float l = __builtin_amdgcn_logf(1.0f + e) * 0.693147180559945309f;
+  return hi + l;
+}
+__device__ __forceinline__ double chain_log_add(double a, double c) { return log_add(a, c); }
+
+struct Counters {
+  int ready[kMaxSweep];                   // seam columns published by sweep wave w
+  int consumed[kMaxSweep];                // tiles sweep wave w has finished
+  int loaded[kMaxSweep * kBwdStagers];    // tiles staged for sweep wave w by stager l (kBwdStagers >= kFwdStagers)
+};
+
+// Geometry of what sweep wave `w` does in band `band`; identical on the sweep
+// wave and on its staging waves.
+struct Band {
+  int row0, nrows, nsteps, ntiles;
+};
+__device__ __forceinline__ Band band_of(int band, int w, int nsweep, int NS, int NT) {
+  Band g;
+  g.row0 = (band * nsweep + w) * kWave;
+  g.nrows = min(kWave, NS + 1 - g.row0);
+  g.nsteps = NT + g.nrows;
+  g.ntiles = (g.nsteps + kTileSteps - 1) / kTileSteps;
+  return g;
+}
+
+// =============================== forward =====================================
+// Staged per step and row: x = px feeding the cell from the row below,
+// y = py feeding it from the left; -inf where that edge does not exist, and
+// y = 0 at the origin cell so that the chain produces p = 0 there.
+template <typename R, bool kModified>
+__global__ void __launch_bounds__((1 + kFwdStagers) * kMaxSweep *kWave)
     mi_forward_kernel(const R *__restrict__ px, const R *__restrict__ py,
                       const int64_t *__restrict__ boundary, R *__restrict__ p,
                       R *__restrict__ ans, int S, int T) {
   extern __shared__ __align__(16) unsigned char dyn_lds[];
-  __shared__ int ready[kMaxWaves];
-  R *seam = reinterpret_cast<R *>(dyn_lds);
+  __shared__ Counters cnt;
 
   const int b = blockIdx.x;
-  const int nw = blockDim.x / kWave;
-  const int w = threadIdx.x / kWave;
+  const int nsweep = blockDim.x / (kWave * (1 + kFwdStagers));
+  const int wave = threadIdx.x / kWave;
   const int lane = threadIdx.x % kWave;
   const int T1 = kModified ? T : T + 1;
   const int TP = T + 1;
+  const int shift = kModified ? 1 : 0;
   const R ninf = Num<R>::neg_inf();
 
   const Window win = load_window(boundary, b, S, T);
@@ -76,112 +132,208 @@ __global__ void __launch_bounds__(kBlock)
     if (threadIdx.x == 0) ans[b] = std::numeric_limits<R>::quiet_NaN();
     return;
   }
-  if (threadIdx.x < kMaxWaves) ready[threadIdx.x] = 0;
+  if (threadIdx.x < (int)(sizeof(Counters) / sizeof(int)))
+    reinterpret_cast<int *>(&cnt)[threadIdx.x] = 0;
   __syncthreads();
 
   const int NS = win.ns, NT = win.nt, cols = NT + 1;
   const R *pxb = px + (size_t)b * S * T1;
   const R *pyb = py + (size_t)b * (S + 1) * T;
   R *pb = p + (size_t)b * (S + 1) * TP;
-  const int band_rows = kWave * nw;
-  const int prev = (w + nw - 1) % nw;
+  R *seam = reinterpret_cast<R *>(dyn_lds);
+  R *tiles = seam + (size_t)nsweep * TP;  // [nsweep][2 arrays][2 buffers][kTileElems]
+  const int band_rows = kWave * nsweep;
+
+  if (wave >= nsweep) {
+    // ------------------------------ staging wave -------------------------------
+    const int w = (wave - nsweep) / kFwdStagers, l = (wave - nsweep) % kFwdStagers;
+    R *xt = tiles + (size_t)w * 4 * kTileElems;
+    R *yt = xt + 2 * kTileElems;
+    const int half = lane >> 5, q = lane & 31;
+    int tile_base = 0;
+    for (int band = 0; band * band_rows <= NS; ++band) {
+      const Band g = band_of(band, w, nsweep, NS, NT);
+      if (g.row0 > NS) break;
+      for (int m = 0; m < g.ntiles; ++m) {
+        const int gt = tile_base + m;
+        if (gt >= 2 && !wait_for(&cnt.consumed[w], gt - 1)) return;
+        R *xdst = xt + (gt & 1) * kTileElems, *ydst = yt + (gt & 1) * kTileElems;
+        // all row fetches of a batch are issued before the first LDS write, so one
+        // memory latency covers the whole batch
+        for (int rb = 2 * l + half; rb < g.nrows; rb += 2 * kFwdStagers * kStageBatch) {
+          R xv[kStageBatch], yv[kStageBatch];
+#pragma unroll
+          for (int u = 0; u < kStageBatch; ++u) {
+            const int r = rb + 2 * kFwdStagers * u;
+            const int i = g.row0 + r, s = win.s0 + i;
+            const int j = m * kTileSteps + q - r;
+            const int jj = j - shift;
+            R x = ninf, y = ninf;
+            if (r < g.nrows) {
+              if (i >= 1 && jj >= 0 && j <= NT) x = pxb[(long)(s - 1) * T1 + win.t0 + jj];
+              if (j >= 1 && j <= NT) y = pyb[(long)s * T + win.t0 + j - 1];
+              if (i == 0 && j == 0) y = 0;
+            }
+            xv[u] = x;
+            yv[u] = y;
+          }
+#pragma unroll
+          for (int u = 0; u < kStageBatch; ++u) {
+            const int r = rb + 2 * kFwdStagers * u;
+            if (r < g.nrows) {
+              xdst[r * kTilePitch + q] = xv[u];
+              ydst[r * kTilePitch + q] = yv[u];
+            }
+          }
+        }
+        if (lane == 0) publish(&cnt.loaded[w * kFwdStagers + l], gt + 1);
+      }
+      tile_base += g.ntiles;
+    }
+    return;
+  }
+
+  // -------------------------------- sweep wave ---------------------------------
+  const int w = wave;
+  const int prev = (w + nsweep - 1) % nsweep;
   R *my_seam = seam + (size_t)w * TP;
   const R *up_seam = seam + (size_t)prev * TP;
-
+  const R *xt = tiles + (size_t)w * 4 * kTileElems;
+  const R *yt = xt + 2 * kTileElems;
+  int tile_base = 0;
   for (int band = 0; band * band_rows <= NS; ++band) {
-    const int row0 = band * band_rows + kWave * w;
-    if (row0 > NS) break;
-    const int i = row0 + lane;  // lattice row relative to the window
-    const int s = win.s0 + i;
+    const Band g = band_of(band, w, nsweep, NS, NT);
+    if (g.row0 > NS) break;
+    const int i = g.row0 + lane;
     const bool row_ok = i <= NS;
-    const int nrows = min(kWave, NS + 1 - row0);
-    const bool has_up = row0 > 0;
+    const bool has_up = g.row0 > 0;
     const int up_base = (w > 0 ? band : band - 1) * cols;
     const int my_base = band * cols;
-    const long x_off = (long)(s - 1) * T1 + win.t0;  // px row feeding this lattice row
-    const long y_off = (long)s * T + win.t0;
-    const long p_off = (long)s * TP + win.t0;
-    const int x_last = kModified ? NT - 1 : NT;
-    const int nsteps = NT + nrows;
+    R *p_row = pb + (long)(win.s0 + i) * TP + win.t0;
 
-    R xn[kChunk], yn[kChunk];
-    auto fetch = [&](int e0) {
+    R own = (i == 0) ? (R)0 : ninf, own2 = ninf;
+    R fin = ninf;  // value of this lane's cell in column NT
+    const bool has_down = g.nrows == kWave;
+    for (int m = 0; m < g.ntiles; ++m) {
+      const int gt = tile_base + m;
 #pragma unroll
-      for (int k = 0; k < kChunk; ++k) {
-        const int j = e0 + k - lane;
-        const int jj = kModified ? j - 1 : j;
-        xn[k] = (row_ok && i >= 1 && jj >= 0 && jj <= x_last) ? pxb[x_off + jj] : ninf;
-        yn[k] = (row_ok && j >= 1 && j <= NT) ? pyb[y_off + j - 1] : ninf;
-      }
-    };
-    fetch(0);
-
-    R own = ninf, own2 = ninf;
-    for (int e0 = 0; e0 < nsteps; e0 += kChunk) {
-      R xc[kChunk], yc[kChunk];
+      for (int l = 0; l < kFwdStagers; ++l)
+        if (!wait_for(&cnt.loaded[w * kFwdStagers + l], gt + 1)) return;
+      // this lane's 32 steps of inputs go to registers in one burst, after which
+      // the staging waves may refill the buffer
+      R xq[kTileSteps], yq[kTileSteps];
+      {
+        const R *xs = xt + (gt & 1) * kTileElems + lane * kTilePitch;
+        const R *ys = yt + (gt & 1) * kTileElems + lane * kTilePitch;
 #pragma unroll
-      for (int k = 0; k < kChunk; ++k) {
-        xc[k] = xn[k];
-        yc[k] = yn[k];
+        for (int kk = 0; kk < kTileSteps; ++kk) {
+          xq[kk] = xs[kk];
+          yq[kk] = ys[kk];
+        }
       }
-      if (e0 + kChunk < nsteps) fetch(e0 + kChunk);
+      if (lane == 0) publish(&cnt.consumed[w], gt + 1);
 
-      R handed = ninf;  // lane k holds the seam value lane 0 needs at step e0 + k
+      // One chunk of kChunk steps, specialised at compile time on whether the wave
+      // receives a seam (kUp), feeds one (kDown), and whether every lane's cell is
+      // inside the window for the whole chunk (!kEdge).
+      bool alive = true;
+      auto chunk = [&](auto up_c, auto down_c, auto edge_c, int c4, int e0)
+                       __attribute__((always_inline)) {
+        constexpr bool kUp = decltype(up_c)::value;
+        constexpr bool kDown = decltype(down_c)::value;
+        constexpr bool kEdge = decltype(edge_c)::value;
+        R handed = ninf;  // lane k: the seam value lane 0 needs at step e0 + k
+        if (kUp) {
+          const int need = min(e0 + kChunk - shift, cols);
+          if (need > 0 && !wait_for(&cnt.ready[prev], up_base + need)) {
+            alive = false;
+            return;
+          }
+          const int col = e0 + lane - shift;
+          if (lane < kChunk && col >= 0 && col <= NT) handed = up_seam[col];
+        }
+        R *pp = p_row + (e0 - lane);
+        R *sp = my_seam + (e0 - (kWave - 1));
+#pragma unroll
+        for (int k = 0; k < kChunk; ++k) {
+          const int kk = c4 * kChunk + k;
+          // lane 0 of a wave without a seam owns lattice row 0, whose x is -inf,
+          // so the 0 it receives from the shift never matters
+          R up = from_lane_below_zero(kModified ? own2 : own);
+          if (kUp) {
+            const R first = lane_value(handed, k);
+            up = (lane == 0) ? first : up;
+          }
+          const R v = chain_log_add(up + xq[kk], own + yq[kk]);
+          const int j63 = e0 + k - (kWave - 1);  // column of the seam lane, wave-uniform
+          if (kEdge) {
+            const int j = e0 + k - lane;
+            if (row_ok && (unsigned)j <= (unsigned)NT) pp[k] = v;
+            fin = (j == NT) ? v : fin;
+            if (kDown && j63 >= 0 && j63 <= NT && lane == kWave - 1) sp[k] = v;
+          } else {
+            pp[k] = v;
+            if (kDown && lane == kWave - 1) sp[k] = v;
+          }
+          own2 = own;
+          own = v;
+        }
+        if (kDown && lane == kWave - 1) {
+          const int done = max(0, min(e0 + kChunk - (kWave - 1), cols));
+          publish(&cnt.ready[w], my_base + done);
+        }
+      };
+      auto tile = [&](auto up_c, auto down_c) __attribute__((always_inline)) {
+#pragma unroll
+        for (int c4 = 0; c4 < kTileSteps / kChunk; ++c4) {
+          const int e0 = m * kTileSteps + c4 * kChunk;
+          if (e0 < g.nsteps && alive) {
+            const bool interior =
+                g.nrows == kWave && e0 >= kWave - 1 && e0 + kChunk <= NT;
+            if (interior)
+              chunk(up_c, down_c, std::false_type{}, c4, e0);
+            else
+              chunk(up_c, down_c, std::true_type{}, c4, e0);
+          }
+        }
+      };
       if (has_up) {
-        const int need = min(e0 + kChunk - (kModified ? 1 : 0), cols);
-        if (need > 0 && !wait_for(&ready[prev], up_base + need)) return;
-        const int col = e0 + lane - (kModified ? 1 : 0);
-        if (lane < kChunk && col >= 0 && col <= NT) handed = up_seam[col];
+        if (has_down)
+          tile(std::true_type{}, std::true_type{});
+        else
+          tile(std::true_type{}, std::false_type{});
+      } else {
+        if (has_down)
+          tile(std::false_type{}, std::true_type{});
+        else
+          tile(std::false_type{}, std::false_type{});
       }
-
-#pragma unroll
-      for (int k = 0; k < kChunk; ++k) {
-        const int j = e0 + k - lane;
-        const int jj = kModified ? j - 1 : j;
-        R up = from_lane_below(kModified ? own2 : own, ninf);
-        if (has_up) {
-          const R first = lane_value(handed, k);
-          if (lane == 0) up = first;
-        }
-        const R a = (i > 0 && jj >= 0) ? up + xc[k] : ninf;
-        const R c = (j > 0) ? own + yc[k] : ninf;
-        R v = log_add(a, c);
-        if (i == 0 && j == 0) v = 0;
-        if (row_ok && j >= 0 && j <= NT) {
-          pb[p_off + j] = v;
-          if (lane == kWave - 1) my_seam[j] = v;
-          if (i == NS && j == NT) ans[b] = v;
-        }
-        own2 = own;
-        own = v;
-      }
-
-      if (nrows == kWave && lane == kWave - 1) {
-        const int done = max(0, min(e0 + kChunk - (kWave - 1), cols));
-        __hip_atomic_store(&ready[w], my_base + done, __ATOMIC_RELEASE,
-                           __HIP_MEMORY_SCOPE_WORKGROUP);
-      }
+      if (!alive) return;
     }
+    if (row_ok && i == NS) ans[b] = fin;
+    tile_base += g.ntiles;
   }
 }
 
-// Reverse sweep.  Rows and columns are counted from the end of the window
-// (r = NS - i, c = NT - j); lane L of a wave owns reversed row r and works on
-// reversed column e - L at local step e.  Each cell adds what its upper
-// neighbour hands down (d1 share) and what its right neighbour hands left
-// (d2 share), then splits the sum for its own two predecessors.
-template <typename R, bool kModified, int kBlock>
-__global__ void __launch_bounds__(kBlock)
+// =============================== backward ====================================
+// Rows and columns are counted from the end of the window (r = NS - i,
+// c = NT - j); lane L of a sweep wave owns reversed row r and works on reversed
+// column e - L at local step e.  A cell's gradient is what the row above hands
+// down plus what its right neighbour hands left; it is then split into a d1
+// share for the cell below and a d2 share for the cell to the left.  The staging
+// waves evaluate d1 / d2 (mutual_information_cpu.cu:196-212 and the two edge
+// loops :219-235) and later write the px / py gradient tiles the sweep produced.
+template <typename R, bool kModified>
+__global__ void __launch_bounds__((1 + kBwdStagers) * kMaxSweep *kWave)
     mi_backward_kernel(const R *__restrict__ px, const int64_t *__restrict__ boundary,
                        const R *__restrict__ p, R *ans_grad, R *__restrict__ px_grad,
                        R *__restrict__ py_grad, int S, int T, int overwrite_ans_grad) {
   extern __shared__ __align__(16) unsigned char dyn_lds[];
-  __shared__ int ready[kMaxWaves];
-  R *seam = reinterpret_cast<R *>(dyn_lds);
+  __shared__ Counters cnt;
 
   const int b = blockIdx.x;
-  const int nw = blockDim.x / kWave;
-  const int w = threadIdx.x / kWave;
+  const int nsweep = blockDim.x / (kWave * (1 + kBwdStagers));
+  const int wave = threadIdx.x / kWave;
   const int lane = threadIdx.x % kWave;
   const int T1 = kModified ? T : T + 1;
   const int TP = T + 1;
@@ -191,10 +343,10 @@ __global__ void __launch_bounds__(kBlock)
   R *gxb = px_grad + (size_t)b * S * T1;
   R *gyb = py_grad + (size_t)b * (S + 1) * T;
 
-  // exact zeros everywhere the sweep below does not write
+  // exact zeros everywhere the sweep does not write
   if (boundary) {
-    const int s_lo = win.s0, s_hi = win.s0 + win.ns;  // window rows  [s_lo, s_hi]
-    const int t_lo = win.t0, t_hi = win.t0 + win.nt;  // window cols  [t_lo, t_hi]
+    const int s_lo = win.s0, s_hi = win.s0 + win.ns;
+    const int t_lo = win.t0, t_hi = win.t0 + win.nt;
     for (int idx = threadIdx.x; idx < S * T1; idx += blockDim.x) {
       const int s = idx / T1, t = idx - s * T1;
       const bool inside = win.ok && s >= s_lo && s < s_hi && t >= t_lo && t <= t_hi - shift;
@@ -207,128 +359,257 @@ __global__ void __launch_bounds__(kBlock)
     }
   }
   if (!win.ok) return;
-  if (threadIdx.x < kMaxWaves) ready[threadIdx.x] = 0;
+  if (threadIdx.x < (int)(sizeof(Counters) / sizeof(int)))
+    reinterpret_cast<int *>(&cnt)[threadIdx.x] = 0;
   __syncthreads();
 
   const int NS = win.ns, NT = win.nt, cols = NT + 1;
   const R *pxb = px + (size_t)b * S * T1;
   const R *pb = p + (size_t)b * (S + 1) * TP;
-  const R seed = ans_grad[b];
-  const int band_rows = kWave * nw;
-  const int prev = (w + nw - 1) % nw;
-  R *my_seam = seam + (size_t)w * TP;
-  const R *up_seam = seam + (size_t)prev * TP;
+  R *seam = reinterpret_cast<R *>(dyn_lds);
+  // per sweep wave: d1[2], d2[2], gx[2], gy[2] tiles
+  R *tiles = seam + (size_t)nsweep * TP;
+  const int band_rows = kWave * nsweep;
 
-  for (int band = 0; band * band_rows <= NS; ++band) {
-    const int row0 = band * band_rows + kWave * w;
-    if (row0 > NS) break;
-    const int r = row0 + lane;  // reversed row
-    const int i = NS - r;       // lattice row relative to the window (may be < 0)
-    const int s = win.s0 + i;
-    const bool row_ok = r <= NS;
-    const int nrows = min(kWave, NS + 1 - row0);
-    const bool has_up = row0 > 0;
-    const int up_base = (w > 0 ? band : band - 1) * cols;
-    const int my_base = band * cols;
-    const long here_off = (long)s * TP + win.t0;          // p[s][t0 + j]
-    const long below_off = (long)(s - 1) * TP + win.t0;   // p[s-1][t0 + j - shift]
-    const long x_off = (long)(s - 1) * T1 + win.t0;       // px[s-1][t0 + j - shift]
-    const long gy_off = (long)s * T + win.t0;             // py_grad[s][t0 + j - 1]
-    const int nsteps = NT + nrows;
+  if (wave >= nsweep) {
+    // ------------------------------ staging wave -------------------------------
+    const int w = (wave - nsweep) / kBwdStagers, l = (wave - nsweep) % kBwdStagers;
+    R *base = tiles + (size_t)w * 8 * kTileElems;
+    const int half = lane >> 5, q = lane & 31;
+    int *my_loaded = &cnt.loaded[w * kBwdStagers + l];
 
-    // d1 / d2 shares of each cell of the chunk (independent of the gradient,
-    // so they stay off the serial chain)
-    R d1n[kChunk], d2n[kChunk];
-    auto shares = [&](int e0) {
-#pragma unroll
-      for (int k = 0; k < kChunk; ++k) {
-        const int c = e0 + k - lane;
+    // writes the gradient tile `m` of band geometry g (global tile index gt)
+    auto flush = [&](const Band &g, int m, int gt) {
+      const R *gxs = base + (4 + (gt & 1)) * kTileElems, *gys = base + (6 + (gt & 1)) * kTileElems;
+      for (int r = 2 * l + half; r < g.nrows; r += 2 * kBwdStagers) {
+        const int i = NS - (g.row0 + r), s = win.s0 + i;
+        const int c = m * kTileSteps + q - r;
         const int j = NT - c;
-        R d1 = 0, d2 = 0;
-        if (row_ok && c >= 0 && c <= NT) {
-          if (i > 0 && j > 0) {
-            const R term1 = pb[below_off + j - shift] + pxb[x_off + j - shift];
-            R total = pb[here_off + j];
-            if (total - total != 0) total = 0;
-            d1 = Num<R>::exp_(term1 - total);
-            d2 = (R)1 - d1;
-            if (d1 - d1 != 0) d1 = d2 = 0;
-          } else if (i == 0 && j > 0) {
-            d2 = 1;
-          } else if (i > 0 && j == 0 && !kModified) {
-            d1 = 1;
-          }
-        }
-        d1n[k] = d1;
-        d2n[k] = d2;
+        if (c < 0 || c > NT) continue;
+        if (i > 0 && (j > 0 || !kModified))
+          gxb[(long)(s - 1) * T1 + win.t0 + j - shift] = gxs[r * kTilePitch + q];
+        if (j > 0) gyb[(long)s * T + win.t0 + j - 1] = gys[r * kTilePitch + q];
       }
     };
-    shares(0);
 
-    R to_below = 0, to_below2 = 0, to_left = 0;
-    for (int e0 = 0; e0 < nsteps; e0 += kChunk) {
-      R d1c[kChunk], d2c[kChunk];
-#pragma unroll
-      for (int k = 0; k < kChunk; ++k) {
-        d1c[k] = d1n[k];
-        d2c[k] = d2n[k];
-      }
-      if (e0 + kChunk < nsteps) shares(e0 + kChunk);
-
-      R handed = 0;
-      if (has_up) {
-        const int need = min(e0 + kChunk - shift, cols);
-        if (need > 0 && !wait_for(&ready[prev], up_base + need)) return;
-        const int col = e0 + lane - shift;
-        if (lane < kChunk && col >= 0 && col <= NT) handed = up_seam[col];
-      }
-
-#pragma unroll
-      for (int k = 0; k < kChunk; ++k) {
-        const int c = e0 + k - lane;
-        const int j = NT - c;
-        R from_above = from_lane_below(kModified ? to_below2 : to_below, (R)0);
-        if (has_up) {
-          const R first = lane_value(handed, k);
-          if (lane == 0) from_above = first;
+    int tile_base = 0;
+    for (int band = 0; band * band_rows <= NS; ++band) {
+      const Band g = band_of(band, w, nsweep, NS, NT);
+      if (g.row0 > NS) break;
+      for (int m = 0; m < g.ntiles; ++m) {
+        const int gt = tile_base + m;
+        if (gt >= 2) {
+          if (!wait_for(&cnt.consumed[w], gt - 1)) return;
+          // tile gt-2 is finished: write its gradients out before its buffers are reused.
+          // It belongs to this band (m >= 2) or to the tail of the previous one.
+          if (m >= 2) {
+            flush(g, m - 2, gt - 2);
+          } else {
+            const Band pg = band_of(band - 1, w, nsweep, NS, NT);
+            flush(pg, pg.ntiles - 2 + m, gt - 2);
+          }
         }
-        const bool live = row_ok && c >= 0 && c <= NT;
-        R g = 0;
-        if (r > 0 && c - shift >= 0) g = from_above;
-        if (c > 0) g += to_left;
-        if (r == 0 && c == 0) g = seed;
-        const R down = d1c[k] * g;
-        const R left = d2c[k] * g;
-        to_below2 = to_below;
-        to_below = live ? down : (R)0;
-        to_left = live ? left : (R)0;
-        if (live) {
-          if (i > 0 && (j > 0 || !kModified)) gxb[x_off + j - shift] = down;
-          if (j > 0) gyb[gy_off + j - 1] = left;
-          if (lane == kWave - 1) my_seam[c] = down;
-          if (i == 0 && j == 0 && overwrite_ans_grad) ans_grad[b] = g;
+        R *d1dst = base + (gt & 1) * kTileElems, *d2dst = base + (2 + (gt & 1)) * kTileElems;
+        for (int rb = 2 * l + half; rb < g.nrows; rb += 2 * kBwdStagers * kStageBatch) {
+          R here[kStageBatch], below[kStageBatch], xv[kStageBatch];
+#pragma unroll
+          for (int u = 0; u < kStageBatch; ++u) {
+            const int r = rb + 2 * kBwdStagers * u;
+            const int i = NS - (g.row0 + r), s = win.s0 + i;
+            const int c = m * kTileSteps + q - r;
+            const int j = NT - c;
+            here[u] = below[u] = xv[u] = 0;
+            if (r < g.nrows && c >= 0 && c <= NT && i > 0 && j > 0) {
+              below[u] = pb[(long)(s - 1) * TP + win.t0 + j - shift];
+              xv[u] = pxb[(long)(s - 1) * T1 + win.t0 + j - shift];
+              here[u] = pb[(long)s * TP + win.t0 + j];
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < kStageBatch; ++u) {
+            const int r = rb + 2 * kBwdStagers * u;
+            const int i = NS - (g.row0 + r);
+            const int c = m * kTileSteps + q - r;
+            const int j = NT - c;
+            if (r >= g.nrows) continue;
+            R d1 = 0, d2 = 0;
+            if (c >= 0 && c <= NT) {
+              if (i > 0 && j > 0) {
+                const R term1 = below[u] + xv[u];
+                R total = here[u];
+                if (total - total != 0) total = 0;
+                d1 = Num<R>::exp_(term1 - total);
+                d2 = (R)1 - d1;
+                if (d1 - d1 != 0) d1 = d2 = 0;
+              } else if (i == 0 && j > 0) {
+                d2 = 1;
+              } else if (i > 0 && j == 0 && !kModified) {
+                d1 = 1;
+              }
+            }
+            d1dst[r * kTilePitch + q] = d1;
+            d2dst[r * kTilePitch + q] = d2;
+          }
         }
+        // every lane's LDS writes precede the release by lane 0 of the same wave
+        if (lane == 0) publish(my_loaded, gt + 1);
       }
-
-      if (nrows == kWave && lane == kWave - 1) {
-        const int done = max(0, min(e0 + kChunk - (kWave - 1), cols));
-        __hip_atomic_store(&ready[w], my_base + done, __ATOMIC_RELEASE,
-                           __HIP_MEMORY_SCOPE_WORKGROUP);
+      tile_base += g.ntiles;
+    }
+    // the last two tiles: flush them once the sweep wave is done with them
+    {
+      int bands_done = 0;
+      while (bands_done * band_rows <= NS &&
+             band_of(bands_done, w, nsweep, NS, NT).row0 <= NS)
+        ++bands_done;
+      if (bands_done == 0) return;
+      const Band g = band_of(bands_done - 1, w, nsweep, NS, NT);
+      for (int back = min(2, tile_base); back >= 1; --back) {
+        const int gt = tile_base - back;
+        if (!wait_for(&cnt.consumed[w], gt + 1)) return;
+        const int m = g.ntiles - back;
+        if (m >= 0) {
+          flush(g, m, gt);
+        } else {
+          const Band pg = band_of(bands_done - 2, w, nsweep, NS, NT);
+          flush(pg, pg.ntiles + m, gt);
+        }
       }
     }
+    return;
+  }
+
+  // -------------------------------- sweep wave ---------------------------------
+  const int w = wave;
+  const int prev = (w + nsweep - 1) % nsweep;
+  R *my_seam = seam + (size_t)w * TP;
+  const R *up_seam = seam + (size_t)prev * TP;
+  R *base = tiles + (size_t)w * 8 * kTileElems;
+  const R seed = ans_grad[b];
+  int tile_base = 0;
+  for (int band = 0; band * band_rows <= NS; ++band) {
+    const Band g = band_of(band, w, nsweep, NS, NT);
+    if (g.row0 > NS) break;
+    const int r = g.row0 + lane;
+    const bool row_ok = r <= NS;
+    const bool has_up = g.row0 > 0;
+    const int up_base = (w > 0 ? band : band - 1) * cols;
+    const int my_base = band * cols;
+
+    // the seed enters as "handed left" into the first cell of the reversed sweep
+    R to_below = 0, to_below2 = 0, to_left = (r == 0) ? seed : (R)0;
+    R g_origin = 0;  // gradient of this lane's cell in reversed column NT
+    const bool has_down = g.nrows == kWave;
+    for (int m = 0; m < g.ntiles; ++m) {
+      const int gt = tile_base + m;
+#pragma unroll
+      for (int l = 0; l < kBwdStagers; ++l)
+        if (!wait_for(&cnt.loaded[w * kBwdStagers + l], gt + 1)) return;
+      R d1q[kTileSteps], d2q[kTileSteps];
+      {
+        const R *d1s = base + (gt & 1) * kTileElems + lane * kTilePitch;
+        const R *d2s = base + (2 + (gt & 1)) * kTileElems + lane * kTilePitch;
+#pragma unroll
+        for (int kk = 0; kk < kTileSteps; ++kk) {
+          d1q[kk] = d1s[kk];
+          d2q[kk] = d2s[kk];
+        }
+      }
+      R *gxs = base + (4 + (gt & 1)) * kTileElems + lane * kTilePitch;
+      R *gys = base + (6 + (gt & 1)) * kTileElems + lane * kTilePitch;
+
+      bool alive = true;
+      auto chunk = [&](auto up_c, auto down_c, auto edge_c, int c4, int e0)
+                       __attribute__((always_inline)) {
+        constexpr bool kUp = decltype(up_c)::value;
+        constexpr bool kDown = decltype(down_c)::value;
+        constexpr bool kEdge = decltype(edge_c)::value;
+        R handed = 0;
+        if (kUp) {
+          const int need = min(e0 + kChunk - shift, cols);
+          if (need > 0 && !wait_for(&cnt.ready[prev], up_base + need)) {
+            alive = false;
+            return;
+          }
+          const int col = e0 + lane - shift;
+          if (lane < kChunk && col >= 0 && col <= NT) handed = up_seam[col];
+        }
+        R *sp = my_seam + (e0 - (kWave - 1));
+#pragma unroll
+        for (int k = 0; k < kChunk; ++k) {
+          const int kk = c4 * kChunk + k;
+          R from_above = from_lane_below_zero(kModified ? to_below2 : to_below);
+          if (kUp) {
+            const R first = lane_value(handed, k);
+            from_above = (lane == 0) ? first : from_above;
+          }
+          // cells outside the window carry d1 = d2 = 0, so nothing leaks in or out
+          const R gcell = from_above + to_left;
+          const R down = d1q[kk] * gcell;
+          const R left = d2q[kk] * gcell;
+          gxs[kk] = down;
+          gys[kk] = left;
+          const int c63 = e0 + k - (kWave - 1);  // reversed column of the seam lane
+          if (kEdge) {
+            const int c = e0 + k - lane;
+            g_origin = (c == NT) ? gcell : g_origin;
+            if (kDown && c63 >= 0 && c63 <= NT && lane == kWave - 1) sp[k] = down;
+          } else {
+            if (kDown && lane == kWave - 1) sp[k] = down;
+          }
+          to_below2 = to_below;
+          to_below = down;
+          to_left = left;
+        }
+        if (kDown && lane == kWave - 1) {
+          const int done = max(0, min(e0 + kChunk - (kWave - 1), cols));
+          publish(&cnt.ready[w], my_base + done);
+        }
+      };
+      auto tile = [&](auto up_c, auto down_c) __attribute__((always_inline)) {
+#pragma unroll
+        for (int c4 = 0; c4 < kTileSteps / kChunk; ++c4) {
+          const int e0 = m * kTileSteps + c4 * kChunk;
+          if (e0 < g.nsteps && alive) {
+            const bool interior = e0 >= kWave - 1 && e0 + kChunk <= NT;
+            if (interior)
+              chunk(up_c, down_c, std::false_type{}, c4, e0);
+            else
+              chunk(up_c, down_c, std::true_type{}, c4, e0);
+          }
+        }
+      };
+      if (has_up) {
+        if (has_down)
+          tile(std::true_type{}, std::true_type{});
+        else
+          tile(std::true_type{}, std::false_type{});
+      } else {
+        if (has_down)
+          tile(std::false_type{}, std::true_type{});
+        else
+          tile(std::false_type{}, std::false_type{});
+      }
+      if (!alive) return;
+      if (lane == 0) publish(&cnt.consumed[w], gt + 1);
+    }
+    if (row_ok && r == NS && overwrite_ans_grad) ans_grad[b] = g_origin;
+    tile_base += g.ntiles;
   }
 }
 
-// Waves per workgroup: enough for every row when the seam rows fit in LDS.
-int pick_waves(int S, int T, size_t elem, size_t lds_budget) {
-  int nw = (S + 1 + kWave - 1) / kWave;
-  if (nw < 1) nw = 1;
-  if (nw > kMaxWaves) nw = kMaxWaves;
-  while (nw > 1 && (size_t)nw * (T + 1) * elem > lds_budget) --nw;
-  return nw;
-}
+constexpr size_t kLdsBudget = 156 * 1024;
 
-constexpr size_t kLdsBudget = 150 * 1024;
+// Sweep waves per workgroup: one per 64 rows, as many as LDS allows.
+int pick_sweep_waves(int S, int T, size_t elem, int arrays) {
+  int n = (S + 1 + kWave - 1) / kWave;
+  n = n < 1 ? 1 : (n > kMaxSweep ? kMaxSweep : n);
+  auto bytes = [&](int k) {
+    return (size_t)k * ((size_t)(T + 1) + (size_t)arrays * 2 * kTileElems) * elem;
+  };
+  while (n > 1 && bytes(n) > kLdsBudget) --n;
+  return n;
+}
 
 template <typename R>
 int forward_impl(const R *px, const R *py, const int64_t *boundary, R *p, R *ans, int B, int S,
@@ -336,21 +617,17 @@ int forward_impl(const R *px, const R *py, const int64_t *boundary, R *p, R *ans
   if (B < 0 || S < 0 || T < 0) return fail(FRNNT_EINVAL, "mi_forward: negative size");
   if (B == 0) return FRNNT_OK;
   if (!px || !py || !p || !ans) return fail(FRNNT_EINVAL, "mi_forward: null pointer");
-  if (modified && S > 0 && T == 0) { /* px has zero columns; still fine */ }
-  const int nw = pick_waves(S, T, sizeof(R), kLdsBudget);
-  const size_t lds = (size_t)nw * (T + 1) * sizeof(R);
-  if (lds > kLdsBudget) return fail(FRNNT_ELIMIT, "mi_forward: T=%d needs %zu bytes of LDS", T, lds);
-  // two register budgets: workgroups of up to 4 waves may use 512 VGPRs per lane
-  auto kernel = nw <= 4 ? (modified ? mi_forward_kernel<R, true, 256> : mi_forward_kernel<R, false, 256>)
-                        : (modified ? mi_forward_kernel<R, true, 1024>
-                                    : mi_forward_kernel<R, false, 1024>);
-  if (lds > 64 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return check_launch("mi_forward: hipFuncSetAttribute");
-  }
-  hipLaunchKernelGGL(kernel, dim3(B), dim3(nw * kWave), lds, static_cast<hipStream_t>(stream), px,
-                     py, boundary, p, ans, S, T);
+  const int n = pick_sweep_waves(S, T, sizeof(R), 2);
+  const size_t lds = (size_t)n * ((size_t)(T + 1) + 4 * kTileElems) * sizeof(R);
+  if (lds > kLdsBudget)
+    return fail(FRNNT_ELIMIT, "mi_forward: T=%d needs %zu bytes of LDS", T, lds);
+  auto kernel = modified ? mi_forward_kernel<R, true> : mi_forward_kernel<R, false>;
+  if (lds > 64 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return check_launch("mi_forward: hipFuncSetAttribute");
+  hipLaunchKernelGGL(kernel, dim3(B), dim3(n * (1 + kFwdStagers) * kWave), lds,
+                     static_cast<hipStream_t>(stream), px, py, boundary, p, ans, S, T);
   return check_launch("mi_forward");
 }
 
@@ -363,21 +640,18 @@ int backward_impl(const R *px, const R *py, const int64_t *boundary, const R *p,
   if (B == 0) return FRNNT_OK;
   if (!px || !p || !ans_grad || !px_grad || !py_grad)
     return fail(FRNNT_EINVAL, "mi_backward: null pointer");
-  const int nw = pick_waves(S, T, sizeof(R), kLdsBudget);
-  const size_t lds = (size_t)nw * (T + 1) * sizeof(R);
+  const int n = pick_sweep_waves(S, T, sizeof(R), 4);
+  const size_t lds = (size_t)n * ((size_t)(T + 1) + 8 * kTileElems) * sizeof(R);
   if (lds > kLdsBudget)
     return fail(FRNNT_ELIMIT, "mi_backward: T=%d needs %zu bytes of LDS", T, lds);
-  auto kernel = nw <= 4 ? (modified ? mi_backward_kernel<R, true, 256>
-                                    : mi_backward_kernel<R, false, 256>)
-                        : (modified ? mi_backward_kernel<R, true, 1024>
-                                    : mi_backward_kernel<R, false, 1024>);
-  if (lds > 64 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return check_launch("mi_backward: hipFuncSetAttribute");
-  }
-  hipLaunchKernelGGL(kernel, dim3(B), dim3(nw * kWave), lds, static_cast<hipStream_t>(stream), px,
-                     boundary, p, ans_grad, px_grad, py_grad, S, T, overwrite_ans_grad);
+  auto kernel = modified ? mi_backward_kernel<R, true> : mi_backward_kernel<R, false>;
+  if (lds > 64 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return check_launch("mi_backward: hipFuncSetAttribute");
+  hipLaunchKernelGGL(kernel, dim3(B), dim3(n * (1 + kBwdStagers) * kWave), lds,
+                     static_cast<hipStream_t>(stream), px, boundary, p, ans_grad, px_grad,
+                     py_grad, S, T, overwrite_ans_grad);
   return check_launch("mi_backward");
 }
 
