@@ -7,5 +7,13 @@ from ._fast_rnnt import with_cuda
 from .mutual_information import mutual_information_recursion
 from .mutual_information import joint_mutual_information_recursion
 
+from .rnnt_loss import do_rnnt_pruning
 from .rnnt_loss import get_rnnt_logprobs
+from .rnnt_loss import get_rnnt_logprobs_joint
+from .rnnt_loss import get_rnnt_logprobs_pruned
+from .rnnt_loss import get_rnnt_logprobs_smoothed
+from .rnnt_loss import get_rnnt_prune_ranges
+from .rnnt_loss import rnnt_loss
+from .rnnt_loss import rnnt_loss_pruned
 from .rnnt_loss import rnnt_loss_simple
+from .rnnt_loss import rnnt_loss_smoothed

@@ -33,6 +33,16 @@ _SIGNATURES = {
     "frnnt_simple_logprobs_fwd_f64": ([_P] * 9 + [_I] * 6 + [_P], _I),
     "frnnt_simple_logprobs_bwd_f32": ([_P] * 15 + [_I] * 6 + [_P], _I),
     "frnnt_simple_logprobs_bwd_f64": ([_P] * 15 + [_I] * 6 + [_P], _I),
+    "frnnt_lattice_logprobs_fwd_f32": ([_P] * 9 + [_I] * 7 + [_P], _I),
+    "frnnt_lattice_logprobs_fwd_f64": ([_P] * 9 + [_I] * 7 + [_P], _I),
+    "frnnt_lattice_logprobs_bwd_f32": ([_P] * 8 + [_I] * 7 + [_P], _I),
+    "frnnt_lattice_logprobs_bwd_f64": ([_P] * 8 + [_I] * 7 + [_P], _I),
+    "frnnt_prune_ranges_f32": ([_P] * 4 + [_I] * 5 + [_P], _I),
+    "frnnt_prune_ranges_f64": ([_P] * 4 + [_I] * 5 + [_P], _I),
+    "frnnt_prune_gather_f32": ([_P] * 3 + [_I] * 5 + [_P], _I),
+    "frnnt_prune_gather_f64": ([_P] * 3 + [_I] * 5 + [_P], _I),
+    "frnnt_prune_gather_bwd_f32": ([_P] * 3 + [_I] * 5 + [_P], _I),
+    "frnnt_prune_gather_bwd_f64": ([_P] * 3 + [_I] * 5 + [_P], _I),
 }
 
 

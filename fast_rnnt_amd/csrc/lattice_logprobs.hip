@@ -1,0 +1,272 @@
+// px / py from joiner logits: the unpruned loss (logits [B][T][S+1][C],
+// fast_rnnt/python/fast_rnnt/rnnt_loss.py:343-449) and the pruned loss
+// (logits [B][T][R][C] plus ranges [B][T][R], rnnt_loss.py:856-1024) share one
+// set of kernels; the unpruned case is R = S+1 with every range starting at 0.
+//
+// Forward, HBM-streaming: one wave per logits row (b, t, j) makes one pass for
+// the maximum and one for sum exp(x - max) (the second pass hits L1/L2), then
+// emits norm = logsumexp and the two picked log-probs
+//   xr[b,t,j] = logits[b,t,j,sym(b, ranges[b,t,j])] - norm   (sym(b, S) = termination symbol)
+//   yr[b,t,j] = logits[b,t,j,term] - norm.
+// A second, small kernel lays them out as px [B][S][T1] / py [B][S+1][T]: row
+// j of frame t lands at lattice row (j + ranges[b,t,0]) mod (S+1), everything
+// else is -inf, plus the -inf columns of the regular lattice and the constrained
+// "px += py[:, 1:]" step.
+//
+// Backward, HBM-streaming: one wave per logits row,
+//   dlogits[c] = -softmax[c] * (gx + gy) + [c = sym] gx + [c = term] gy
+// with gx / gy the px / py gradients of the lattice cell the row was placed at.
+#include "common.hip.h"
+
+namespace frnnt {
+namespace {
+
+enum { kRegular = 0, kModified = 1, kConstrained = 2 };
+
+template <typename R>
+__device__ __forceinline__ R wave_max_all(R v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const R o = __shfl_xor(v, off, 64);
+    v = (o > v || o != o) ? o : v;
+  }
+  return v;
+}
+template <typename R>
+__device__ __forceinline__ R wave_sum_all(R v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+template <typename R>
+__device__ __forceinline__ R exp_acc(R x);
+template <>
+__device__ __forceinline__ float exp_acc<float>(float x) {
+  return __expf(x);
+}
+template <>
+__device__ __forceinline__ double exp_acc<double>(double x) {
+  return exp(x);
+}
+template <typename R>
+__device__ __forceinline__ R log_acc(R x);
+template <>
+__device__ __forceinline__ float log_acc<float>(float x) {
+  return logf(x);
+}
+template <>
+__device__ __forceinline__ double log_acc<double>(double x) {
+  return log(x);
+}
+
+// Symbol scored by row j of frame (b, t): symbols[b][s] for s < S, the
+// termination symbol for s == S; -1 if the range entry is out of [0, S].
+__device__ __forceinline__ int64_t row_symbol(const int64_t *symbols, const int64_t *ranges,
+                                              long row, int b, int j, int S, int term) {
+  const int64_t s = ranges ? ranges[row] : j;
+  if (s < 0 || s > S) return -1;
+  return s == S ? (int64_t)term : symbols[(long)b * S + s];
+}
+
+// 4 rows per 256-thread block.
+template <typename R>
+__global__ void __launch_bounds__(256)
+    row_norm_kernel(const R *__restrict__ logits, const int64_t *__restrict__ symbols,
+                    const int64_t *__restrict__ ranges, R *__restrict__ norm, R *__restrict__ xr,
+                    R *__restrict__ yr, long rows, int T, int Rr, int S, int C, int term) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const R *x = logits + row * C;
+  R m = Num<R>::neg_inf();
+  for (int c = lane; c < C; c += kWave) {
+    const R v = x[c];
+    m = (v > m || v != v) ? v : m;
+  }
+  m = wave_max_all(m);
+  const R shift = (m - m == 0) ? m : (R)0;  // torch.logsumexp: infinite max -> shift by 0
+  R sum = 0;
+  for (int c = lane; c < C; c += kWave) sum += exp_acc<R>(x[c] - shift);
+  sum = wave_sum_all(sum);
+  const R lse = log_acc<R>(sum) + shift;
+  if (lane == 0) {
+    const int j = (int)(row % Rr);
+    const int b = (int)(row / ((long)Rr * T));
+    const int64_t sym = row_symbol(symbols, ranges, row, b, j, S, term);
+    norm[row] = lse;
+    xr[row] = (sym >= 0 && sym < C) ? x[sym] - lse : std::numeric_limits<R>::quiet_NaN();
+    yr[row] = x[term] - lse;
+  }
+}
+
+// One thread per px / py element, t fastest (coalesced stores).
+template <typename R>
+__global__ void __launch_bounds__(256)
+    assemble_kernel(const R *__restrict__ xr, const R *__restrict__ yr,
+                    const int64_t *__restrict__ ranges, const int64_t *__restrict__ boundary,
+                    R *__restrict__ px, R *__restrict__ py, int B, int S, int T, int Rr,
+                    int rnnt_type) {
+  const int T1 = rnnt_type == kRegular ? T + 1 : T;
+  const int S1 = S + 1;
+  const long n_px = (long)B * S * T1, n_py = (long)B * S1 * T;
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  const R ninf = Num<R>::neg_inf();
+  // value of the staged row that the roll places at lattice row s of frame t
+  auto placed = [&](const R *src, int b, int s, int t) -> R {
+    const long frame = ((long)b * T + t) * Rr;
+    const int64_t r0 = ranges ? ranges[frame] : 0;
+    int64_t rel = ((int64_t)s - r0) % S1;
+    if (rel < 0) rel += S1;
+    return rel < Rr ? src[frame + rel] : ninf;
+  };
+  if (idx < n_px) {
+    const int b = (int)(idx / ((long)S * T1));
+    const long rem = idx - (long)b * S * T1;
+    const int s = (int)(rem / T1), t = (int)(rem % T1);
+    R v = ninf;
+    if (t < T) {
+      v = placed(xr, b, s, t);
+      if (rnnt_type == kRegular && boundary && boundary[4 * b + 3] == t) v = ninf;
+      if (rnnt_type == kConstrained) v += placed(yr, b, s + 1, t);
+    }
+    px[idx] = v;
+  } else if (idx < n_px + n_py) {
+    const long k = idx - n_px;
+    const int b = (int)(k / ((long)S1 * T));
+    const long rem = k - (long)b * S1 * T;
+    const int s = (int)(rem / T), t = (int)(rem % T);
+    py[k] = placed(yr, b, s, t);
+  }
+}
+
+// One wave per logits row.
+template <typename R>
+__global__ void __launch_bounds__(256)
+    row_grad_kernel(const R *__restrict__ logits, const int64_t *__restrict__ symbols,
+                    const int64_t *__restrict__ ranges, const int64_t *__restrict__ boundary,
+                    const R *__restrict__ norm, const R *__restrict__ gpx,
+                    const R *__restrict__ gpy, R *__restrict__ glogits, long rows, int S, int T,
+                    int Rr, int C, int term, int rnnt_type) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const int S1 = S + 1;
+  const int T1 = rnnt_type == kRegular ? T + 1 : T;
+  const int j = (int)(row % Rr);
+  const long frame = row / Rr;
+  const int t = (int)(frame % T), b = (int)(frame / T);
+  const int64_t r0 = ranges ? ranges[frame * Rr] : 0;
+  // lattice row this logits row was placed at; rows the roll pushes past S+1 wrap
+  // around exactly as in the forward pass
+  int64_t s64 = ((int64_t)j + r0) % S1;
+  if (s64 < 0) s64 += S1;
+  const int s = (int)s64;
+  const bool masked = rnnt_type == kRegular && boundary && boundary[4 * b + 3] == t;
+  auto gx_at = [&](int ss) -> R {
+    if (ss < 0 || ss >= S || masked) return (R)0;
+    return gpx[((long)b * S + ss) * T1 + t];
+  };
+  const R gx = gx_at(s);
+  R gy = gpy[((long)b * S1 + s) * T + t];
+  if (rnnt_type == kConstrained) gy += gx_at(s - 1);
+  const int64_t sym = row_symbol(symbols, ranges, row, b, j, S, term);
+  const R lse = norm[row];
+  const R w = -(gx + gy);
+  const R *x = logits + row * C;
+  R *g = glogits + row * C;
+  for (int c = lane; c < C; c += kWave) {
+    R v = exp_acc<R>(x[c] - lse) * w;
+    if (c == sym) v += gx;
+    if (c == term) v += gy;
+    g[c] = v;
+  }
+}
+
+template <typename R>
+int fwd_impl(const R *logits, const int64_t *symbols, const int64_t *ranges,
+             const int64_t *boundary, R *px, R *py, R *norm, R *xr, R *yr, int B, int S, int T,
+             int Rr, int C, int term, int rnnt_type, void *stream_) {
+  if (B < 0 || S < 0 || T < 0 || Rr < 1 || C < 1)
+    return fail(FRNNT_EINVAL, "lattice_logprobs_fwd: bad size");
+  if (Rr > S + 1) return fail(FRNNT_EINVAL, "lattice_logprobs_fwd: more range rows than S + 1");
+  if (!ranges && Rr != S + 1)
+    return fail(FRNNT_EINVAL, "lattice_logprobs_fwd: without ranges the logits need S + 1 rows");
+  if (rnnt_type < 0 || rnnt_type > 2 || term < 0 || term >= C)
+    return fail(FRNNT_EINVAL, "lattice_logprobs_fwd: bad rnnt_type or termination symbol");
+  if (B == 0) return FRNNT_OK;
+  if (!logits || (!symbols && S > 0) || !px || !py || !norm || !xr || !yr)
+    return fail(FRNNT_EINVAL, "lattice_logprobs_fwd: null pointer");
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  const long rows = (long)B * T * Rr;
+  if (rows > 0)
+    hipLaunchKernelGGL(row_norm_kernel<R>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream,
+                       logits, symbols, ranges, norm, xr, yr, rows, T, Rr, S, C, term);
+  const int T1 = rnnt_type == kRegular ? T + 1 : T;
+  const long total = (long)B * S * T1 + (long)B * (S + 1) * T;
+  if (total > 0)
+    hipLaunchKernelGGL(assemble_kernel<R>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                       stream, xr, yr, ranges, boundary, px, py, B, S, T, Rr, rnnt_type);
+  return check_launch("lattice_logprobs_fwd");
+}
+
+template <typename R>
+int bwd_impl(const R *logits, const int64_t *symbols, const int64_t *ranges,
+             const int64_t *boundary, const R *norm, const R *px_grad, const R *py_grad,
+             R *logits_grad, int B, int S, int T, int Rr, int C, int term, int rnnt_type,
+             void *stream_) {
+  if (B < 0 || S < 0 || T < 0 || Rr < 1 || C < 1 || Rr > S + 1 || (!ranges && Rr != S + 1))
+    return fail(FRNNT_EINVAL, "lattice_logprobs_bwd: bad size");
+  if (rnnt_type < 0 || rnnt_type > 2 || term < 0 || term >= C)
+    return fail(FRNNT_EINVAL, "lattice_logprobs_bwd: bad rnnt_type or termination symbol");
+  if (B == 0 || T == 0) return FRNNT_OK;
+  if (!logits || (!symbols && S > 0) || !norm || !px_grad || !py_grad || !logits_grad)
+    return fail(FRNNT_EINVAL, "lattice_logprobs_bwd: null pointer");
+  const long rows = (long)B * T * Rr;
+  hipLaunchKernelGGL(row_grad_kernel<R>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream_), logits, symbols, ranges, boundary, norm,
+                     px_grad, py_grad, logits_grad, rows, S, T, Rr, C, term, rnnt_type);
+  return check_launch("lattice_logprobs_bwd");
+}
+
+}  // namespace
+}  // namespace frnnt
+
+extern "C" {
+
+int frnnt_lattice_logprobs_fwd_f32(const float *logits, const int64_t *symbols,
+                                   const int64_t *ranges, const int64_t *boundary, float *px,
+                                   float *py, float *norm, float *xr, float *yr, int B, int S,
+                                   int T, int R, int C, int termination_symbol, int rnnt_type,
+                                   void *stream) {
+  return frnnt::fwd_impl<float>(logits, symbols, ranges, boundary, px, py, norm, xr, yr, B, S, T, R,
+                                C, termination_symbol, rnnt_type, stream);
+}
+int frnnt_lattice_logprobs_fwd_f64(const double *logits, const int64_t *symbols,
+                                   const int64_t *ranges, const int64_t *boundary, double *px,
+                                   double *py, double *norm, double *xr, double *yr, int B, int S,
+                                   int T, int R, int C, int termination_symbol, int rnnt_type,
+                                   void *stream) {
+  return frnnt::fwd_impl<double>(logits, symbols, ranges, boundary, px, py, norm, xr, yr, B, S, T,
+                                 R, C, termination_symbol, rnnt_type, stream);
+}
+int frnnt_lattice_logprobs_bwd_f32(const float *logits, const int64_t *symbols,
+                                   const int64_t *ranges, const int64_t *boundary,
+                                   const float *norm, const float *px_grad, const float *py_grad,
+                                   float *logits_grad, int B, int S, int T, int R, int C,
+                                   int termination_symbol, int rnnt_type, void *stream) {
+  return frnnt::bwd_impl<float>(logits, symbols, ranges, boundary, norm, px_grad, py_grad,
+                                logits_grad, B, S, T, R, C, termination_symbol, rnnt_type, stream);
+}
+int frnnt_lattice_logprobs_bwd_f64(const double *logits, const int64_t *symbols,
+                                   const int64_t *ranges, const int64_t *boundary,
+                                   const double *norm, const double *px_grad,
+                                   const double *py_grad, double *logits_grad, int B, int S, int T,
+                                   int R, int C, int termination_symbol, int rnnt_type,
+                                   void *stream) {
+  return frnnt::bwd_impl<double>(logits, symbols, ranges, boundary, norm, px_grad, py_grad,
+                                 logits_grad, B, S, T, R, C, termination_symbol, rnnt_type,
+                                 stream);
+}
+
+}  // extern "C"

@@ -184,3 +184,322 @@ def rnnt_loss_simple(
                                boundary=boundary, rnnt_type=rnnt_type)
     return _recursion_and_reduce(px, py, boundary, rnnt_type, delay_penalty, reduction,
                                  return_grad)
+
+
+class _LatticeLogprobs(torch.autograd.Function):
+    """(px, py) from joiner logits, pruned (``ranges`` given) or not:
+    frnnt_lattice_logprobs_fwd/bwd."""
+
+    @staticmethod
+    def forward(ctx, logits, symbols, ranges, boundary, termination_symbol, rnnt_type):
+        B, T, R, C = logits.shape
+        S = symbols.shape[1]
+        kind = _RNNT_TYPES[rnnt_type]
+        sfx = _lib.suffix(logits.dtype)
+        lg = logits.contiguous()
+        sym_c = symbols.contiguous()
+        rng_c = ranges.contiguous() if ranges is not None else None
+        bnd_c = boundary.contiguous() if boundary is not None else None
+        opts = dict(dtype=logits.dtype, device=logits.device)
+        T1 = T + 1 if kind == 0 else T
+        with torch.cuda.device(logits.device):
+            px = torch.empty(B, S, T1, **opts)
+            py = torch.empty(B, S + 1, T, **opts)
+            norm = torch.empty(B, T, R, **opts)
+            xr = torch.empty(B, T, R, **opts)
+            yr = torch.empty(B, T, R, **opts)
+            _lib.call("frnnt_lattice_logprobs_fwd_" + sfx, lg.data_ptr(), sym_c.data_ptr(),
+                      _lib.ptr(rng_c), _lib.ptr(bnd_c), px.data_ptr(), py.data_ptr(),
+                      norm.data_ptr(), xr.data_ptr(), yr.data_ptr(), B, S, T, R, C,
+                      int(termination_symbol), kind, _lib.stream_of(logits))
+        if ctx.needs_input_grad[0]:
+            ctx.save_for_backward(lg, sym_c, rng_c, bnd_c, norm)
+            ctx.meta = (B, S, T, R, C, int(termination_symbol), kind, sfx)
+        return px, py
+
+    @staticmethod
+    def backward(ctx, gpx, gpy):
+        lg, sym, rng, bnd, norm = ctx.saved_tensors
+        B, S, T, R, C, term, kind, sfx = ctx.meta
+        opts = dict(dtype=lg.dtype, device=lg.device)
+        T1 = T + 1 if kind == 0 else T
+        with torch.cuda.device(lg.device):
+            gpx = torch.zeros(B, S, T1, **opts) if gpx is None else gpx.contiguous()
+            gpy = torch.zeros(B, S + 1, T, **opts) if gpy is None else gpy.contiguous()
+            grad = torch.empty_like(lg)
+            _lib.call("frnnt_lattice_logprobs_bwd_" + sfx, lg.data_ptr(), sym.data_ptr(),
+                      _lib.ptr(rng), _lib.ptr(bnd), norm.data_ptr(), gpx.data_ptr(),
+                      gpy.data_ptr(), grad.data_ptr(), B, S, T, R, C, term, kind,
+                      _lib.stream_of(lg))
+        return grad, None, None, None, None, None
+
+
+def get_rnnt_logprobs_joint(
+    logits: Tensor, symbols: Tensor, termination_symbol: int,
+    boundary: Optional[Tensor] = None, rnnt_type: str = "regular",
+) -> Tuple[Tensor, Tensor]:
+    """(px, py) from the full joiner output ``logits`` of shape ``(B, T, S+1, C)``
+    (fast_rnnt/python/fast_rnnt/rnnt_loss.py:343-449)."""
+    assert logits.ndim == 4, logits.ndim
+    (B, T, S1, C) = logits.shape
+    S = S1 - 1
+    assert symbols.shape == (B, S), symbols.shape
+    validate_st_lengths(S, T, rnnt_type == "regular", boundary)
+    assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
+    _require_gpu(logits, symbols, boundary)
+    return _LatticeLogprobs.apply(logits, symbols, None, boundary, termination_symbol, rnnt_type)
+
+
+def rnnt_loss(
+    logits: Tensor, symbols: Tensor, termination_symbol: int,
+    boundary: Optional[Tensor] = None, rnnt_type: str = "regular",
+    delay_penalty: float = 0.0, reduction: Optional[str] = "mean", return_grad: bool = False,
+) -> Tensor:
+    """The unpruned RNN-T loss on joiner logits ``(B, T, S+1, C)`` (rnnt_loss.py:452-547)."""
+    px, py = get_rnnt_logprobs_joint(logits=logits, symbols=symbols,
+                                     termination_symbol=termination_symbol,
+                                     boundary=boundary, rnnt_type=rnnt_type)
+    return _recursion_and_reduce(px, py, boundary, rnnt_type, delay_penalty, reduction,
+                                 return_grad)
+
+
+def _monotonic_lower_bound(x: Tensor) -> Tensor:
+    """Suffix minimum along the last axis: the largest non-decreasing sequence
+    below ``x`` (rnnt_loss.py:550-581), e.g. [0,2,1,3,6,5,8] -> [0,1,1,3,5,5,8]."""
+    x = torch.flip(x, dims=(-1,))
+    x, _ = torch.cummin(x, dim=-1)
+    return torch.flip(x, dims=(-1,))
+
+
+def _adjust_pruning_lower_bound(s_begin: Tensor, s_range: int) -> Tensor:
+    """Make ``s_begin`` (B, T) non-decreasing, starting at 0, with steps below
+    ``s_range`` (rnnt_loss.py:584-632).  Torch-op form of what the prune-range
+    kernel does in LDS; kept for callers that use it on its own."""
+    (B, T) = s_begin.shape
+    ramp = (s_range - 1) * torch.arange(0, T, device=s_begin.device)
+    s_begin = _monotonic_lower_bound(s_begin)
+    s_begin = torch.clamp(_monotonic_lower_bound(ramp - s_begin), min=0)
+    return ramp - s_begin
+
+
+def get_rnnt_prune_ranges(px_grad: Tensor, py_grad: Tensor, boundary: Tensor,
+                          s_range: int) -> Tensor:
+    """Pruning bounds from the occupation gradients (rnnt_loss.py:638-777).
+
+    Returns an int64 tensor ``(B, T, s_range)``: for each frame the ``s_range``
+    consecutive symbol positions kept.  As in the reference, ``s_range`` is raised
+    (with a printed warning) to the minimum the regular lattice needs and capped
+    at ``S + 1``, so the last dimension can differ from the request.
+    """
+    (B, S, T1) = px_grad.shape
+    T = py_grad.shape[-1]
+    is_regular = T1 != T
+    assert T1 in [T, T + 1], T1
+    assert py_grad.shape == (B, S + 1, T), py_grad.shape
+    assert boundary.shape == (B, 4), boundary.shape
+    validate_st_lengths(S, T, is_regular, boundary)
+    _require_gpu(px_grad, py_grad, boundary)
+
+    if is_regular:
+        Ss = boundary[:, 2]
+        Ts = boundary[:, 3]
+        s_range_min = Ss.sub(1).div(Ts, rounding_mode="trunc").add(2).max().item()
+        if s_range < s_range_min:
+            print(f"Warning: get_rnnt_prune_ranges - got s_range={s_range} "
+                  f"for boundaries S={Ss}, T={Ts}. Adjusting to {s_range_min}")
+            s_range = s_range_min
+    if s_range > S:
+        s_range = S + 1
+    if is_regular:
+        assert s_range >= 2, (
+            "Pruning range for standard RNN-T should be equal to or greater than 2, "
+            "or no valid paths could survive pruning.")
+    else:
+        assert s_range >= 1, (
+            "Pruning range for modified RNN-T should be equal to or greater than 1, "
+            "or no valid paths could survive pruning.")
+
+    sfx = _lib.suffix(px_grad.dtype)
+    gx, gy = px_grad.detach().contiguous(), py_grad.detach().contiguous()
+    bnd = boundary.contiguous()
+    with torch.cuda.device(px_grad.device):
+        ranges = torch.empty(B, T, int(s_range), dtype=torch.int64, device=px_grad.device)
+        _lib.call("frnnt_prune_ranges_" + sfx, gx.data_ptr(), gy.data_ptr(), bnd.data_ptr(),
+                  ranges.data_ptr(), B, S, T, int(not is_regular), int(s_range),
+                  _lib.stream_of(px_grad))
+    return ranges
+
+
+class _PruneGather(torch.autograd.Function):
+    """lm_pruned[b,t,j,:] = lm[b, ranges[b,t,j], :]: frnnt_prune_gather / _bwd."""
+
+    @staticmethod
+    def forward(ctx, lm, ranges):
+        B, S1, C = lm.shape
+        _, T, R = ranges.shape
+        sfx = _lib.suffix(lm.dtype)
+        lm_c, rng_c = lm.contiguous(), ranges.contiguous()
+        with torch.cuda.device(lm.device):
+            out = torch.empty(B, T, R, C, dtype=lm.dtype, device=lm.device)
+            _lib.call("frnnt_prune_gather_" + sfx, lm_c.data_ptr(), rng_c.data_ptr(),
+                      out.data_ptr(), B, S1 - 1, T, R, C, _lib.stream_of(lm))
+        ctx.save_for_backward(rng_c)
+        ctx.meta = (B, S1, T, R, C, sfx)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        (rng,) = ctx.saved_tensors
+        B, S1, T, R, C, sfx = ctx.meta
+        grad = grad.contiguous()
+        with torch.cuda.device(grad.device):
+            lm_grad = torch.empty(B, S1, C, dtype=grad.dtype, device=grad.device)
+            _lib.call("frnnt_prune_gather_bwd_" + sfx, grad.data_ptr(), rng.data_ptr(),
+                      lm_grad.data_ptr(), B, S1 - 1, T, R, C, _lib.stream_of(grad))
+        return lm_grad, None
+
+
+def do_rnnt_pruning(am: Tensor, lm: Tensor, ranges: Tensor) -> Tuple[Tensor, Tensor]:
+    """Prune encoder and predictor outputs with ``ranges`` (rnnt_loss.py:780-818).
+
+    Returns ``(am_pruned, lm_pruned)``, both ``(B, T, s_range, C)``; ``am_pruned``
+    is a zero-copy expanded view of ``am``, as in the reference.
+    """
+    assert ranges.shape[0] == am.shape[0], (ranges.shape[0], am.shape[0])
+    assert ranges.shape[0] == lm.shape[0], (ranges.shape[0], lm.shape[0])
+    assert am.shape[1] == ranges.shape[1], (am.shape[1], ranges.shape[1])
+    (B, T, s_range) = ranges.shape
+    (B, S1, C) = lm.shape
+    _require_gpu(am, lm, ranges)
+    am_pruning = am.unsqueeze(2).expand((B, T, s_range, C))
+    lm_pruning = _PruneGather.apply(lm, ranges)
+    return am_pruning, lm_pruning
+
+
+def _roll_by_shifts(src: Tensor, shifts: torch.LongTensor):
+    """``out[b,t,s] = src[b,t,(s - shifts[b,t]) mod S]`` (rnnt_loss.py:821-853).
+    The fused pruned-logprob kernel applies this roll itself; kept for callers."""
+    assert src.dim() == 3, src.dim()
+    (B, T, S) = src.shape
+    assert shifts.shape == (B, T), shifts.shape
+    index = (torch.arange(S, device=src.device).view(1, 1, S) - shifts.reshape(B, T, 1)) % S
+    return torch.gather(src, 2, index)
+
+
+def get_rnnt_logprobs_pruned(
+    logits: Tensor, symbols: Tensor, ranges: Tensor, termination_symbol: int,
+    boundary: Optional[Tensor] = None, rnnt_type: str = "regular",
+) -> Tuple[Tensor, Tensor]:
+    """(px, py) from pruned joiner logits ``(B, T, s_range, C)`` and the
+    ``ranges`` they were computed for (rnnt_loss.py:856-1024); lattice cells
+    outside the kept range of their frame are -inf."""
+    assert logits.ndim == 4, logits.ndim
+    (B, T, s_range, C) = logits.shape
+    assert ranges.shape == (B, T, s_range), f"{ranges.shape} == ({B}, {T}, {s_range})"
+    (B, S) = symbols.shape
+    validate_st_lengths(S, T, rnnt_type == "regular", boundary)
+    assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
+    _require_gpu(logits, symbols, ranges, boundary)
+    return _LatticeLogprobs.apply(logits, symbols, ranges, boundary, termination_symbol,
+                                  rnnt_type)
+
+
+def rnnt_loss_pruned(
+    logits: Tensor, symbols: Tensor, ranges: Tensor, termination_symbol: int,
+    boundary: Optional[Tensor] = None, rnnt_type: str = "regular",
+    delay_penalty: float = 0.0, reduction: Optional[str] = "mean", return_grad: bool = False,
+) -> Tensor:
+    """The pruned RNN-T loss on joiner logits ``(B, T, s_range, C)`` (rnnt_loss.py:1027-1132)."""
+    px, py = get_rnnt_logprobs_pruned(logits=logits, symbols=symbols, ranges=ranges,
+                                      termination_symbol=termination_symbol,
+                                      boundary=boundary, rnnt_type=rnnt_type)
+    return _recursion_and_reduce(px, py, boundary, rnnt_type, delay_penalty, reduction,
+                                 return_grad)
+
+
+def get_rnnt_logprobs_smoothed(
+    lm: Tensor, am: Tensor, symbols: Tensor, termination_symbol: int,
+    lm_only_scale: float = 0.1, am_only_scale: float = 0.1,
+    boundary: Optional[Tensor] = None, rnnt_type: str = "regular",
+) -> Tuple[Tensor, Tensor]:
+    """(px, py) interpolating the joint model with an lm-only and an am-only
+    (unigram-lm) model (rnnt_loss.py:1135-1369)::
+
+        (1 - lm_only_scale - am_only_scale) * joint + lm_only_scale * lm_only
+                                                    + am_only_scale * am_only
+
+    The joint part -- the [B,S+1,C] x [B,C,T] contraction and its px / py -- comes
+    from the fused MFMA kernel; the lm-only / am-only corrections are small
+    tensors handled with torch ops in the reference's order.
+    """
+    assert lm.ndim == 3, lm.ndim
+    assert am.ndim == 3, am.ndim
+    assert lm.shape[0] == am.shape[0], (lm.shape[0], am.shape[0])
+    assert lm.shape[2] == am.shape[2], (lm.shape[2], am.shape[2])
+    (B, T, C) = am.shape
+    S = lm.shape[1] - 1
+    assert symbols.shape == (B, S), symbols.shape
+    validate_st_lengths(S, T, rnnt_type == "regular", boundary)
+    assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
+    _require_gpu(lm, am, symbols, boundary)
+
+    # joint part, without the boundary / constrained post-processing (applied last)
+    base_type = "regular" if rnnt_type == "regular" else "modified"
+    px, py = _SimpleLogprobs.apply(lm, am, symbols, None, termination_symbol, base_type)
+
+    tiny = torch.finfo(lm.dtype).tiny
+    am_max, _ = torch.max(am, dim=2, keepdim=True)
+    lm_max, _ = torch.max(lm, dim=2, keepdim=True)
+    am_probs = (am - am_max).exp()
+    lm_probs = (lm - lm_max).exp()
+    lmonly_normalizers = lm_probs.sum(dim=2, keepdim=True)  # [B][S+1][1]
+    unigram_lm = torch.mean(lm_probs / lmonly_normalizers, dim=(0, 1), keepdim=True) + tiny
+    amonly_normalizers = (torch.mv(am_probs.reshape(-1, C), unigram_lm.reshape(C))
+                          .reshape(B, T, 1).log() + am_max).transpose(1, 2)  # [B][1][T]
+    unigram_lm = unigram_lm.log()
+    lmonly_normalizers = lmonly_normalizers.log() + lm_max
+
+    rows = torch.arange(B, device=am.device).reshape(B, 1)
+    px_am = am[rows, :, symbols]  # [B][S][T]
+    if rnnt_type == "regular":
+        px_am = torch.cat((px_am, px_am.new_full((B, S, 1), float("-inf"))), dim=2)
+    px_lm = torch.gather(lm[:, :S], dim=2, index=symbols.unsqueeze(-1))  # [B][S][1]
+    px_lm_unigram = unigram_lm.reshape(C)[symbols].unsqueeze(-1)  # [B][S][1]
+    px_amonly = px_am + px_lm_unigram
+    px_amonly[:, :, :T] -= amonly_normalizers
+    px_lmonly = px_lm - lmonly_normalizers[:, :S, :]
+
+    py_am = am[:, :, termination_symbol].unsqueeze(1)
+    py_lm = lm[:, :, termination_symbol].unsqueeze(2)
+    py_amonly = py_am + unigram_lm[0][0][termination_symbol] - amonly_normalizers
+    py_lmonly = py_lm - lmonly_normalizers
+
+    combined_scale = 1.0 - lm_only_scale - am_only_scale
+    # exact zeros would turn -inf * 0 into nan
+    if lm_only_scale == 0.0:
+        lm_only_scale = 1.0e-20
+    if am_only_scale == 0.0:
+        am_only_scale = 1.0e-20
+    px_interp = px * combined_scale + px_lmonly * lm_only_scale + px_amonly * am_only_scale
+    py_interp = py * combined_scale + py_lmonly * lm_only_scale + py_amonly * am_only_scale
+
+    if rnnt_type == "regular":
+        px_interp = fix_for_boundary(px_interp, boundary)
+    elif rnnt_type == "constrained":
+        px_interp += py_interp[:, 1:, :]
+    return (px_interp, py_interp)
+
+
+def rnnt_loss_smoothed(
+    lm: Tensor, am: Tensor, symbols: Tensor, termination_symbol: int,
+    lm_only_scale: float = 0.1, am_only_scale: float = 0.1,
+    boundary: Optional[Tensor] = None, rnnt_type: str = "regular",
+    delay_penalty: float = 0.0, reduction: Optional[str] = "mean", return_grad: bool = False,
+) -> Union[Tuple[Tensor, Tuple[Tensor, Tensor]], Tensor]:
+    """rnnt_loss_simple with lm-only / am-only smoothing (rnnt_loss.py:1372-1494)."""
+    px, py = get_rnnt_logprobs_smoothed(
+        lm=lm, am=am, symbols=symbols, termination_symbol=termination_symbol,
+        lm_only_scale=lm_only_scale, am_only_scale=am_only_scale, boundary=boundary,
+        rnnt_type=rnnt_type)
+    return _recursion_and_reduce(px, py, boundary, rnnt_type, delay_penalty, reduction,
+                                 return_grad)

@@ -131,6 +131,80 @@ int frnnt_simple_logprobs_bwd_f64(const double *lm, const double *am, const int6
                                   double *am_grad, int B, int S, int T, int C,
                                   int termination_symbol, int rnnt_type, void *stream);
 
+/*
+ * px / py from joiner logits.  Replaces the tensor algebra of
+ *   get_rnnt_logprobs_joint  (rnnt_loss.py:343-449)  when ranges == NULL, R == S+1,
+ *   get_rnnt_logprobs_pruned (rnnt_loss.py:856-1024) when ranges is given:
+ * logsumexp over the vocabulary, the symbol / termination-symbol picks, the -inf
+ * padding and per-frame roll that places range row j at lattice row
+ * (j + ranges[b][t][0]) mod (S+1), the -inf columns of the regular lattice and
+ * the constrained "px += py[:, 1:]" step.
+ *   logits [B][T][R][C]; symbols int64 [B][S]; ranges int64 [B][T][R] or NULL   in
+ *   boundary int64 [B][4] or NULL (only boundary[b][3] is used, regular lattice)
+ *   px [B][S][T+1] (rnnt_type 0) or [B][S][T]; py [B][S+1][T]                   out
+ *   norm, xr, yr [B][T][R]: out; norm (the logsumexp) is needed by the backward
+ *   entry point, xr / yr are staging buffers
+ */
+int frnnt_lattice_logprobs_fwd_f32(const float *logits, const int64_t *symbols,
+                                   const int64_t *ranges, const int64_t *boundary, float *px,
+                                   float *py, float *norm, float *xr, float *yr, int B, int S,
+                                   int T, int R, int C, int termination_symbol, int rnnt_type,
+                                   void *stream);
+int frnnt_lattice_logprobs_fwd_f64(const double *logits, const int64_t *symbols,
+                                   const int64_t *ranges, const int64_t *boundary, double *px,
+                                   double *py, double *norm, double *xr, double *yr, int B, int S,
+                                   int T, int R, int C, int termination_symbol, int rnnt_type,
+                                   void *stream);
+
+/*
+ * Backward of the above (what autograd derives for rnnt_loss.py:418-447 /
+ * :940-1022): logits_grad [B][T][R][C] =
+ *   -softmax * (gx + gy) + onehot(symbol) * gx + onehot(termination) * gy.
+ */
+int frnnt_lattice_logprobs_bwd_f32(const float *logits, const int64_t *symbols,
+                                   const int64_t *ranges, const int64_t *boundary,
+                                   const float *norm, const float *px_grad, const float *py_grad,
+                                   float *logits_grad, int B, int S, int T, int R, int C,
+                                   int termination_symbol, int rnnt_type, void *stream);
+int frnnt_lattice_logprobs_bwd_f64(const double *logits, const int64_t *symbols,
+                                   const int64_t *ranges, const int64_t *boundary,
+                                   const double *norm, const double *px_grad,
+                                   const double *py_grad, double *logits_grad, int B, int S, int T,
+                                   int R, int C, int termination_symbol, int rnnt_type,
+                                   void *stream);
+
+/*
+ * Pruning bounds.  Replaces the device work of get_rnnt_prune_ranges
+ * (rnnt_loss.py:726-777 with _adjust_pruning_lower_bound :584-632).  s_range is
+ * the FINAL window size: the caller has already raised it to the regular
+ * lattice's minimum and capped it at S+1 (rnnt_loss.py:696-724), so
+ * 1 <= s_range <= S+1.
+ *   px_grad [B][S][T+1] (modified: [B][S][T]), py_grad [B][S+1][T], boundary [B][4]  in
+ *   ranges int64 [B][T][s_range]                                                     out
+ */
+int frnnt_prune_ranges_f32(const float *px_grad, const float *py_grad, const int64_t *boundary,
+                           int64_t *ranges, int B, int S, int T, int modified, int s_range,
+                           void *stream);
+int frnnt_prune_ranges_f64(const double *px_grad, const double *py_grad, const int64_t *boundary,
+                           int64_t *ranges, int B, int S, int T, int modified, int s_range,
+                           void *stream);
+
+/*
+ * Pruning gather and its adjoint.  Replaces the gather of do_rnnt_pruning
+ * (rnnt_loss.py:813-817): lm_pruned[b][t][j][:] = lm[b][ranges[b][t][j]][:]
+ * (NaN rows for entries outside [0, S]); the adjoint sums the rows of `grad`
+ * that were taken from each lm row, in frame order.
+ *   lm [B][S+1][C], ranges int64 [B][T][R]; lm_pruned / grad [B][T][R][C]; lm_grad [B][S+1][C]
+ */
+int frnnt_prune_gather_f32(const float *lm, const int64_t *ranges, float *lm_pruned, int B, int S,
+                           int T, int R, int C, void *stream);
+int frnnt_prune_gather_f64(const double *lm, const int64_t *ranges, double *lm_pruned, int B, int S,
+                           int T, int R, int C, void *stream);
+int frnnt_prune_gather_bwd_f32(const float *grad, const int64_t *ranges, float *lm_grad, int B,
+                               int S, int T, int R, int C, void *stream);
+int frnnt_prune_gather_bwd_f64(const double *grad, const int64_t *ranges, double *lm_grad, int B,
+                               int S, int T, int R, int C, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
