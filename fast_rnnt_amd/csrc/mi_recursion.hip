@@ -485,7 +485,7 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kMaxSweep *kWave)
   R *my_seam = seam + (size_t)w * TP;
   const R *up_seam = seam + (size_t)prev * TP;
   R *base = tiles + (size_t)w * 8 * kTileElems;
-  const R seed = ans_grad[b];
+  const R seed = ans_grad ? ans_grad[b] : (R)1;
   int tile_base = 0;
   for (int band = 0; band * band_rows <= NS; ++band) {
     const Band g = band_of(band, w, nsweep, NS, NT);
@@ -593,7 +593,7 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kMaxSweep *kWave)
       if (!alive) return;
       if (lane == 0) publish(&cnt.consumed[w], gt + 1);
     }
-    if (row_ok && r == NS && overwrite_ans_grad) ans_grad[b] = g_origin;
+    if (row_ok && r == NS && overwrite_ans_grad && ans_grad) ans_grad[b] = g_origin;
     tile_base += g.ntiles;
   }
 }
@@ -638,7 +638,7 @@ int backward_impl(const R *px, const R *py, const int64_t *boundary, const R *p,
   (void)py;  // the d2 = 1 - d1 split needs only p and px
   if (B < 0 || S < 0 || T < 0) return fail(FRNNT_EINVAL, "mi_backward: negative size");
   if (B == 0) return FRNNT_OK;
-  if (!px || !p || !ans_grad || !px_grad || !py_grad)
+  if (!px || !p || !px_grad || !py_grad)
     return fail(FRNNT_EINVAL, "mi_backward: null pointer");
   const int n = pick_sweep_waves(S, T, sizeof(R), 4);
   const size_t lds = (size_t)n * ((size_t)(T + 1) + 8 * kTileElems) * sizeof(R);

@@ -18,24 +18,25 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from .mutual_information import mutual_information_recursion
+from .mutual_information import boundary_rows, mutual_information_recursion
 
 _RNNT_TYPES = {"regular": 0, "modified": 1, "constrained": 2}
 
 
 def validate_st_lengths(S: int, T: int, is_rnnt_type_regular: bool,
                         boundary: Optional[Tensor] = None):
-    """fast_rnnt/python/fast_rnnt/rnnt_loss.py:25-42."""
+    """fast_rnnt/python/fast_rnnt/rnnt_loss.py:25-42 (same assertions; the boundary
+    rows are looked at on the host copy shared with the recursion's own check, so a
+    loss call waits for the device at most once)."""
     if boundary is None:
         assert S >= 1, S
         assert is_rnnt_type_regular or T >= S, \
             f"Modified transducer requires T >= S, but got T={T} and S={S}"
     else:
-        Ss = boundary[:, 2]
-        Ts = boundary[:, 3]
-        assert (Ss >= 1).all(), Ss
-        assert is_rnnt_type_regular or (Ts >= Ss).all(), \
-            f"Modified transducer requires T >= S, but got T={Ts} and S={Ss}"
+        rows = boundary_rows(boundary)
+        assert all(r[2] >= 1 for r in rows), boundary[:, 2]
+        assert is_rnnt_type_regular or all(r[3] >= r[2] for r in rows), \
+            f"Modified transducer requires T >= S, but got T={boundary[:, 3]} and S={boundary[:, 2]}"
 
 
 def fix_for_boundary(px: Tensor, boundary: Optional[Tensor] = None) -> Tensor:
@@ -96,7 +97,7 @@ class _SimpleLogprobs(torch.autograd.Function):
         with torch.cuda.device(am.device):
             gpx = torch.zeros(B, S, T1, **opts) if gpx is None else gpx.contiguous()
             gpy = torch.zeros(B, S + 1, T, **opts) if gpy is None else gpy.contiguous()
-            dmat = torch.empty(B, S + 1, T, **opts)
+            dmat = torch.empty(B, S + 1, (T + 3) // 4 * 4, **opts)
             row_x = torch.empty(B, S + 1, **opts)
             row_y = torch.empty(B, S + 1, **opts)
             col_y = torch.empty(B, T, **opts)
@@ -104,7 +105,7 @@ class _SimpleLogprobs(torch.autograd.Function):
             am_grad = torch.empty_like(am) if ctx.needs_input_grad[1] else None
             _lib.call("frnnt_simple_logprobs_bwd_" + sfx, lm.data_ptr(), am.data_ptr(),
                       sym.data_ptr(), _lib.ptr(bnd), lm_max.data_ptr(), am_max.data_ptr(),
-                      norm_raw.data_ptr(), gpx.data_ptr(), gpy.data_ptr(), dmat.data_ptr(),
+                      norm_raw.data_ptr(), None, gpx.data_ptr(), gpy.data_ptr(), dmat.data_ptr(),
                       row_x.data_ptr(), row_y.data_ptr(), col_y.data_ptr(), _lib.ptr(lm_grad),
                       _lib.ptr(am_grad), B, S, T, C, term, kind, _lib.stream_of(am))
         return lm_grad, am_grad, None, None, None, None
@@ -168,6 +169,96 @@ def _recursion_and_reduce(px, py, boundary, rnnt_type, delay_penalty, reduction,
     return (loss, scores_and_grads[1]) if return_grad else loss
 
 
+class _SimpleLossScores(torch.autograd.Function):
+    """rnnt_loss_simple's whole device pipeline behind one autograd node:
+    px/py (row maxima + MFMA contraction), the lattice recursion forward, and --
+    as the recursion's autograd wrapper does (mutual_information.py:159-168) --
+    its backward with a gradient of ones, whose result both is handed out as
+    (px_grad, py_grad) and is what backward() scales in place and pushes through
+    the two gradient GEMMs.  Same arithmetic as get_rnnt_logprobs followed by
+    mutual_information_recursion; it only saves Python and launch overhead."""
+
+    @staticmethod
+    def forward(ctx, lm, am, symbols, boundary, termination_symbol, rnnt_type, delay_penalty,
+                want_grads):
+        B, T, C = am.shape
+        S = lm.shape[1] - 1
+        kind = _RNNT_TYPES[rnnt_type]
+        sfx = _lib.suffix(am.dtype)
+        lm_c, am_c = lm.contiguous(), am.contiguous()
+        sym_c = symbols.contiguous()
+        bnd_c = boundary.contiguous() if boundary is not None else None
+        opts = dict(dtype=am.dtype, device=am.device)
+        T1 = T + 1 if kind == 0 else T
+        need_grad = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        with torch.cuda.device(am.device):
+            stream = _lib.stream_of(am)
+            px = torch.empty(B, S, T1, **opts)
+            py = torch.empty(B, S + 1, T, **opts)
+            lm_max = torch.empty(B, S + 1, **opts)
+            am_max = torch.empty(B, T, **opts)
+            norm_raw = torch.empty(B, S + 1, T, **opts) if need_grad else None
+            _lib.call("frnnt_simple_logprobs_fwd_" + sfx, lm_c.data_ptr(), am_c.data_ptr(),
+                      sym_c.data_ptr(), _lib.ptr(bnd_c), px.data_ptr(), py.data_ptr(),
+                      lm_max.data_ptr(), am_max.data_ptr(), _lib.ptr(norm_raw), B, S, T, C,
+                      int(termination_symbol), kind, stream)
+            if delay_penalty > 0.0:
+                _apply_delay_penalty(px, boundary, rnnt_type, delay_penalty)
+            p = torch.empty(B, S + 1, T + 1, **opts)
+            scores = torch.empty(B, **opts)
+            modified = int(kind != 0)
+            _lib.call("frnnt_mi_forward_" + sfx, px.data_ptr(), py.data_ptr(), _lib.ptr(bnd_c),
+                      p.data_ptr(), scores.data_ptr(), B, S, T, modified, stream)
+            px_grad = py_grad = None
+            if want_grads or need_grad:
+                px_grad = torch.empty_like(px)
+                py_grad = torch.empty_like(py)
+                _lib.call("frnnt_mi_backward_" + sfx, px.data_ptr(), py.data_ptr(),
+                          _lib.ptr(bnd_c), p.data_ptr(), None, px_grad.data_ptr(),
+                          py_grad.data_ptr(), B, S, T, modified, 0, stream)
+        if need_grad:
+            ctx.save_for_backward(lm_c, am_c, sym_c, bnd_c, lm_max, am_max, norm_raw, px_grad,
+                                  py_grad)
+            ctx.meta = (B, S, T, C, int(termination_symbol), kind, sfx)
+        if px_grad is None:
+            return scores, None, None
+        ctx.mark_non_differentiable(px_grad, py_grad)
+        return scores, px_grad, py_grad
+
+    @staticmethod
+    def backward(ctx, g_scores, _gx, _gy):
+        lm, am, sym, bnd, lm_max, am_max, norm_raw, px_grad, py_grad = ctx.saved_tensors
+        B, S, T, C, term, kind, sfx = ctx.meta
+        opts = dict(dtype=am.dtype, device=am.device)
+        with torch.cuda.device(am.device):
+            g = g_scores.contiguous()
+            dmat = torch.empty(B, S + 1, (T + 3) // 4 * 4, **opts)
+            row_x = torch.empty(B, S + 1, **opts)
+            row_y = torch.empty(B, S + 1, **opts)
+            col_y = torch.empty(B, T, **opts)
+            lm_grad = torch.empty_like(lm) if ctx.needs_input_grad[0] else None
+            am_grad = torch.empty_like(am) if ctx.needs_input_grad[1] else None
+            # px_grad / py_grad are scaled in place by the scores' gradient, exactly as
+            # MutualInformationRecursionFunction.backward does to the tensors it handed out
+            _lib.call("frnnt_simple_logprobs_bwd_" + sfx, lm.data_ptr(), am.data_ptr(),
+                      sym.data_ptr(), _lib.ptr(bnd), lm_max.data_ptr(), am_max.data_ptr(),
+                      norm_raw.data_ptr(), g.data_ptr(), px_grad.data_ptr(), py_grad.data_ptr(),
+                      dmat.data_ptr(), row_x.data_ptr(), row_y.data_ptr(), col_y.data_ptr(),
+                      _lib.ptr(lm_grad), _lib.ptr(am_grad), B, S, T, C, term, kind,
+                      _lib.stream_of(am))
+        return lm_grad, am_grad, None, None, None, None, None, None
+
+
+def _reduce(negated_loss: Tensor, reduction: Optional[str]) -> Tensor:
+    if reduction == "none":
+        return -negated_loss
+    if reduction == "mean":
+        return -torch.mean(negated_loss)
+    if reduction == "sum":
+        return -torch.sum(negated_loss)
+    raise ValueError(f"reduction should be ('none' | 'mean' | 'sum'), given {reduction}")
+
+
 def rnnt_loss_simple(
     lm: Tensor, am: Tensor, symbols: Tensor, termination_symbol: int,
     boundary: Optional[Tensor] = None, rnnt_type: str = "regular",
@@ -179,11 +270,31 @@ def rnnt_loss_simple(
     ``return_grad=True``, also ``(px_grad, py_grad)``: the occupation
     probabilities of the lattice, used by :func:`get_rnnt_prune_ranges`.
     """
-    px, py = get_rnnt_logprobs(lm=lm, am=am, symbols=symbols,
-                               termination_symbol=termination_symbol,
-                               boundary=boundary, rnnt_type=rnnt_type)
-    return _recursion_and_reduce(px, py, boundary, rnnt_type, delay_penalty, reduction,
-                                 return_grad)
+    # the argument checks of get_rnnt_logprobs and mutual_information_recursion
+    assert lm.ndim == 3, lm.ndim
+    assert am.ndim == 3, am.ndim
+    assert lm.shape[0] == am.shape[0], (lm.shape[0], am.shape[0])
+    assert lm.shape[2] == am.shape[2], (lm.shape[2], am.shape[2])
+    (B, T, C) = am.shape
+    S = lm.shape[1] - 1
+    assert symbols.shape == (B, S), symbols.shape
+    validate_st_lengths(S, T, rnnt_type == "regular", boundary)
+    assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
+    assert lm.dtype == am.dtype, (lm.dtype, am.dtype)
+    _require_gpu(lm, am, symbols, boundary)
+    if boundary is not None:
+        assert boundary.dtype == torch.int64
+        assert boundary.shape == (B, 4)
+        for s_begin, t_begin, s_end, t_end in boundary_rows(boundary):
+            assert 0 <= s_begin <= s_end <= S
+            assert 0 <= t_begin <= t_end <= T
+    if reduction not in ("none", "mean", "sum"):
+        raise ValueError(f"reduction should be ('none' | 'mean' | 'sum'), given {reduction}")
+    scores, px_grad, py_grad = _SimpleLossScores.apply(
+        lm, am, symbols, boundary, termination_symbol, rnnt_type, float(delay_penalty),
+        bool(return_grad))
+    loss = _reduce(scores, reduction)
+    return (loss, (px_grad, py_grad)) if return_grad else loss
 
 
 class _LatticeLogprobs(torch.autograd.Function):

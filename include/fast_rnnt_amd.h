@@ -67,7 +67,8 @@ int frnnt_mi_forward_f64(const double *px, const double *py, const int64_t *boun
  *     (fast_rnnt/csrc/mutual_information.h:136-143,
  *      fast_rnnt/csrc/mutual_information_cpu.cu:128-256).
  *   p        [B][S+1][T+1]   in: the table frnnt_mi_forward_* produced
- *   ans_grad [B]             in; if overwrite_ans_grad != 0 it is overwritten
+ *   ans_grad [B]             in, or NULL for a gradient of 1 on every row (then
+ *                            nothing is written back); if overwrite_ans_grad != 0 it is overwritten
  *                            with the gradient that reaches (s_begin, t_begin),
  *                            which equals the input when the sweep is consistent
  *                            (mutual_information_cuda.cu:667-669)
@@ -113,22 +114,27 @@ int frnnt_simple_logprobs_fwd_f64(const double *lm, const double *am, const int6
  * Backward of the above: what autograd derives for rnnt_loss.py:174-225, as one
  * elementwise pass plus two MFMA GEMMs.
  *   px_grad, py_grad: dL/dpx, dL/dpy (shapes of px, py)                    in
- *   dmat [B][S+1][T], row_x [B][S+1], row_y [B][S+1], col_y [B][T]         scratch
+ *   score_grad [B] or NULL: when given, px_grad[b] and py_grad[b] are first multiplied
+ *     IN PLACE by score_grad[b] -- the scaling step of the recursion's autograd
+ *     backward (mutual_information.py:173-181), for callers that hold the occupation
+ *     gradients and the gradient of the scores separately
+ *   dmat [B][S+1][T rounded up to a multiple of 4], row_x [B][S+1], row_y [B][S+1],
+ *   col_y [B][T]                                                           scratch
  *   lm_grad [B][S+1][C], am_grad [B][T][C]: out; either may be NULL to skip it
  */
 int frnnt_simple_logprobs_bwd_f32(const float *lm, const float *am, const int64_t *symbols,
                                   const int64_t *boundary, const float *lm_max,
-                                  const float *am_max, const float *norm_raw, const float *px_grad,
-                                  const float *py_grad, float *dmat, float *row_x, float *row_y,
-                                  float *col_y, float *lm_grad, float *am_grad, int B, int S,
-                                  int T, int C, int termination_symbol, int rnnt_type,
-                                  void *stream);
+                                  const float *am_max, const float *norm_raw,
+                                  const float *score_grad, float *px_grad, float *py_grad,
+                                  float *dmat, float *row_x, float *row_y, float *col_y,
+                                  float *lm_grad, float *am_grad, int B, int S, int T, int C,
+                                  int termination_symbol, int rnnt_type, void *stream);
 int frnnt_simple_logprobs_bwd_f64(const double *lm, const double *am, const int64_t *symbols,
                                   const int64_t *boundary, const double *lm_max,
                                   const double *am_max, const double *norm_raw,
-                                  const double *px_grad, const double *py_grad, double *dmat,
-                                  double *row_x, double *row_y, double *col_y, double *lm_grad,
-                                  double *am_grad, int B, int S, int T, int C,
+                                  const double *score_grad, double *px_grad, double *py_grad,
+                                  double *dmat, double *row_x, double *row_y, double *col_y,
+                                  double *lm_grad, double *am_grad, int B, int S, int T, int C,
                                   int termination_symbol, int rnnt_type, void *stream);
 
 /*
