@@ -123,19 +123,31 @@ def main():
             args.kernel_reps)
     stages = {"mi_forward_ms": t_fwd, "mi_backward_ms": t_bwd, "logprobs_fwd_ms": t_logp}
 
-    fwd_bytes = _recursion_bytes(w.boundary, S, T, B, backward=False)
-    achieved = fwd_bytes / (t_fwd * 1e-3) / 1e9
-    roofline = {
-        "kernel": "mi_forward_kernel<float,false,256>",
-        "bound": "hbm",
-        "achieved": round(achieved, 2),
-        "peak": HBM_PEAK_GBS,
-        "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 5),
-        "traffic": None,
-        "algorithmic_bytes": fwd_bytes,
-        "avg_launch_us": round(1e3 * t_fwd, 2),
-    }
+    def hbm_line(kernel, nbytes, t_ms):
+        achieved = nbytes / (t_ms * 1e-3) / 1e9
+        return {"kernel": kernel, "bound": "hbm", "achieved": round(achieved, 2),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5),
+                "traffic": None, "algorithmic_bytes": nbytes, "avg_launch_us": round(1e3 * t_ms, 2)}
+
+    lines = [
+        hbm_line("mi_forward_kernel<float, false, 2>",
+                 _recursion_bytes(w.boundary, S, T, B, backward=False), t_fwd),
+        hbm_line("mi_backward_kernel<float, false, 2>",
+                 _recursion_bytes(w.boundary, S, T, B, backward=True), t_bwd),
+    ]
+    # the dominant kernel of the step is the slower of the two recursion sweeps
+    lines.sort(key=lambda r: -r["avg_launch_us"])
+    roofline = lines[0]
+    # normalizer contraction exp(lm - max) . exp(am - max)^T on the fp32 matrix cores;
+    # its entry point also runs the row-max and the px/py assembly kernels, so this
+    # figure is a lower bound on the GEMM kernel's own rate
+    gemm_flops = 2.0 * B * (S + 1) * T * w.C
+    gemm_tflops = gemm_flops / (t_logp * 1e-3) / 1e12
+    other = lines[1:] + [{
+        "kernel": "simple_fwd_direct_kernel<true> (whole frnnt_simple_logprobs_fwd call)",
+        "bound": "mfma", "achieved": round(gemm_tflops, 3), "peak": FP32_MFMA_PEAK_TFLOPS,
+        "unit": "TFLOP/s", "frac": round(gemm_tflops / FP32_MFMA_PEAK_TFLOPS, 5), "traffic": None,
+        "algorithmic_flops": gemm_flops, "avg_launch_us": round(1e3 * t_logp, 2)}]
 
     # ---- CPU baseline: the oracle restatement of the reference path ------------------
     cpu = None
@@ -192,6 +204,7 @@ def main():
                                f"C={w.C}, ragged boundary, reduction=sum, return_grad=True",
                    "call_bytes": workloads.simple_call_bytes(w)},
         "roofline": roofline,
+        "roofline_other_kernels": other,
         "cpu_baseline": cpu,
         "stages": {k: round(v, 4) for k, v in stages.items()},
         "whole_call_hbm_GBs": round(workloads.simple_call_bytes(w) / elapsed * args.steps / 1e9, 2),

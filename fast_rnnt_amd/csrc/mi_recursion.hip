@@ -34,7 +34,6 @@ constexpr int kTileSteps = 32;         // steps per staged tile
 constexpr int kTilePitch = kTileSteps + 1;
 constexpr int kTileElems = kWave * kTilePitch;
 constexpr int kFwdStagers = 2;         // staging waves per sweep wave
-constexpr int kStageBatch = 8;         // rows a staging lane fetches before it writes LDS
 constexpr int kBwdStagers = 3;
 constexpr int kSpinLimit = 1 << 22;
 
@@ -86,6 +85,22 @@ __device__ __forceinline__ float chain_log_add(float a, float c) {
 }
 __device__ __forceinline__ double chain_log_add(double a, double c) { return log_add(a, c); }
 
+// Four consecutive elements with one 16-byte store; the address only needs element
+// alignment (global memory accepts unaligned vector stores).
+template <typename R>
+struct Vec4 {
+  typedef R type __attribute__((ext_vector_type(4), aligned(sizeof(R))));
+};
+template <typename R>
+__device__ __forceinline__ void store4(R *dst, R a, R b, R c, R d) {
+  typename Vec4<R>::type v;
+  v[0] = a;
+  v[1] = b;
+  v[2] = c;
+  v[3] = d;
+  *reinterpret_cast<typename Vec4<R>::type *>(dst) = v;
+}
+
 struct Counters {
   int ready[kMaxSweep];                   // seam columns published by sweep wave w
   int consumed[kMaxSweep];                // tiles sweep wave w has finished
@@ -110,8 +125,9 @@ __device__ __forceinline__ Band band_of(int band, int w, int nsweep, int NS, int
 // Staged per step and row: x = px feeding the cell from the row below,
 // y = py feeding it from the left; -inf where that edge does not exist, and
 // y = 0 at the origin cell so that the chain produces p = 0 there.
-template <typename R, bool kModified>
-__global__ void __launch_bounds__((1 + kFwdStagers) * kMaxSweep *kWave)
+// kSweepCap: most sweep waves the launch may use; it only sets the register budget.
+template <typename R, bool kModified, int kSweepCap>
+__global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
     mi_forward_kernel(const R *__restrict__ px, const R *__restrict__ py,
                       const int64_t *__restrict__ boundary, R *__restrict__ p,
                       R *__restrict__ ans, int S, int T) {
@@ -150,43 +166,52 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kMaxSweep *kWave)
     R *xt = tiles + (size_t)w * 4 * kTileElems;
     R *yt = xt + 2 * kTileElems;
     const int half = lane >> 5, q = lane & 31;
+    // rows of a tile this wave stages: r(u) = 2*l + half + 2*kFwdStagers*u
+    constexpr int kRows = (kWave + 2 * kFwdStagers - 1) / (2 * kFwdStagers);
+    struct Staged {
+      R x[kRows], y[kRows];
+    };
+    // Global fetches of a tile go to registers and do not need the LDS buffer, so
+    // the fetch of tile m+1 is issued before this wave waits for the buffer of tile
+    // m to be released: the memory latency overlaps the sweep.
+    auto fetch = [&](Staged &in, const Band &g, int m) {
+#pragma unroll
+      for (int u = 0; u < kRows; ++u) {
+        const int r = 2 * l + half + 2 * kFwdStagers * u;
+        const int i = g.row0 + r, s = win.s0 + i;
+        const int j = m * kTileSteps + q - r;
+        const int jj = j - shift;
+        R x = ninf, y = ninf;
+        if (r < g.nrows) {
+          if (i >= 1 && jj >= 0 && j <= NT) x = pxb[(long)(s - 1) * T1 + win.t0 + jj];
+          if (j >= 1 && j <= NT) y = pyb[(long)s * T + win.t0 + j - 1];
+          if (i == 0 && j == 0) y = 0;
+        }
+        in.x[u] = x;
+        in.y[u] = y;
+      }
+    };
     int tile_base = 0;
     for (int band = 0; band * band_rows <= NS; ++band) {
       const Band g = band_of(band, w, nsweep, NS, NT);
       if (g.row0 > NS) break;
+      Staged cur, nxt;
+      fetch(cur, g, 0);
       for (int m = 0; m < g.ntiles; ++m) {
         const int gt = tile_base + m;
+        if (m + 1 < g.ntiles) fetch(nxt, g, m + 1);
         if (gt >= 2 && !wait_for(&cnt.consumed[w], gt - 1)) return;
         R *xdst = xt + (gt & 1) * kTileElems, *ydst = yt + (gt & 1) * kTileElems;
-        // all row fetches of a batch are issued before the first LDS write, so one
-        // memory latency covers the whole batch
-        for (int rb = 2 * l + half; rb < g.nrows; rb += 2 * kFwdStagers * kStageBatch) {
-          R xv[kStageBatch], yv[kStageBatch];
 #pragma unroll
-          for (int u = 0; u < kStageBatch; ++u) {
-            const int r = rb + 2 * kFwdStagers * u;
-            const int i = g.row0 + r, s = win.s0 + i;
-            const int j = m * kTileSteps + q - r;
-            const int jj = j - shift;
-            R x = ninf, y = ninf;
-            if (r < g.nrows) {
-              if (i >= 1 && jj >= 0 && j <= NT) x = pxb[(long)(s - 1) * T1 + win.t0 + jj];
-              if (j >= 1 && j <= NT) y = pyb[(long)s * T + win.t0 + j - 1];
-              if (i == 0 && j == 0) y = 0;
-            }
-            xv[u] = x;
-            yv[u] = y;
-          }
-#pragma unroll
-          for (int u = 0; u < kStageBatch; ++u) {
-            const int r = rb + 2 * kFwdStagers * u;
-            if (r < g.nrows) {
-              xdst[r * kTilePitch + q] = xv[u];
-              ydst[r * kTilePitch + q] = yv[u];
-            }
+        for (int u = 0; u < kRows; ++u) {
+          const int r = 2 * l + half + 2 * kFwdStagers * u;
+          if (r < g.nrows) {
+            xdst[r * kTilePitch + q] = cur.x[u];
+            ydst[r * kTilePitch + q] = cur.y[u];
           }
         }
         if (lane == 0) publish(&cnt.loaded[w * kFwdStagers + l], gt + 1);
+        cur = nxt;
       }
       tile_base += g.ntiles;
     }
@@ -254,6 +279,7 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kMaxSweep *kWave)
         }
         R *pp = p_row + (e0 - lane);
         R *sp = my_seam + (e0 - (kWave - 1));
+        R vals[kChunk];
 #pragma unroll
         for (int k = 0; k < kChunk; ++k) {
           const int kk = c4 * kChunk + k;
@@ -265,18 +291,31 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kMaxSweep *kWave)
             up = (lane == 0) ? first : up;
           }
           const R v = chain_log_add(up + xq[kk], own + yq[kk]);
+          vals[k] = v;
           const int j63 = e0 + k - (kWave - 1);  // column of the seam lane, wave-uniform
           if (kEdge) {
             const int j = e0 + k - lane;
-            if (row_ok && (unsigned)j <= (unsigned)NT) pp[k] = v;
             fin = (j == NT) ? v : fin;
             if (kDown && j63 >= 0 && j63 <= NT && lane == kWave - 1) sp[k] = v;
           } else {
-            pp[k] = v;
             if (kDown && lane == kWave - 1) sp[k] = v;
           }
           own2 = own;
           own = v;
+        }
+        // p goes out in groups of four columns: one 16-byte store when the whole
+        // group lies inside the window, single stores otherwise
+#pragma unroll
+        for (int q4 = 0; q4 < kChunk; q4 += 4) {
+          const int j0 = e0 + q4 - lane;
+          const bool whole = !kEdge || (j0 >= 0 && j0 + 3 <= NT);
+          if (whole && row_ok) {
+            store4(pp + q4, vals[q4], vals[q4 + 1], vals[q4 + 2], vals[q4 + 3]);
+          } else if (row_ok) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+              if ((unsigned)(j0 + k) <= (unsigned)NT) pp[q4 + k] = vals[q4 + k];
+          }
         }
         if (kDown && lane == kWave - 1) {
           const int done = max(0, min(e0 + kChunk - (kWave - 1), cols));
@@ -322,9 +361,10 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kMaxSweep *kWave)
 // down plus what its right neighbour hands left; it is then split into a d1
 // share for the cell below and a d2 share for the cell to the left.  The staging
 // waves evaluate d1 / d2 (mutual_information_cpu.cu:196-212 and the two edge
-// loops :219-235) and later write the px / py gradient tiles the sweep produced.
-template <typename R, bool kModified>
-__global__ void __launch_bounds__((1 + kBwdStagers) * kMaxSweep *kWave)
+// loops :219-235); the sweep wave keeps four steps of px / py gradients in
+// registers and writes them with one 16-byte store per array.
+template <typename R, bool kModified, int kSweepCap>
+__global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
     mi_backward_kernel(const R *__restrict__ px, const int64_t *__restrict__ boundary,
                        const R *__restrict__ p, R *ans_grad, R *__restrict__ px_grad,
                        R *__restrict__ py_grad, int S, int T, int overwrite_ans_grad) {
@@ -333,6 +373,7 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kMaxSweep *kWave)
 
   const int b = blockIdx.x;
   const int nsweep = blockDim.x / (kWave * (1 + kBwdStagers));
+  const int nwaves = blockDim.x / kWave;
   const int wave = threadIdx.x / kWave;
   const int lane = threadIdx.x % kWave;
   const int T1 = kModified ? T : T + 1;
@@ -343,19 +384,19 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kMaxSweep *kWave)
   R *gxb = px_grad + (size_t)b * S * T1;
   R *gyb = py_grad + (size_t)b * (S + 1) * T;
 
-  // exact zeros everywhere the sweep does not write
+  // exact zeros everywhere the sweep does not write: one wave per row
   if (boundary) {
     const int s_lo = win.s0, s_hi = win.s0 + win.ns;
     const int t_lo = win.t0, t_hi = win.t0 + win.nt;
-    for (int idx = threadIdx.x; idx < S * T1; idx += blockDim.x) {
-      const int s = idx / T1, t = idx - s * T1;
-      const bool inside = win.ok && s >= s_lo && s < s_hi && t >= t_lo && t <= t_hi - shift;
-      if (!inside) gxb[idx] = 0;
-    }
-    for (int idx = threadIdx.x; idx < (S + 1) * T; idx += blockDim.x) {
-      const int s = idx / T, t = idx - s * T;
-      const bool inside = win.ok && s >= s_lo && s <= s_hi && t >= t_lo && t < t_hi;
-      if (!inside) gyb[idx] = 0;
+    for (int s = wave; s <= S; s += nwaves) {
+      if (s < S) {
+        const bool row_in = win.ok && s >= s_lo && s < s_hi;
+        for (int t = lane; t < T1; t += kWave)
+          if (!(row_in && t >= t_lo && t <= t_hi - shift)) gxb[(long)s * T1 + t] = 0;
+      }
+      const bool row_in = win.ok && s >= s_lo && s <= s_hi;
+      for (int t = lane; t < T; t += kWave)
+        if (!(row_in && t >= t_lo && t < t_hi)) gyb[(long)s * T + t] = 0;
     }
   }
   if (!win.ok) return;
@@ -367,67 +408,86 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kMaxSweep *kWave)
   const R *pxb = px + (size_t)b * S * T1;
   const R *pb = p + (size_t)b * (S + 1) * TP;
   R *seam = reinterpret_cast<R *>(dyn_lds);
-  // per sweep wave: d1[2], d2[2], gx[2], gy[2] tiles
-  R *tiles = seam + (size_t)nsweep * TP;
+  R *tiles = seam + (size_t)nsweep * TP;  // per sweep wave: d1[2], d2[2] tiles
   const int band_rows = kWave * nsweep;
 
   if (wave >= nsweep) {
     // ------------------------------ staging wave -------------------------------
     const int w = (wave - nsweep) / kBwdStagers, l = (wave - nsweep) % kBwdStagers;
-    R *base = tiles + (size_t)w * 8 * kTileElems;
+    R *base = tiles + (size_t)w * 4 * kTileElems;
     const int half = lane >> 5, q = lane & 31;
     int *my_loaded = &cnt.loaded[w * kBwdStagers + l];
-
-    // writes the gradient tile `m` of band geometry g (global tile index gt)
-    auto flush = [&](const Band &g, int m, int gt) {
-      const R *gxs = base + (4 + (gt & 1)) * kTileElems, *gys = base + (6 + (gt & 1)) * kTileElems;
-      for (int r = 2 * l + half; r < g.nrows; r += 2 * kBwdStagers) {
-        const int i = NS - (g.row0 + r), s = win.s0 + i;
-        const int c = m * kTileSteps + q - r;
-        const int j = NT - c;
-        if (c < 0 || c > NT) continue;
-        if (i > 0 && (j > 0 || !kModified))
-          gxb[(long)(s - 1) * T1 + win.t0 + j - shift] = gxs[r * kTilePitch + q];
-        if (j > 0) gyb[(long)s * T + win.t0 + j - 1] = gys[r * kTilePitch + q];
+    // rows of a tile this wave stages: r(u) = 2*l + half + 2*kBwdStagers*u
+    constexpr int kRows = (kWave + 2 * kBwdStagers - 1) / (2 * kBwdStagers);
+    struct Staged {
+      R here[kRows], below[kRows], x[kRows];
+    };
+    // global fetches of tile m+1 are issued (into registers) before this wave waits
+    // for the LDS buffers of tile m, so their latency overlaps the sweep
+    auto fetch = [&](Staged &in, const Band &g, int m) {
+      const bool inner_tile = g.nrows == kWave && g.row0 + kWave - 1 < NS &&
+                              m * kTileSteps - (kWave - 1) >= 0 &&
+                              m * kTileSteps + kTileSteps - 1 <= NT - 1;
+      // element offsets of row u = 0; each further u is 2*kBwdStagers rows up the
+      // reversed lattice, i.e. that many rows down in memory and as many columns right
+      const int r_first = 2 * l + half;
+      const int s_first = win.s0 + NS - (g.row0 + r_first);
+      const int j_first = NT - (m * kTileSteps + q - r_first);
+      const int below0 = (s_first - 1) * TP + win.t0 + j_first - shift;
+      const int x0 = (s_first - 1) * T1 + win.t0 + j_first - shift;
+      const int here0 = s_first * TP + win.t0 + j_first;
+      constexpr int kStep = 2 * kBwdStagers;
+#pragma unroll
+      for (int u = 0; u < kRows; ++u) {
+        const int r = r_first + kStep * u;
+        bool ok = r < g.nrows;
+        if (!inner_tile) {
+          const int i = NS - (g.row0 + r);
+          const int c = m * kTileSteps + q - r;
+          ok = ok && c >= 0 && c <= NT && i > 0 && NT - c > 0;
+        }
+        in.here[u] = in.below[u] = in.x[u] = 0;
+        if (ok) {
+          in.below[u] = pb[below0 - u * kStep * (TP - 1)];
+          in.x[u] = pxb[x0 - u * kStep * (T1 - 1)];
+          in.here[u] = pb[here0 - u * kStep * (TP - 1)];
+        }
       }
     };
-
     int tile_base = 0;
     for (int band = 0; band * band_rows <= NS; ++band) {
       const Band g = band_of(band, w, nsweep, NS, NT);
       if (g.row0 > NS) break;
+      Staged cur, nxt;
+      fetch(cur, g, 0);
       for (int m = 0; m < g.ntiles; ++m) {
         const int gt = tile_base + m;
-        if (gt >= 2) {
-          if (!wait_for(&cnt.consumed[w], gt - 1)) return;
-          // tile gt-2 is finished: write its gradients out before its buffers are reused.
-          // It belongs to this band (m >= 2) or to the tail of the previous one.
-          if (m >= 2) {
-            flush(g, m - 2, gt - 2);
-          } else {
-            const Band pg = band_of(band - 1, w, nsweep, NS, NT);
-            flush(pg, pg.ntiles - 2 + m, gt - 2);
-          }
-        }
+        if (m + 1 < g.ntiles) fetch(nxt, g, m + 1);
+        if (gt >= 2 && !wait_for(&cnt.consumed[w], gt - 1)) return;
         R *d1dst = base + (gt & 1) * kTileElems, *d2dst = base + (2 + (gt & 1)) * kTileElems;
-        for (int rb = 2 * l + half; rb < g.nrows; rb += 2 * kBwdStagers * kStageBatch) {
-          R here[kStageBatch], below[kStageBatch], xv[kStageBatch];
+        // A tile of a full wave whose 64 x 32 cells all lie strictly inside the window
+        // (below the top row, right of column 0) needs none of the edge cases.
+        const bool inner_tile = g.nrows == kWave && g.row0 + kWave - 1 < NS &&
+                                m * kTileSteps - (kWave - 1) >= 0 &&
+                                m * kTileSteps + kTileSteps - 1 <= NT - 1;
+        if (inner_tile) {
 #pragma unroll
-          for (int u = 0; u < kStageBatch; ++u) {
-            const int r = rb + 2 * kBwdStagers * u;
-            const int i = NS - (g.row0 + r), s = win.s0 + i;
-            const int c = m * kTileSteps + q - r;
-            const int j = NT - c;
-            here[u] = below[u] = xv[u] = 0;
-            if (r < g.nrows && c >= 0 && c <= NT && i > 0 && j > 0) {
-              below[u] = pb[(long)(s - 1) * TP + win.t0 + j - shift];
-              xv[u] = pxb[(long)(s - 1) * T1 + win.t0 + j - shift];
-              here[u] = pb[(long)s * TP + win.t0 + j];
-            }
+          for (int u = 0; u < kRows; ++u) {
+            const int r = 2 * l + half + 2 * kBwdStagers * u;
+            if (r >= kWave) continue;
+            const R term1 = cur.below[u] + cur.x[u];
+            R total = cur.here[u];
+            if (total - total != 0) total = 0;
+            R d1 = Num<R>::exp_(term1 - total);
+            R d2 = (R)1 - d1;
+            if (d1 - d1 != 0) d1 = d2 = 0;
+            d1dst[r * kTilePitch + q] = d1;
+            d2dst[r * kTilePitch + q] = d2;
           }
+        } else {
 #pragma unroll
-          for (int u = 0; u < kStageBatch; ++u) {
-            const int r = rb + 2 * kBwdStagers * u;
+          for (int u = 0; u < kRows; ++u) {
+            const int r = 2 * l + half + 2 * kBwdStagers * u;
             const int i = NS - (g.row0 + r);
             const int c = m * kTileSteps + q - r;
             const int j = NT - c;
@@ -435,8 +495,8 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kMaxSweep *kWave)
             R d1 = 0, d2 = 0;
             if (c >= 0 && c <= NT) {
               if (i > 0 && j > 0) {
-                const R term1 = below[u] + xv[u];
-                R total = here[u];
+                const R term1 = cur.below[u] + cur.x[u];
+                R total = cur.here[u];
                 if (total - total != 0) total = 0;
                 d1 = Num<R>::exp_(term1 - total);
                 d2 = (R)1 - d1;
@@ -453,28 +513,9 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kMaxSweep *kWave)
         }
         // every lane's LDS writes precede the release by lane 0 of the same wave
         if (lane == 0) publish(my_loaded, gt + 1);
+        cur = nxt;
       }
       tile_base += g.ntiles;
-    }
-    // the last two tiles: flush them once the sweep wave is done with them
-    {
-      int bands_done = 0;
-      while (bands_done * band_rows <= NS &&
-             band_of(bands_done, w, nsweep, NS, NT).row0 <= NS)
-        ++bands_done;
-      if (bands_done == 0) return;
-      const Band g = band_of(bands_done - 1, w, nsweep, NS, NT);
-      for (int back = min(2, tile_base); back >= 1; --back) {
-        const int gt = tile_base - back;
-        if (!wait_for(&cnt.consumed[w], gt + 1)) return;
-        const int m = g.ntiles - back;
-        if (m >= 0) {
-          flush(g, m, gt);
-        } else {
-          const Band pg = band_of(bands_done - 2, w, nsweep, NS, NT);
-          flush(pg, pg.ntiles + m, gt);
-        }
-      }
     }
     return;
   }
@@ -484,17 +525,22 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kMaxSweep *kWave)
   const int prev = (w + nsweep - 1) % nsweep;
   R *my_seam = seam + (size_t)w * TP;
   const R *up_seam = seam + (size_t)prev * TP;
-  R *base = tiles + (size_t)w * 8 * kTileElems;
+  const R *base = tiles + (size_t)w * 4 * kTileElems;
   const R seed = ans_grad ? ans_grad[b] : (R)1;
   int tile_base = 0;
   for (int band = 0; band * band_rows <= NS; ++band) {
     const Band g = band_of(band, w, nsweep, NS, NT);
     if (g.row0 > NS) break;
     const int r = g.row0 + lane;
+    const int i = NS - r;
     const bool row_ok = r <= NS;
     const bool has_up = g.row0 > 0;
     const int up_base = (w > 0 ? band : band - 1) * cols;
     const int my_base = band * cols;
+    // gx of cell (i, j) goes to px_grad[s-1][t0 + j - shift], gy to py_grad[s][t0 + j - 1]
+    R *gx_row = gxb + (long)(win.s0 + i - 1) * T1 + win.t0 - shift;
+    R *gy_row = gyb + (long)(win.s0 + i) * T + win.t0 - 1;
+    const bool gx_ok = row_ok && i > 0;
 
     // the seed enters as "handed left" into the first cell of the reversed sweep
     R to_below = 0, to_below2 = 0, to_left = (r == 0) ? seed : (R)0;
@@ -515,8 +561,7 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kMaxSweep *kWave)
           d2q[kk] = d2s[kk];
         }
       }
-      R *gxs = base + (4 + (gt & 1)) * kTileElems + lane * kTilePitch;
-      R *gys = base + (6 + (gt & 1)) * kTileElems + lane * kTilePitch;
+      if (lane == 0) publish(&cnt.consumed[w], gt + 1);
 
       bool alive = true;
       auto chunk = [&](auto up_c, auto down_c, auto edge_c, int c4, int e0)
@@ -535,6 +580,7 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kMaxSweep *kWave)
           if (lane < kChunk && col >= 0 && col <= NT) handed = up_seam[col];
         }
         R *sp = my_seam + (e0 - (kWave - 1));
+        R down[kChunk], left[kChunk];
 #pragma unroll
         for (int k = 0; k < kChunk; ++k) {
           const int kk = c4 * kChunk + k;
@@ -545,21 +591,45 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kMaxSweep *kWave)
           }
           // cells outside the window carry d1 = d2 = 0, so nothing leaks in or out
           const R gcell = from_above + to_left;
-          const R down = d1q[kk] * gcell;
-          const R left = d2q[kk] * gcell;
-          gxs[kk] = down;
-          gys[kk] = left;
+          down[k] = d1q[kk] * gcell;
+          left[k] = d2q[kk] * gcell;
           const int c63 = e0 + k - (kWave - 1);  // reversed column of the seam lane
           if (kEdge) {
             const int c = e0 + k - lane;
             g_origin = (c == NT) ? gcell : g_origin;
-            if (kDown && c63 >= 0 && c63 <= NT && lane == kWave - 1) sp[k] = down;
+            if (kDown && c63 >= 0 && c63 <= NT && lane == kWave - 1) sp[k] = down[k];
           } else {
-            if (kDown && lane == kWave - 1) sp[k] = down;
+            if (kDown && lane == kWave - 1) sp[k] = down[k];
           }
           to_below2 = to_below;
-          to_below = down;
-          to_left = left;
+          to_below = down[k];
+          to_left = left[k];
+        }
+        // write-out in groups of four steps: columns j0-3 .. j0, one 16-byte store per
+        // array when the whole group lies inside the window, single stores otherwise
+#pragma unroll
+        for (int q4 = 0; q4 < kChunk; q4 += 4) {
+          const int c0 = e0 + q4 - lane;     // reversed column of the group's first step
+          const int j0 = NT - c0;            // its column; the group covers j0-3 .. j0
+          const bool whole = !kEdge || (c0 >= 0 && j0 - 3 >= 1);
+          if (whole && gx_ok) {
+            store4(gx_row + (j0 - 3), down[q4 + 3], down[q4 + 2], down[q4 + 1], down[q4]);
+          } else if (gx_ok) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const int j = j0 - k;
+              if (c0 + k >= 0 && j >= 0 && (j > 0 || !kModified)) gx_row[j] = down[q4 + k];
+            }
+          }
+          if (whole && row_ok) {
+            store4(gy_row + (j0 - 3), left[q4 + 3], left[q4 + 2], left[q4 + 1], left[q4]);
+          } else if (row_ok) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const int j = j0 - k;
+              if (c0 + k >= 0 && j > 0) gy_row[j] = left[q4 + k];
+            }
+          }
         }
         if (kDown && lane == kWave - 1) {
           const int done = max(0, min(e0 + kChunk - (kWave - 1), cols));
@@ -571,7 +641,10 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kMaxSweep *kWave)
         for (int c4 = 0; c4 < kTileSteps / kChunk; ++c4) {
           const int e0 = m * kTileSteps + c4 * kChunk;
           if (e0 < g.nsteps && alive) {
-            const bool interior = e0 >= kWave - 1 && e0 + kChunk <= NT;
+            // interior: every lane of a full wave is inside the window, below the
+            // top row and right of column 0 for all of the chunk's steps
+            const bool interior = g.nrows == kWave && g.row0 + kWave - 1 < NS &&
+                                  e0 >= kWave - 1 && e0 + kChunk <= NT;
             if (interior)
               chunk(up_c, down_c, std::false_type{}, c4, e0);
             else
@@ -591,7 +664,6 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kMaxSweep *kWave)
           tile(std::false_type{}, std::false_type{});
       }
       if (!alive) return;
-      if (lane == 0) publish(&cnt.consumed[w], gt + 1);
     }
     if (row_ok && r == NS && overwrite_ans_grad && ans_grad) ans_grad[b] = g_origin;
     tile_base += g.ntiles;
@@ -621,7 +693,9 @@ int forward_impl(const R *px, const R *py, const int64_t *boundary, R *p, R *ans
   const size_t lds = (size_t)n * ((size_t)(T + 1) + 4 * kTileElems) * sizeof(R);
   if (lds > kLdsBudget)
     return fail(FRNNT_ELIMIT, "mi_forward: T=%d needs %zu bytes of LDS", T, lds);
-  auto kernel = modified ? mi_forward_kernel<R, true> : mi_forward_kernel<R, false>;
+  auto kernel = n <= 2 ? (modified ? mi_forward_kernel<R, true, 2> : mi_forward_kernel<R, false, 2>)
+                       : (modified ? mi_forward_kernel<R, true, kMaxSweep>
+                                   : mi_forward_kernel<R, false, kMaxSweep>);
   if (lds > 64 * 1024 &&
       hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -640,11 +714,13 @@ int backward_impl(const R *px, const R *py, const int64_t *boundary, const R *p,
   if (B == 0) return FRNNT_OK;
   if (!px || !p || !px_grad || !py_grad)
     return fail(FRNNT_EINVAL, "mi_backward: null pointer");
-  const int n = pick_sweep_waves(S, T, sizeof(R), 4);
-  const size_t lds = (size_t)n * ((size_t)(T + 1) + 8 * kTileElems) * sizeof(R);
+  const int n = pick_sweep_waves(S, T, sizeof(R), 2);
+  const size_t lds = (size_t)n * ((size_t)(T + 1) + 4 * kTileElems) * sizeof(R);
   if (lds > kLdsBudget)
     return fail(FRNNT_ELIMIT, "mi_backward: T=%d needs %zu bytes of LDS", T, lds);
-  auto kernel = modified ? mi_backward_kernel<R, true> : mi_backward_kernel<R, false>;
+  auto kernel = n <= 2 ? (modified ? mi_backward_kernel<R, true, 2> : mi_backward_kernel<R, false, 2>)
+                       : (modified ? mi_backward_kernel<R, true, kMaxSweep>
+                                   : mi_backward_kernel<R, false, kMaxSweep>);
   if (lds > 64 * 1024 &&
       hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
