@@ -242,17 +242,46 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-// px_grad[b,:,:] *= score_grad[b], py_grad[b,:,:] *= score_grad[b], in place.
+// px_grad[b,:,:] *= g_b, py_grad[b,:,:] *= g_b in place, with
+// g_b = scale * score_grad[b * stride].  blockIdx.y is the utterance; a workgroup
+// takes 1024 consecutive elements of its px_grad part or of its py_grad part.
 template <typename R>
 __global__ void __launch_bounds__(256)
     scale_by_batch_kernel(R *__restrict__ gpx, R *__restrict__ gpy,
-                          const R *__restrict__ score_grad, long per_x, long per_y, int B) {
-  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
-  const long nx = per_x * B, ny = per_y * B;
-  if (idx < nx)
-    gpx[idx] *= score_grad[idx / per_x];
-  else if (idx < nx + ny)
-    gpy[idx - nx] *= score_grad[(idx - nx) / per_y];
+                          const R *__restrict__ score_grad, int stride, R scale, int per_x,
+                          int per_y, int x_blocks) {
+  const int b = blockIdx.y;
+  const R g = scale * score_grad[(long)b * stride];
+  const bool is_x = (int)blockIdx.x < x_blocks;
+  R *base = is_x ? gpx + (long)b * per_x : gpy + (long)b * per_y;
+  const int n = is_x ? per_x : per_y;
+  const int first = (is_x ? blockIdx.x : blockIdx.x - x_blocks) * 1024 + threadIdx.x;
+  R v[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) v[u] = (first + 256 * u < n) ? base[first + 256 * u] : (R)0;
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+    if (first + 256 * u < n) base[first + 256 * u] = v[u] * g;
+}
+
+// loss = -scores, -mean(scores) or -sum(scores); one wave: every lane sums a
+// contiguous slice, then a fixed butterfly over the lanes
+template <typename R>
+__global__ void __launch_bounds__(kWave)
+    loss_reduce_kernel(const R *__restrict__ scores, R *__restrict__ loss, int B, int reduction) {
+  const int lane = threadIdx.x;
+  if (reduction == 0) {
+    for (int b = lane; b < B; b += kWave) loss[b] = -scores[b];
+    return;
+  }
+  const int per = (B + kWave - 1) / kWave;
+  R acc = 0;
+  for (int k = 0; k < per; ++k) {
+    const int b = lane * per + k;
+    if (b < B) acc += scores[b];
+  }
+  acc = wave_sum(acc);
+  if (lane == 0) loss[0] = reduction == 1 ? -(acc / (R)B) : -acc;
 }
 
 // lm gradient: grid = (ceil(C/64), ceil((S+1)/64), B); K runs over frames.
@@ -609,6 +638,201 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// am gradient, LDS-panel form.  k runs over the S+1 lattice rows, which is short, so
+// a workgroup brings ALL of k for its 64 (frames) x 64 (vocabulary) tile into LDS:
+// D[k][t], gx[k][t] and exp(lm[k][c] - max[k]) are all contiguous along the output
+// dimension, so the panels arrive as coalesced 16-byte loads, and the matrix cores
+// read their operands from LDS only.  What bounds this kernel is the number of
+// vector-memory INSTRUCTIONS a compute unit can retire (an instruction costs about
+// the same whether it moves 4 or 16 bytes per lane), so every global access here is
+// 16 bytes wide and row-contiguous: the am tile comes in that way too, and the
+// result leaves through an LDS transpose as whole 256-byte row segments.
+// Every global load is in flight before the first one is consumed: a workgroup pays
+// one memory round trip.
+// The per-symbol term  sum_s [c = sym[b,s]] gx[b,s,t]  is a second product on the
+// matrix core, gx^T times a one-hot matrix made in registers from the symbols: it is
+// exact (products by 0 or 1) and has a fixed summation order; k-pairs none of whose
+// symbols falls into the wave's 32 vocabulary columns are skipped (wave-uniform).
+constexpr int kAmT = 64;       // frames per workgroup
+constexpr int kAmC = 64;       // vocabulary entries per workgroup
+constexpr int kAmRows = 96;    // lattice rows per LDS pass (even)
+constexpr int kAmPairs = kAmRows / 2;
+constexpr int kAmOutPitch = 68;  // row pitch of the result tiles staged in LDS
+constexpr int kAmQ = kAmT / 4;   // 16-byte pieces per panel row (kAmT == kAmC)
+
+// four consecutive floats at any element-aligned address (global memory takes
+// unaligned 16-byte accesses); `valid` (0..4) leading elements are read, the rest is 0
+typedef float floatx4u __attribute__((ext_vector_type(4), aligned(4)));
+template <bool kVec>
+__device__ __forceinline__ dgemm::floatx4 load4_guarded(const float *base, int off, int valid) {
+  dgemm::floatx4 r = {0.f, 0.f, 0.f, 0.f};
+  if (kVec && valid >= 4) {
+    const floatx4u t = *reinterpret_cast<const floatx4u *>(base + off);
+    r[0] = t[0], r[1] = t[1], r[2] = t[2], r[3] = t[3];
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i < valid) r[i] = base[off + i];
+  }
+  return r;
+}
+
+size_t am_panel_lds_bytes(int rows_cap) {
+  const size_t panels = (size_t)rows_cap * (2 * kAmT + kAmC) * sizeof(float);
+  const size_t staging = (size_t)2 * kAmT * kAmOutPitch * sizeof(float);
+  return std::max(panels, staging) + (size_t)(2 * rows_cap + 2 * kAmT) * sizeof(float);
+}
+
+template <bool kVec>
+__global__ void __launch_bounds__(256, 2)
+    simple_bwd_am_panel_kernel(const float *__restrict__ lm, const float *__restrict__ am,
+                               const int64_t *__restrict__ symbols,
+                               const int64_t *__restrict__ boundary,
+                               const float *__restrict__ lm_max,
+                               const float *__restrict__ am_max, const float *__restrict__ dmat,
+                               const float *__restrict__ gpx, const float *__restrict__ col_y,
+                               float *__restrict__ am_grad, int B, int S, int T, int C, int ldd,
+                               int term, int rnnt_type, int rows_cap) {
+  using namespace dgemm;
+  extern __shared__ float am_lds[];
+  int *sym_s = reinterpret_cast<int *>(am_lds);   // [rows_cap] symbols of the pass (-1: none)
+  float *lmx_s = am_lds + rows_cap;               // [rows_cap] lm_max of the pass
+  float *shift_s = lmx_s + rows_cap;              // [kAmT] am_max of the tile's frames
+  float *extra_s = shift_s + kAmT;                // [kAmT] col_y of the tile's frames
+  float *As = extra_s + kAmT;                     // [rows_cap][kAmT]   D[k][t]
+  float *Gs = As + rows_cap * kAmT;               // [rows_cap][kAmT]   gx[k][t]
+  float *Bs = Gs + rows_cap * kAmT;               // [rows_cap][kAmC]   exp(lm[k][c] - max[k])
+  float *out_acc = As;                            // result tiles, after the last pass
+  float *out_hot = As + kAmT * kAmOutPitch;
+  const int S1 = S + 1;
+  const int T1 = rnnt_type == kRegular ? T + 1 : T;
+  const int c_tiles = (C + kAmC - 1) / kAmC, t_tiles = (T + kAmT - 1) / kAmT;
+  int b, tile;
+  if (!decode_block(c_tiles * t_tiles, B, b, tile)) return;
+  const int t_tile = (tile / c_tiles) * kAmT, c_tile = (tile % c_tiles) * kAmC;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, r32 = lane & 31;
+  const int wt = (wave >> 1) * 32, wc = (wave & 1) * 32;  // this wave's 32 x 32 sub-tile
+  const float *lmb = lm + (long)b * S1 * C;
+  const float *amb = am + (long)b * T * C;
+  const float *db = dmat + (long)b * S1 * ldd;
+  const float *gxb = gpx + (long)b * S * T1;
+  // symbols are < C < 2^31: their low words (little endian) are enough to compare
+  const int *sym_lo = reinterpret_cast<const int *>(symbols + (long)b * S);
+  const int t_mask = (rnnt_type == kRegular && boundary) ? (int)boundary[4 * b + 3] : -1;
+  const int c_lo = c_tile + wc;  // first vocabulary column of this wave
+  // a thread's 16-byte piece of a 64-wide row: row q_row + 16 * step, columns 4 * q_col ..
+  const int q_row = tid / kAmQ, q_col = 4 * (tid % kAmQ);
+
+  // epilogue inputs: per-frame terms through LDS (visible after the barriers of the
+  // first pass), and this thread's pieces of the am tile, rows q_row + 16 * j
+  if (tid < kAmT) {
+    const int t = t_tile + tid;
+    shift_s[tid] = t < T ? am_max[(long)b * T + t] : 0.f;
+    extra_s[tid] = t < T ? col_y[(long)b * T + t] : 0.f;
+  }
+  floatx4 am_in[kAmT / 16];
+#pragma unroll
+  for (int j = 0; j < kAmT / 16; ++j) {
+    const int t = t_tile + q_row + 16 * j, c = c_tile + q_col;
+    am_in[j] = load4_guarded<kVec>(amb, t * C + c, t < T ? min(4, max(C - c, 0)) : 0);
+  }
+
+  floatx16 acc, hot;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = hot[v] = 0.f;
+  for (int k0 = 0; k0 < S1; k0 += rows_cap) {
+    const int rows = min(rows_cap, S1 - k0);
+    const int pairs = (rows + 1) / 2;
+    constexpr int kSteps = kAmRows / 16;
+    floatx4 ra[kSteps], rg[kSteps], rb[kSteps];
+#pragma unroll
+    for (int j = 0; j < kSteps; ++j) {
+      const int k = q_row + 16 * j, t = t_tile + q_col, c = c_tile + q_col;
+      ra[j] = load4_guarded<kVec>(db, (k0 + k) * ldd + t, (k < rows && t < ldd) ? 4 : 0);
+      rg[j] = load4_guarded<kVec>(gxb, (k0 + k) * T1 + t,
+                                  (k < rows && k0 + k < S) ? min(4, max(T - t, 0)) : 0);
+      rb[j] = load4_guarded<kVec>(lmb, (k0 + k) * C + c, k < rows ? min(4, max(C - c, 0)) : 0);
+    }
+    if (k0 > 0) __syncthreads();  // the previous pass's readers are done with the panels
+    for (int k = tid; k < 2 * pairs; k += 256) {
+      sym_s[k] = (k0 + k < S) ? sym_lo[2 * (k0 + k)] : -1;
+      lmx_s[k] = (k < rows) ? lm_max[(long)b * S1 + k0 + k] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < kSteps; ++j) {
+      const int k = q_row + 16 * j;
+      if (k >= 2 * pairs) continue;
+      floatx4 gz = rg[j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) gz[i] = (t_tile + q_col + i == t_mask) ? 0.f : gz[i];
+      *reinterpret_cast<floatx4 *>(As + k * kAmT + q_col) = ra[j];
+      *reinterpret_cast<floatx4 *>(Gs + k * kAmT + q_col) = gz;
+    }
+    __syncthreads();  // lmx_s is visible
+#pragma unroll
+    for (int j = 0; j < kSteps; ++j) {
+      const int k = q_row + 16 * j, c = c_tile + q_col;
+      if (k >= 2 * pairs) continue;
+      const float mx = lmx_s[k];
+      floatx4 e;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) e[i] = (k < rows && c + i < C) ? __expf(rb[j][i] - mx) : 0.f;
+      *reinterpret_cast<floatx4 *>(Bs + k * kAmC + q_col) = e;
+    }
+    __syncthreads();
+    // dense product
+    const float *ap = As + half * kAmT + wt + r32;
+    const float *bp = Bs + half * kAmC + wc + r32;
+#pragma unroll 4
+    for (int i = 0; i < pairs; ++i)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[2 * i * kAmT], bp[2 * i * kAmC], acc, 0, 0, 0);
+    // per-symbol product, only for pairs with a symbol among this wave's columns
+    bool in = false;
+    if (lane < pairs)
+      in = (unsigned)(sym_s[2 * lane] - c_lo) < 32u || (unsigned)(sym_s[2 * lane + 1] - c_lo) < 32u;
+    unsigned long long wanted = __ballot(in);
+    const float *gp = Gs + half * kAmT + wt + r32;
+    while (wanted) {
+      const int i = __builtin_ctzll(wanted);
+      wanted &= wanted - 1;
+      const float h = (sym_s[2 * i + half] == c_lo + r32) ? 1.f : 0.f;
+      hot = __builtin_amdgcn_mfma_f32_32x32x2f32(gp[2 * i * kAmT], h, hot, 0, 0, 0);
+    }
+  }
+  // results through LDS, so that they leave as whole row segments
+  __syncthreads();
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int row = wt + 8 * (v / 4) + 4 * half + (v % 4);
+    out_acc[row * kAmOutPitch + wc + r32] = acc[v];
+    out_hot[row * kAmOutPitch + wc + r32] = hot[v];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kAmT / 16; ++j) {
+    const int row = q_row + 16 * j, t = t_tile + row, c = c_tile + q_col;
+    if (t >= T || c >= C) continue;
+    const floatx4 sum = *reinterpret_cast<const floatx4 *>(out_acc + row * kAmOutPitch + q_col);
+    const floatx4 one = *reinterpret_cast<const floatx4 *>(out_hot + row * kAmOutPitch + q_col);
+    const float shift = shift_s[row], extra = extra_s[row];
+    floatx4 res;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      res[i] = __expf(am_in[j][i] - shift) * sum[i] + one[i];
+      if (c + i == term) res[i] += extra;
+    }
+    float *dst = am_grad + ((long)b * T + t) * C + c;
+    if (kVec && c + 4 <= C) {
+      *reinterpret_cast<floatx4u *>(dst) = floatx4u{res[0], res[1], res[2], res[3]};
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (c + i < C) dst[i] = res[i];
+    }
+  }
+}
+
 // launchers: float goes to the register-direct kernels, double to the LDS-tiled ones
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
@@ -657,10 +881,19 @@ void launch_bwd_am(const float *lm, const float *am, const int64_t *symbols,
                    const int64_t *boundary, const float *lm_max, const float *am_max,
                    const float *dmat, const float *gpx, const float *col_y, float *am_grad, int B,
                    int S, int T, int C, int ldd, int term, int rnnt_type, hipStream_t stream) {
-  const int tiles = ((C + 31) / 32) * ((T + 4 * dgemm::kBM - 1) / (4 * dgemm::kBM));
-  hipLaunchKernelGGL(simple_bwd_am_direct_kernel, dim3(dgemm::xcd_grid(tiles, B)), dim3(256), 0,
-                     stream, lm, am, symbols, boundary, lm_max, am_max, dmat, gpx, col_y, am_grad,
-                     B, S, T, C, ldd, term, rnnt_type);
+  const int tiles = ((C + kAmC - 1) / kAmC) * ((T + kAmT - 1) / kAmT);
+  // rows of k held in LDS per pass: all of them when they fit
+  const int rows_cap = std::min(kAmRows, (S + 2) & ~1);
+  const size_t lds = am_panel_lds_bytes(rows_cap);
+  // (the 16-byte accesses need no alignment; the scalar variant exists for checking)
+  const bool vec = true;
+  auto kernel = vec ? simple_bwd_am_panel_kernel<true> : simple_bwd_am_panel_kernel<false>;
+  if (lds > 64 * 1024)
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(tiles, B)), dim3(256), lds, stream, lm, am,
+                     symbols, boundary, lm_max, am_max, dmat, gpx, col_y, am_grad, B, S, T, C, ldd,
+                     term, rnnt_type, rows_cap);
 }
 void launch_bwd_am(const double *lm, const double *am, const int64_t *symbols,
                    const int64_t *boundary, const double *lm_max, const double *am_max,
@@ -711,8 +944,8 @@ int fwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
 
 template <typename R>
 int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *boundary,
-             const R *lm_max, const R *am_max, const R *norm_raw, const R *score_grad, R *px_grad,
-             R *py_grad, R *dmat, R *row_x, R *row_y, R *col_y, R *lm_grad, R *am_grad, int B,
+             const R *lm_max, const R *am_max, const R *norm_raw, const R *score_grad,
+             int score_grad_stride, double score_grad_scale, R *px_grad, R *py_grad, R *dmat, R *row_x, R *row_y, R *col_y, R *lm_grad, R *am_grad, int B,
              int S, int T, int C, int term, int rnnt_type, void *stream_) {
   if (B < 0 || S < 0 || T < 0 || C < 1) return fail(FRNNT_EINVAL, "simple_logprobs_bwd: bad size");
   if (rnnt_type < 0 || rnnt_type > 2 || term < 0 || term >= C)
@@ -723,12 +956,15 @@ int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
     return fail(FRNNT_EINVAL, "simple_logprobs_bwd: null pointer");
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   if (score_grad) {
+    if (score_grad_stride != 0 && score_grad_stride != 1)
+      return fail(FRNNT_EINVAL, "simple_logprobs_bwd: score_grad_stride must be 0 or 1");
     const int T1 = rnnt_type == kRegular ? T + 1 : T;
-    const long per_x = (long)S * T1, per_y = (long)(S + 1) * T;
-    const long total = (per_x + per_y) * B;
-    if (total > 0)
-      hipLaunchKernelGGL(scale_by_batch_kernel<R>, dim3((unsigned)((total + 255) / 256)),
-                         dim3(256), 0, stream, px_grad, py_grad, score_grad, per_x, per_y, B);
+    const int per_x = S * T1, per_y = (S + 1) * T;
+    const int x_blocks = (per_x + 1023) / 1024, y_blocks = (per_y + 1023) / 1024;
+    if (x_blocks + y_blocks > 0)
+      hipLaunchKernelGGL(scale_by_batch_kernel<R>, dim3(x_blocks + y_blocks, B), dim3(256), 0,
+                         stream, px_grad, py_grad, score_grad, score_grad_stride,
+                         (R)score_grad_scale, per_x, per_y, x_blocks);
   }
   const int ldd = (T + 3) & ~3;  // leading dimension of dmat: 16-byte rows
   const long prep_blocks = ((long)B * (S + 1) + 3) / 4 + (long)B * ((T + kWave - 1) / kWave);
@@ -742,6 +978,17 @@ int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
     launch_bwd_am(lm, am, symbols, boundary, lm_max, am_max, dmat, px_grad, col_y, am_grad, B, S,
                   T, C, ldd, term, rnnt_type, stream);
   return check_launch("simple_logprobs_bwd");
+}
+
+template <typename R>
+int reduce_impl(const R *scores, R *loss, int B, int reduction, void *stream) {
+  if (B < 0 || reduction < 0 || reduction > 2)
+    return fail(FRNNT_EINVAL, "loss_reduce: bad size or reduction");
+  if (!loss || (B > 0 && !scores)) return fail(FRNNT_EINVAL, "loss_reduce: null pointer");
+  if (B == 0 && reduction == 0) return FRNNT_OK;
+  hipLaunchKernelGGL(loss_reduce_kernel<R>, dim3(1), dim3(kWave), 0,
+                     static_cast<hipStream_t>(stream), scores, loss, B, reduction);
+  return check_launch("loss_reduce");
 }
 
 }  // namespace
@@ -766,24 +1013,33 @@ int frnnt_simple_logprobs_fwd_f64(const double *lm, const double *am, const int6
 int frnnt_simple_logprobs_bwd_f32(const float *lm, const float *am, const int64_t *symbols,
                                   const int64_t *boundary, const float *lm_max,
                                   const float *am_max, const float *norm_raw,
-                                  const float *score_grad, float *px_grad, float *py_grad,
+                                  const float *score_grad, int score_grad_stride,
+                                  double score_grad_scale, float *px_grad, float *py_grad,
                                   float *dmat, float *row_x, float *row_y, float *col_y,
                                   float *lm_grad, float *am_grad, int B, int S, int T, int C,
                                   int termination_symbol, int rnnt_type, void *stream) {
   return frnnt::bwd_impl<float>(lm, am, symbols, boundary, lm_max, am_max, norm_raw, score_grad,
-                                px_grad, py_grad, dmat, row_x, row_y, col_y, lm_grad, am_grad, B,
+                                score_grad_stride, score_grad_scale, px_grad, py_grad, dmat, row_x, row_y, col_y, lm_grad, am_grad, B,
                                 S, T, C, termination_symbol, rnnt_type, stream);
 }
 int frnnt_simple_logprobs_bwd_f64(const double *lm, const double *am, const int64_t *symbols,
                                   const int64_t *boundary, const double *lm_max,
                                   const double *am_max, const double *norm_raw,
-                                  const double *score_grad, double *px_grad, double *py_grad,
+                                  const double *score_grad, int score_grad_stride,
+                                  double score_grad_scale, double *px_grad, double *py_grad,
                                   double *dmat, double *row_x, double *row_y, double *col_y,
                                   double *lm_grad, double *am_grad, int B, int S, int T, int C,
                                   int termination_symbol, int rnnt_type, void *stream) {
   return frnnt::bwd_impl<double>(lm, am, symbols, boundary, lm_max, am_max, norm_raw, score_grad,
-                                 px_grad, py_grad, dmat, row_x, row_y, col_y, lm_grad, am_grad, B,
+                                 score_grad_stride, score_grad_scale, px_grad, py_grad, dmat, row_x, row_y, col_y, lm_grad, am_grad, B,
                                  S, T, C, termination_symbol, rnnt_type, stream);
+}
+
+int frnnt_loss_reduce_f32(const float *scores, float *loss, int B, int reduction, void *stream) {
+  return frnnt::reduce_impl<float>(scores, loss, B, reduction, stream);
+}
+int frnnt_loss_reduce_f64(const double *scores, double *loss, int B, int reduction, void *stream) {
+  return frnnt::reduce_impl<double>(scores, loss, B, reduction, stream);
 }
 
 }  // extern "C"

@@ -105,7 +105,8 @@ class _SimpleLogprobs(torch.autograd.Function):
             am_grad = torch.empty_like(am) if ctx.needs_input_grad[1] else None
             _lib.call("frnnt_simple_logprobs_bwd_" + sfx, lm.data_ptr(), am.data_ptr(),
                       sym.data_ptr(), _lib.ptr(bnd), lm_max.data_ptr(), am_max.data_ptr(),
-                      norm_raw.data_ptr(), None, gpx.data_ptr(), gpy.data_ptr(), dmat.data_ptr(),
+                      norm_raw.data_ptr(), None, 0, 1.0, gpx.data_ptr(), gpy.data_ptr(),
+                      dmat.data_ptr(),
                       row_x.data_ptr(), row_y.data_ptr(), col_y.data_ptr(), _lib.ptr(lm_grad),
                       _lib.ptr(am_grad), B, S, T, C, term, kind, _lib.stream_of(am))
         return lm_grad, am_grad, None, None, None, None
@@ -169,18 +170,23 @@ def _recursion_and_reduce(px, py, boundary, rnnt_type, delay_penalty, reduction,
     return (loss, scores_and_grads[1]) if return_grad else loss
 
 
-class _SimpleLossScores(torch.autograd.Function):
+_REDUCTIONS = {"none": 0, "mean": 1, "sum": 2}
+
+
+class _SimpleLoss(torch.autograd.Function):
     """rnnt_loss_simple's whole device pipeline behind one autograd node:
-    px/py (row maxima + MFMA contraction), the lattice recursion forward, and --
-    as the recursion's autograd wrapper does (mutual_information.py:159-168) --
-    its backward with a gradient of ones, whose result both is handed out as
-    (px_grad, py_grad) and is what backward() scales in place and pushes through
-    the two gradient GEMMs.  Same arithmetic as get_rnnt_logprobs followed by
-    mutual_information_recursion; it only saves Python and launch overhead."""
+    px/py (row maxima + MFMA contraction), the lattice recursion forward, the
+    reduction of the scores to the loss, and -- as the recursion's autograd wrapper
+    does (mutual_information.py:159-168) -- the recursion's backward with a gradient
+    of ones, whose result both is handed out as (px_grad, py_grad) and is what
+    backward() scales in place and pushes through the two gradient GEMMs.  Same
+    arithmetic as get_rnnt_logprobs, mutual_information_recursion and the
+    reduction of rnnt_loss.py:330-340; it only saves Python, launch and
+    elementwise-kernel overhead."""
 
     @staticmethod
     def forward(ctx, lm, am, symbols, boundary, termination_symbol, rnnt_type, delay_penalty,
-                want_grads):
+                want_grads, reduction):
         B, T, C = am.shape
         S = lm.shape[1] - 1
         kind = _RNNT_TYPES[rnnt_type]
@@ -191,6 +197,8 @@ class _SimpleLossScores(torch.autograd.Function):
         opts = dict(dtype=am.dtype, device=am.device)
         T1 = T + 1 if kind == 0 else T
         need_grad = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        # gradients of the non-differentiable outputs are not wanted as zero tensors
+        ctx.set_materialize_grads(False)
         with torch.cuda.device(am.device):
             stream = _lib.stream_of(am)
             px = torch.empty(B, S, T1, **opts)
@@ -216,22 +224,30 @@ class _SimpleLossScores(torch.autograd.Function):
                 _lib.call("frnnt_mi_backward_" + sfx, px.data_ptr(), py.data_ptr(),
                           _lib.ptr(bnd_c), p.data_ptr(), None, px_grad.data_ptr(),
                           py_grad.data_ptr(), B, S, T, modified, 0, stream)
+            loss = torch.empty((B,) if reduction == 0 else (), **opts)
+            _lib.call("frnnt_loss_reduce_" + sfx, scores.data_ptr(), loss.data_ptr(), B,
+                      reduction, stream)
         if need_grad:
             ctx.save_for_backward(lm_c, am_c, sym_c, bnd_c, lm_max, am_max, norm_raw, px_grad,
                                   py_grad)
-            ctx.meta = (B, S, T, C, int(termination_symbol), kind, sfx)
+            ctx.meta = (B, S, T, C, int(termination_symbol), kind, sfx, reduction)
         if px_grad is None:
-            return scores, None, None
+            return loss, None, None
         ctx.mark_non_differentiable(px_grad, py_grad)
-        return scores, px_grad, py_grad
+        return loss, px_grad, py_grad
 
     @staticmethod
-    def backward(ctx, g_scores, _gx, _gy):
+    def backward(ctx, g_loss, _gx, _gy):
+        if g_loss is None:
+            return (None,) * 9
         lm, am, sym, bnd, lm_max, am_max, norm_raw, px_grad, py_grad = ctx.saved_tensors
-        B, S, T, C, term, kind, sfx = ctx.meta
+        B, S, T, C, term, kind, sfx, reduction = ctx.meta
         opts = dict(dtype=am.dtype, device=am.device)
         with torch.cuda.device(am.device):
-            g = g_scores.contiguous()
+            # d loss / d scores[b] = scale * g_loss[b * stride]
+            g = g_loss.contiguous()
+            stride = 1 if reduction == 0 else 0
+            scale = -1.0 / B if reduction == 1 else -1.0
             dmat = torch.empty(B, S + 1, (T + 3) // 4 * 4, **opts)
             row_x = torch.empty(B, S + 1, **opts)
             row_y = torch.empty(B, S + 1, **opts)
@@ -242,21 +258,11 @@ class _SimpleLossScores(torch.autograd.Function):
             # MutualInformationRecursionFunction.backward does to the tensors it handed out
             _lib.call("frnnt_simple_logprobs_bwd_" + sfx, lm.data_ptr(), am.data_ptr(),
                       sym.data_ptr(), _lib.ptr(bnd), lm_max.data_ptr(), am_max.data_ptr(),
-                      norm_raw.data_ptr(), g.data_ptr(), px_grad.data_ptr(), py_grad.data_ptr(),
-                      dmat.data_ptr(), row_x.data_ptr(), row_y.data_ptr(), col_y.data_ptr(),
-                      _lib.ptr(lm_grad), _lib.ptr(am_grad), B, S, T, C, term, kind,
-                      _lib.stream_of(am))
-        return lm_grad, am_grad, None, None, None, None, None, None
-
-
-def _reduce(negated_loss: Tensor, reduction: Optional[str]) -> Tensor:
-    if reduction == "none":
-        return -negated_loss
-    if reduction == "mean":
-        return -torch.mean(negated_loss)
-    if reduction == "sum":
-        return -torch.sum(negated_loss)
-    raise ValueError(f"reduction should be ('none' | 'mean' | 'sum'), given {reduction}")
+                      norm_raw.data_ptr(), g.data_ptr(), stride, scale, px_grad.data_ptr(),
+                      py_grad.data_ptr(), dmat.data_ptr(), row_x.data_ptr(), row_y.data_ptr(),
+                      col_y.data_ptr(), _lib.ptr(lm_grad), _lib.ptr(am_grad), B, S, T, C, term,
+                      kind, _lib.stream_of(am))
+        return lm_grad, am_grad, None, None, None, None, None, None, None
 
 
 def rnnt_loss_simple(
@@ -290,10 +296,9 @@ def rnnt_loss_simple(
             assert 0 <= t_begin <= t_end <= T
     if reduction not in ("none", "mean", "sum"):
         raise ValueError(f"reduction should be ('none' | 'mean' | 'sum'), given {reduction}")
-    scores, px_grad, py_grad = _SimpleLossScores.apply(
+    loss, px_grad, py_grad = _SimpleLoss.apply(
         lm, am, symbols, boundary, termination_symbol, rnnt_type, float(delay_penalty),
-        bool(return_grad))
-    loss = _reduce(scores, reduction)
+        bool(return_grad), _REDUCTIONS[reduction])
     return (loss, (px_grad, py_grad)) if return_grad else loss
 
 

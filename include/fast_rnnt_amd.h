@@ -114,10 +114,13 @@ int frnnt_simple_logprobs_fwd_f64(const double *lm, const double *am, const int6
  * Backward of the above: what autograd derives for rnnt_loss.py:174-225, as one
  * elementwise pass plus two MFMA GEMMs.
  *   px_grad, py_grad: dL/dpx, dL/dpy (shapes of px, py)                    in
- *   score_grad [B] or NULL: when given, px_grad[b] and py_grad[b] are first multiplied
- *     IN PLACE by score_grad[b] -- the scaling step of the recursion's autograd
- *     backward (mutual_information.py:173-181), for callers that hold the occupation
- *     gradients and the gradient of the scores separately
+ *   score_grad or NULL: when given, px_grad[b] and py_grad[b] are first multiplied
+ *     IN PLACE by score_grad_scale * score_grad[b * score_grad_stride] -- the scaling
+ *     step of the recursion's autograd backward (mutual_information.py:173-181), for
+ *     callers that hold the occupation gradients and the gradient of the scores
+ *     separately.  score_grad_stride 1: one value per utterance; 0: one scalar for
+ *     all (the gradient of a summed or averaged loss, with the sign and the 1/B of
+ *     rnnt_loss.py:160-169 in score_grad_scale)
  *   dmat [B][S+1][T rounded up to a multiple of 4], row_x [B][S+1], row_y [B][S+1],
  *   col_y [B][T]                                                           scratch
  *   lm_grad [B][S+1][C], am_grad [B][T][C]: out; either may be NULL to skip it
@@ -125,17 +128,27 @@ int frnnt_simple_logprobs_fwd_f64(const double *lm, const double *am, const int6
 int frnnt_simple_logprobs_bwd_f32(const float *lm, const float *am, const int64_t *symbols,
                                   const int64_t *boundary, const float *lm_max,
                                   const float *am_max, const float *norm_raw,
-                                  const float *score_grad, float *px_grad, float *py_grad,
+                                  const float *score_grad, int score_grad_stride,
+                                  double score_grad_scale, float *px_grad, float *py_grad,
                                   float *dmat, float *row_x, float *row_y, float *col_y,
                                   float *lm_grad, float *am_grad, int B, int S, int T, int C,
                                   int termination_symbol, int rnnt_type, void *stream);
 int frnnt_simple_logprobs_bwd_f64(const double *lm, const double *am, const int64_t *symbols,
                                   const int64_t *boundary, const double *lm_max,
                                   const double *am_max, const double *norm_raw,
-                                  const double *score_grad, double *px_grad, double *py_grad,
+                                  const double *score_grad, int score_grad_stride,
+                                  double score_grad_scale, double *px_grad, double *py_grad,
                                   double *dmat, double *row_x, double *row_y, double *col_y,
                                   double *lm_grad, double *am_grad, int B, int S, int T, int C,
                                   int termination_symbol, int rnnt_type, void *stream);
+/*
+ * The reduction at the end of every loss function (rnnt_loss.py:160-169, :330-340):
+ * loss = -scores (reduction 0, [B]), -mean(scores) (1, one value) or -sum(scores)
+ * (2, one value), summed in a fixed order by one workgroup.
+ */
+int frnnt_loss_reduce_f32(const float *scores, float *loss, int B, int reduction, void *stream);
+int frnnt_loss_reduce_f64(const double *scores, double *loss, int B, int reduction, void *stream);
+
 
 /*
  * px / py from joiner logits.  Replaces the tensor algebra of
