@@ -33,6 +33,8 @@ constexpr int kChunk = 8;              // steps per seam hand-over
 constexpr int kTileSteps = 32;         // steps per staged tile
 constexpr int kTilePitch = kTileSteps + 1;
 constexpr int kTileElems = kWave * kTilePitch;
+constexpr int kSeamPad = kChunk;        // slack on either side of a seam row, so that a whole
+                                       // chunk of seam values is written without bounds tests
 constexpr int kFwdStagers = 2;         // staging waves per sweep wave
 constexpr int kBwdStagers = 3;
 constexpr int kSpinLimit = 1 << 22;
@@ -66,6 +68,15 @@ __device__ __forceinline__ bool wait_for(const int *counter, int target) {
   }
   return true;
 }
+// Non-blocking look at a counter: the value is used a chunk or a tile later, when it
+// has long arrived.  LDS serves the reads of one wave in order, so data read after
+// the counter is at least as recent as the counter; the empty asm keeps the compiler
+// from moving such reads ahead of it.
+__device__ __forceinline__ int peek(const int *counter) {
+  const int v = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  asm volatile("" ::: "memory");
+  return v;
+}
 __device__ __forceinline__ void publish(int *counter, int value) {
   __hip_atomic_store(counter, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
@@ -74,33 +85,57 @@ __device__ __forceinline__ void publish(int *counter, int value) {
 // written so that the only fix-up is the NaN that (-inf) - (-inf) produces.
 __device__ __forceinline__ float chain_log_add(float a, float c) {
   const float d = a - c;
-  const float hi = (a > c) ? a : c;
+  const float hi = fmaxf(a, c);  // neither operand is ever NaN
   // -|d| * log2(e) is <= 0 or NaN ((-inf) - (-inf)); fminf maps the NaN to 0, and
   // the result is then hi + log(2) = hi, because hi is infinite in that case --
   // exactly the "return the larger operand" rule of the reference, without a branch.
   const float t = fminf(-fabsf(d) * 1.44269504088896341f, 0.0f);
   const float e = __builtin_amdgcn_exp2f(t);
-  const float l = __builtin_amdgcn_logf(1.0f + e) * 0.693147180559945309f;
-  return hi + l;
+  return __builtin_fmaf(__builtin_amdgcn_logf(1.0f + e), 0.693147180559945309f, hi);
 }
 __device__ __forceinline__ double chain_log_add(double a, double c) { return log_add(a, c); }
 
-// Four consecutive elements with one 16-byte store; the address only needs element
-// alignment (global memory accepts unaligned vector stores).
-template <typename R>
-struct Vec4 {
-  typedef R type __attribute__((ext_vector_type(4), aligned(sizeof(R))));
-};
-template <typename R>
-__device__ __forceinline__ void store4(R *dst, R a, R b, R c, R d) {
-  typename Vec4<R>::type v;
-  v[0] = a;
-  v[1] = b;
-  v[2] = c;
-  v[3] = d;
-  *reinterpret_cast<typename Vec4<R>::type *>(dst) = v;
-}
+// Results leave the sweep waves through raw buffer stores: the resource covers one
+// utterance's array, a lane passes a byte offset, and an offset of kDropped lies
+// outside every resource, so the hardware's range check discards the store.  That
+// turns "this lane has nothing to write here" into one select on the offset, with
+// no branch and no change of the execution mask.
+constexpr int kDropped = (int)0x80000000;
+// Byte offset standing for "this lane has no row": adding any in-row displacement
+// (less than 2^30 in magnitude) to it still lies outside every resource.
+constexpr int kNoRow = (int)0xC0000000;
+typedef int intx2 __attribute__((ext_vector_type(2)));
+typedef int intx4 __attribute__((ext_vector_type(4)));
 
+template <typename R>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(R *base, size_t elems) {
+  // raw buffer (stride 0), 32-bit elements as far as the descriptor is concerned
+  return __builtin_amdgcn_make_buffer_rsrc(base, 0, (int)(elems * sizeof(R)), 0x00020000);
+}
+__device__ __forceinline__ void put1(__amdgpu_buffer_rsrc_t rs, int off, float v) {
+  __builtin_amdgcn_raw_buffer_store_b32(__float_as_int(v), rs, off, 0, 0);
+}
+__device__ __forceinline__ void put1(__amdgpu_buffer_rsrc_t rs, int off, double v) {
+  const long long bits = __double_as_longlong(v);
+  __builtin_amdgcn_raw_buffer_store_b64(intx2{(int)bits, (int)(bits >> 32)}, rs, off, 0, 0);
+}
+// four consecutive elements (the address only needs element alignment)
+__device__ __forceinline__ void put4(__amdgpu_buffer_rsrc_t rs, int off, float a, float b, float c,
+                                     float d) {
+  __builtin_amdgcn_raw_buffer_store_b128(
+      intx4{__float_as_int(a), __float_as_int(b), __float_as_int(c), __float_as_int(d)}, rs, off,
+      0, 0);
+}
+__device__ __forceinline__ void put4(__amdgpu_buffer_rsrc_t rs, int off, double a, double b,
+                                     double c, double d) {
+  const long long ab = __double_as_longlong(a), bb = __double_as_longlong(b);
+  const long long cb = __double_as_longlong(c), db = __double_as_longlong(d);
+  __builtin_amdgcn_raw_buffer_store_b128(
+      intx4{(int)ab, (int)(ab >> 32), (int)bb, (int)(bb >> 32)}, rs, off, 0, 0);
+  __builtin_amdgcn_raw_buffer_store_b128(
+      intx4{(int)cb, (int)(cb >> 32), (int)db, (int)(db >> 32)}, rs, off == kDropped ? off : off + 16,
+      0, 0);
+}
 struct Counters {
   int ready[kMaxSweep];                   // seam columns published by sweep wave w
   int consumed[kMaxSweep];                // tiles sweep wave w has finished
@@ -156,8 +191,10 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
   const R *pxb = px + (size_t)b * S * T1;
   const R *pyb = py + (size_t)b * (S + 1) * T;
   R *pb = p + (size_t)b * (S + 1) * TP;
+  const __amdgpu_buffer_rsrc_t p_rsrc = buffer_of(pb, (size_t)(S + 1) * TP);
   R *seam = reinterpret_cast<R *>(dyn_lds);
-  R *tiles = seam + (size_t)nsweep * TP;  // [nsweep][2 arrays][2 buffers][kTileElems]
+  const int seam_pitch = TP + 2 * kSeamPad;
+  R *tiles = seam + (size_t)nsweep * seam_pitch;  // [nsweep][2 arrays][2 buffers][kTileElems]
   const int band_rows = kWave * nsweep;
 
   if (wave >= nsweep) {
@@ -221,8 +258,8 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
   // -------------------------------- sweep wave ---------------------------------
   const int w = wave;
   const int prev = (w + nsweep - 1) % nsweep;
-  R *my_seam = seam + (size_t)w * TP;
-  const R *up_seam = seam + (size_t)prev * TP;
+  R *my_seam = seam + (size_t)w * seam_pitch + kSeamPad;
+  const R *up_seam = seam + (size_t)prev * seam_pitch + kSeamPad;
   const R *xt = tiles + (size_t)w * 4 * kTileElems;
   const R *yt = xt + 2 * kTileElems;
   int tile_base = 0;
@@ -234,16 +271,30 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
     const bool has_up = g.row0 > 0;
     const int up_base = (w > 0 ? band : band - 1) * cols;
     const int my_base = band * cols;
-    R *p_row = pb + (long)(win.s0 + i) * TP + win.t0;
+    // byte offset in p[b] of (this lane's row, column -lane): a chunk adds its first
+    // step; lanes without a row get an offset that every store drops
+    const int p_lane = row_ok ? ((win.s0 + i) * TP + win.t0 - lane) * (int)sizeof(R) : kNoRow;
+    // the answer is the cell (NS, NT): lane NS - row0 at step NT + NS - row0
+    const int fin_lane = NS - g.row0;
+    const int fin_step = (fin_lane < kWave) ? NT + fin_lane : -1;
 
     R own = (i == 0) ? (R)0 : ninf, own2 = ninf;
-    R fin = ninf;  // value of this lane's cell in column NT
+    R fin = ninf;
     const bool has_down = g.nrows == kWave;
+    // counters and seam values are read one chunk (one tile) ahead of their use, so
+    // that the LDS round trip is off the chain; a stale value only costs a re-read
+    int seen_ready = 0;
+    R seen_seam = ninf;
+    int seen_loaded[kFwdStagers];
+#pragma unroll
+    for (int l = 0; l < kFwdStagers; ++l) seen_loaded[l] = 0;
     for (int m = 0; m < g.ntiles; ++m) {
       const int gt = tile_base + m;
 #pragma unroll
       for (int l = 0; l < kFwdStagers; ++l)
-        if (!wait_for(&cnt.loaded[w * kFwdStagers + l], gt + 1)) return;
+        if (__builtin_amdgcn_readfirstlane(seen_loaded[l]) < gt + 1 &&
+            !wait_for(&cnt.loaded[w * kFwdStagers + l], gt + 1))
+          return;
       // this lane's 32 steps of inputs go to registers in one burst, after which
       // the staging waves may refill the buffer
       R xq[kTileSteps], yq[kTileSteps];
@@ -259,8 +310,8 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
       if (lane == 0) publish(&cnt.consumed[w], gt + 1);
 
       // One chunk of kChunk steps, specialised at compile time on whether the wave
-      // receives a seam (kUp), feeds one (kDown), and whether every lane's cell is
-      // inside the window for the whole chunk (!kEdge).
+      // receives a seam (kUp), feeds one (kDown), and whether some lane's column
+      // leaves the window during the chunk (kEdge).
       bool alive = true;
       auto chunk = [&](auto up_c, auto down_c, auto edge_c, int c4, int e0)
                        __attribute__((always_inline)) {
@@ -270,15 +321,26 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
         R handed = ninf;  // lane k: the seam value lane 0 needs at step e0 + k
         if (kUp) {
           const int need = min(e0 + kChunk - shift, cols);
-          if (need > 0 && !wait_for(&cnt.ready[prev], up_base + need)) {
-            alive = false;
-            return;
+          handed = seen_seam;
+          if (need > 0 && __builtin_amdgcn_readfirstlane(seen_ready) < up_base + need) {
+            if (!wait_for(&cnt.ready[prev], up_base + need)) {
+              alive = false;
+              return;
+            }
+            const int col = e0 + lane - shift;
+            handed = (lane < kChunk && col >= 0 && col <= NT) ? up_seam[col] : ninf;
           }
-          const int col = e0 + lane - shift;
-          if (lane < kChunk && col >= 0 && col <= NT) handed = up_seam[col];
+          // next chunk's counter, then its seam values (LDS serves a wave in order)
+          seen_ready = peek(&cnt.ready[prev]);
+          const int col = e0 + kChunk + lane - shift;
+          seen_seam = ninf;
+          if (lane < kChunk && col >= 0 && col <= NT)
+            seen_seam = up_seam[col];
         }
-        R *pp = p_row + (e0 - lane);
-        R *sp = my_seam + (e0 - (kWave - 1));
+        if (c4 == kTileSteps / kChunk - 1) {
+#pragma unroll
+          for (int l = 0; l < kFwdStagers; ++l) seen_loaded[l] = peek(&cnt.loaded[w * kFwdStagers + l]);
+        }
         R vals[kChunk];
 #pragma unroll
         for (int k = 0; k < kChunk; ++k) {
@@ -292,34 +354,39 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
           }
           const R v = chain_log_add(up + xq[kk], own + yq[kk]);
           vals[k] = v;
-          const int j63 = e0 + k - (kWave - 1);  // column of the seam lane, wave-uniform
-          if (kEdge) {
-            const int j = e0 + k - lane;
-            fin = (j == NT) ? v : fin;
-            if (kDown && j63 >= 0 && j63 <= NT && lane == kWave - 1) sp[k] = v;
-          } else {
-            if (kDown && lane == kWave - 1) sp[k] = v;
-          }
           own2 = own;
           own = v;
         }
-        // p goes out in groups of four columns: one 16-byte store when the whole
-        // group lies inside the window, single stores otherwise
+        const int kf = fin_step - e0;  // wave-uniform
+        if ((unsigned)kf < (unsigned)kChunk) {
 #pragma unroll
-        for (int q4 = 0; q4 < kChunk; q4 += 4) {
-          const int j0 = e0 + q4 - lane;
-          const bool whole = !kEdge || (j0 >= 0 && j0 + 3 <= NT);
-          if (whole && row_ok) {
-            store4(pp + q4, vals[q4], vals[q4 + 1], vals[q4 + 2], vals[q4 + 3]);
-          } else if (row_ok) {
+          for (int k = 0; k < kChunk; ++k)
+            if (k == kf) fin = vals[k];
+        }
+        // seam: the last lane's columns e0 - 63 ... (the pads take what falls outside)
+        if (kDown && e0 + kChunk > kWave - 1) {
+          if (lane == kWave - 1) {
+            R *sp = my_seam + (e0 - (kWave - 1));
 #pragma unroll
-            for (int k = 0; k < 4; ++k)
-              if ((unsigned)(j0 + k) <= (unsigned)NT) pp[q4 + k] = vals[q4 + k];
+            for (int k = 0; k < kChunk; ++k) sp[k] = vals[k];
+            const int done = max(0, min(e0 + kChunk - (kWave - 1), cols));
+            publish(&cnt.ready[w], my_base + done);
           }
         }
-        if (kDown && lane == kWave - 1) {
-          const int done = max(0, min(e0 + kChunk - (kWave - 1), cols));
-          publish(&cnt.ready[w], my_base + done);
+        // p: whole groups of four columns inside the window, single columns at its ends
+        const int first = p_lane + e0 * (int)sizeof(R);
+        if (!kEdge) {
+#pragma unroll
+          for (int q4 = 0; q4 < kChunk; q4 += 4)
+            put4(p_rsrc, first + q4 * (int)sizeof(R), vals[q4], vals[q4 + 1], vals[q4 + 2],
+                 vals[q4 + 3]);
+        } else {
+          const int j0 = e0 - lane;
+#pragma unroll
+          for (int k = 0; k < kChunk; ++k) {
+            const bool ok = (unsigned)(j0 + k) <= (unsigned)NT;
+            put1(p_rsrc, (ok ? first : kDropped) + k * (int)sizeof(R), vals[k]);
+          }
         }
       };
       auto tile = [&](auto up_c, auto down_c) __attribute__((always_inline)) {
@@ -327,8 +394,8 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
         for (int c4 = 0; c4 < kTileSteps / kChunk; ++c4) {
           const int e0 = m * kTileSteps + c4 * kChunk;
           if (e0 < g.nsteps && alive) {
-            const bool interior =
-                g.nrows == kWave && e0 >= kWave - 1 && e0 + kChunk <= NT;
+            // interior: the columns of all lanes that have a row stay inside the window
+            const bool interior = e0 >= g.nrows - 1 && e0 + kChunk <= NT + 1;
             if (interior)
               chunk(up_c, down_c, std::false_type{}, c4, e0);
             else
@@ -349,7 +416,7 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
       }
       if (!alive) return;
     }
-    if (row_ok && i == NS) ans[b] = fin;
+    if (lane == fin_lane) ans[b] = fin;
     tile_base += g.ntiles;
   }
 }
@@ -383,23 +450,54 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
   const Window win = load_window(boundary, b, S, T);
   R *gxb = px_grad + (size_t)b * S * T1;
   R *gyb = py_grad + (size_t)b * (S + 1) * T;
+  const __amdgpu_buffer_rsrc_t gx_rsrc = buffer_of(gxb, (size_t)S * T1);
+  const __amdgpu_buffer_rsrc_t gy_rsrc = buffer_of(gyb, (size_t)(S + 1) * T);
 
-  // exact zeros everywhere the sweep does not write: one wave per row
-  if (boundary) {
+  // Exact zeros everywhere the sweep does not write, one wave per row.  The staging
+  // waves do this after their last tile, off the critical path (a barrier after these
+  // stores would have to wait until they have all reached memory).
+  // elements [begin, end) of the row that starts at element `row` of the resource;
+  // begin and end are wave-uniform
+  auto zero_range = [&](__amdgpu_buffer_rsrc_t rs, int row, int begin, int end) {
+    const int len = end - begin;
+    if (len <= 0) return;
+    const R z = 0;
+    if (len < 4) {
+      put1(rs, lane < len ? (row + begin + lane) * (int)sizeof(R) : kDropped, z);
+      return;
+    }
+    for (int t0 = begin; t0 + 4 <= end; t0 += 4 * kWave) {
+      const int t = t0 + 4 * lane;
+      put4(rs, t + 4 <= end ? (row + t) * (int)sizeof(R) : kDropped, z, z, z, z);
+    }
+    // what is left of the last group, as one group that ends with the range
+    if (len & 3) put4(rs, lane == 0 ? (row + end - 4) * (int)sizeof(R) : kDropped, z, z, z, z);
+  };
+  auto zero_outside = [&](int part, int parts) {
+    if (!boundary) return;
     const int s_lo = win.s0, s_hi = win.s0 + win.ns;
     const int t_lo = win.t0, t_hi = win.t0 + win.nt;
-    for (int s = wave; s <= S; s += nwaves) {
+    for (int s = part; s <= S; s += parts) {
       if (s < S) {
-        const bool row_in = win.ok && s >= s_lo && s < s_hi;
-        for (int t = lane; t < T1; t += kWave)
-          if (!(row_in && t >= t_lo && t <= t_hi - shift)) gxb[(long)s * T1 + t] = 0;
+        if (win.ok && s >= s_lo && s < s_hi) {
+          zero_range(gx_rsrc, s * T1, 0, t_lo);
+          zero_range(gx_rsrc, s * T1, t_hi - shift + 1, T1);
+        } else {
+          zero_range(gx_rsrc, s * T1, 0, T1);
+        }
       }
-      const bool row_in = win.ok && s >= s_lo && s <= s_hi;
-      for (int t = lane; t < T; t += kWave)
-        if (!(row_in && t >= t_lo && t < t_hi)) gyb[(long)s * T + t] = 0;
+      if (win.ok && s >= s_lo && s <= s_hi) {
+        zero_range(gy_rsrc, s * T, 0, t_lo);
+        zero_range(gy_rsrc, s * T, t_hi, T);
+      } else {
+        zero_range(gy_rsrc, s * T, 0, T);
+      }
     }
+  };
+  if (!win.ok) {
+    zero_outside(wave, nwaves);
+    return;
   }
-  if (!win.ok) return;
   if (threadIdx.x < (int)(sizeof(Counters) / sizeof(int)))
     reinterpret_cast<int *>(&cnt)[threadIdx.x] = 0;
   __syncthreads();
@@ -408,7 +506,8 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
   const R *pxb = px + (size_t)b * S * T1;
   const R *pb = p + (size_t)b * (S + 1) * TP;
   R *seam = reinterpret_cast<R *>(dyn_lds);
-  R *tiles = seam + (size_t)nsweep * TP;  // per sweep wave: d1[2], d2[2] tiles
+  const int seam_pitch = TP + 2 * kSeamPad;
+  R *tiles = seam + (size_t)nsweep * seam_pitch;  // per sweep wave: d1[2], d2[2] tiles
   const int band_rows = kWave * nsweep;
 
   if (wave >= nsweep) {
@@ -517,16 +616,18 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
       }
       tile_base += g.ntiles;
     }
+    zero_outside(wave - nsweep, nwaves - nsweep);
     return;
   }
 
   // -------------------------------- sweep wave ---------------------------------
   const int w = wave;
   const int prev = (w + nsweep - 1) % nsweep;
-  R *my_seam = seam + (size_t)w * TP;
-  const R *up_seam = seam + (size_t)prev * TP;
+  R *my_seam = seam + (size_t)w * seam_pitch + kSeamPad;
+  const R *up_seam = seam + (size_t)prev * seam_pitch + kSeamPad;
   const R *base = tiles + (size_t)w * 4 * kTileElems;
   const R seed = ans_grad ? ans_grad[b] : (R)1;
+  constexpr int kSize = (int)sizeof(R);
   int tile_base = 0;
   for (int band = 0; band * band_rows <= NS; ++band) {
     const Band g = band_of(band, w, nsweep, NS, NT);
@@ -537,20 +638,34 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
     const bool has_up = g.row0 > 0;
     const int up_base = (w > 0 ? band : band - 1) * cols;
     const int my_base = band * cols;
-    // gx of cell (i, j) goes to px_grad[s-1][t0 + j - shift], gy to py_grad[s][t0 + j - 1]
-    R *gx_row = gxb + (long)(win.s0 + i - 1) * T1 + win.t0 - shift;
-    R *gy_row = gyb + (long)(win.s0 + i) * T + win.t0 - 1;
-    const bool gx_ok = row_ok && i > 0;
+    // gx of cell (i, j) goes to px_grad[s-1][t0 + j - shift], gy to py_grad[s][t0 + j - 1].
+    // Byte offsets of (this lane's row, column NT + lane): step e of the sweep is column
+    // NT + lane - e, so a store subtracts its step; lanes without a row (or, for gx, in
+    // the top row) get an offset that every store drops.
+    const int gx_lane = (row_ok && i > 0)
+                            ? ((win.s0 + i - 1) * T1 + win.t0 - shift + NT + lane) * kSize
+                            : kNoRow;
+    const int gy_lane = row_ok ? ((win.s0 + i) * T + win.t0 - 1 + NT + lane) * kSize : kNoRow;
+    // the gradient of the origin cell: lane NS - row0 at step NT + NS - row0
+    const int fin_lane = NS - g.row0;
+    const int fin_step = (fin_lane < kWave) ? NT + fin_lane : -1;
 
     // the seed enters as "handed left" into the first cell of the reversed sweep
     R to_below = 0, to_below2 = 0, to_left = (r == 0) ? seed : (R)0;
-    R g_origin = 0;  // gradient of this lane's cell in reversed column NT
+    R g_origin = 0;
     const bool has_down = g.nrows == kWave;
+    int seen_ready = 0;
+    R seen_seam = 0;
+    int seen_loaded[kBwdStagers];
+#pragma unroll
+    for (int l = 0; l < kBwdStagers; ++l) seen_loaded[l] = 0;
     for (int m = 0; m < g.ntiles; ++m) {
       const int gt = tile_base + m;
 #pragma unroll
       for (int l = 0; l < kBwdStagers; ++l)
-        if (!wait_for(&cnt.loaded[w * kBwdStagers + l], gt + 1)) return;
+        if (__builtin_amdgcn_readfirstlane(seen_loaded[l]) < gt + 1 &&
+            !wait_for(&cnt.loaded[w * kBwdStagers + l], gt + 1))
+          return;
       R d1q[kTileSteps], d2q[kTileSteps];
       {
         const R *d1s = base + (gt & 1) * kTileElems + lane * kTilePitch;
@@ -572,15 +687,27 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
         R handed = 0;
         if (kUp) {
           const int need = min(e0 + kChunk - shift, cols);
-          if (need > 0 && !wait_for(&cnt.ready[prev], up_base + need)) {
-            alive = false;
-            return;
+          handed = seen_seam;
+          if (need > 0 && __builtin_amdgcn_readfirstlane(seen_ready) < up_base + need) {
+            if (!wait_for(&cnt.ready[prev], up_base + need)) {
+              alive = false;
+              return;
+            }
+            const int col = e0 + lane - shift;
+            handed = (lane < kChunk && col >= 0 && col <= NT) ? up_seam[col] : (R)0;
           }
-          const int col = e0 + lane - shift;
-          if (lane < kChunk && col >= 0 && col <= NT) handed = up_seam[col];
+          // next chunk's counter, then its seam values (LDS serves a wave in order)
+          seen_ready = peek(&cnt.ready[prev]);
+          const int col = e0 + kChunk + lane - shift;
+          seen_seam = 0;
+          if (lane < kChunk && col >= 0 && col <= NT)
+            seen_seam = up_seam[col];
         }
-        R *sp = my_seam + (e0 - (kWave - 1));
-        R down[kChunk], left[kChunk];
+        if (c4 == kTileSteps / kChunk - 1) {
+#pragma unroll
+          for (int l = 0; l < kBwdStagers; ++l) seen_loaded[l] = peek(&cnt.loaded[w * kBwdStagers + l]);
+        }
+        R down[kChunk], left[kChunk], cell[kChunk];
 #pragma unroll
         for (int k = 0; k < kChunk; ++k) {
           const int kk = c4 * kChunk + k;
@@ -590,50 +717,51 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
             from_above = (lane == 0) ? first : from_above;
           }
           // cells outside the window carry d1 = d2 = 0, so nothing leaks in or out
-          const R gcell = from_above + to_left;
-          down[k] = d1q[kk] * gcell;
-          left[k] = d2q[kk] * gcell;
-          const int c63 = e0 + k - (kWave - 1);  // reversed column of the seam lane
-          if (kEdge) {
-            const int c = e0 + k - lane;
-            g_origin = (c == NT) ? gcell : g_origin;
-            if (kDown && c63 >= 0 && c63 <= NT && lane == kWave - 1) sp[k] = down[k];
-          } else {
-            if (kDown && lane == kWave - 1) sp[k] = down[k];
-          }
+          cell[k] = from_above + to_left;
+          down[k] = d1q[kk] * cell[k];
+          left[k] = d2q[kk] * cell[k];
           to_below2 = to_below;
           to_below = down[k];
           to_left = left[k];
         }
-        // write-out in groups of four steps: columns j0-3 .. j0, one 16-byte store per
-        // array when the whole group lies inside the window, single stores otherwise
+        const int kf = fin_step - e0;  // wave-uniform
+        if ((unsigned)kf < (unsigned)kChunk) {
 #pragma unroll
-        for (int q4 = 0; q4 < kChunk; q4 += 4) {
-          const int c0 = e0 + q4 - lane;     // reversed column of the group's first step
-          const int j0 = NT - c0;            // its column; the group covers j0-3 .. j0
-          const bool whole = !kEdge || (c0 >= 0 && j0 - 3 >= 1);
-          if (whole && gx_ok) {
-            store4(gx_row + (j0 - 3), down[q4 + 3], down[q4 + 2], down[q4 + 1], down[q4]);
-          } else if (gx_ok) {
+          for (int k = 0; k < kChunk; ++k)
+            if (k == kf) g_origin = cell[k];
+        }
+        // seam: the last lane's reversed columns e0 - 63 ... (the pads take what falls
+        // outside)
+        if (kDown && e0 + kChunk > kWave - 1) {
+          if (lane == kWave - 1) {
+            R *sp = my_seam + (e0 - (kWave - 1));
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-              const int j = j0 - k;
-              if (c0 + k >= 0 && j >= 0 && (j > 0 || !kModified)) gx_row[j] = down[q4 + k];
-            }
-          }
-          if (whole && row_ok) {
-            store4(gy_row + (j0 - 3), left[q4 + 3], left[q4 + 2], left[q4 + 1], left[q4]);
-          } else if (row_ok) {
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-              const int j = j0 - k;
-              if (c0 + k >= 0 && j > 0) gy_row[j] = left[q4 + k];
-            }
+            for (int k = 0; k < kChunk; ++k) sp[k] = down[k];
+            const int done = max(0, min(e0 + kChunk - (kWave - 1), cols));
+            publish(&cnt.ready[w], my_base + done);
           }
         }
-        if (kDown && lane == kWave - 1) {
-          const int done = max(0, min(e0 + kChunk - (kWave - 1), cols));
-          publish(&cnt.ready[w], my_base + done);
+        // write-out: a group of four steps is the columns j-3 .. j of its first step
+        const int gx_first = gx_lane - e0 * kSize, gy_first = gy_lane - e0 * kSize;
+        if (!kEdge) {
+#pragma unroll
+          for (int q4 = 0; q4 < kChunk; q4 += 4) {
+            put4(gx_rsrc, gx_first - (q4 + 3) * kSize, down[q4 + 3], down[q4 + 2], down[q4 + 1],
+                 down[q4]);
+            put4(gy_rsrc, gy_first - (q4 + 3) * kSize, left[q4 + 3], left[q4 + 2], left[q4 + 1],
+                 left[q4]);
+          }
+        } else {
+          const int j0 = NT - e0 + lane;  // column of the chunk's first step
+          constexpr int kMinX = kModified ? 1 : 0;
+#pragma unroll
+          for (int k = 0; k < kChunk; ++k) {
+            // inside the window: column <= NT (the lane has started) and >= its first
+            const bool okx = (unsigned)(j0 - k - kMinX) < (unsigned)(NT + 1 - kMinX);
+            const bool oky = (unsigned)(j0 - k - 1) < (unsigned)NT;
+            put1(gx_rsrc, (okx ? gx_first : kDropped) - k * kSize, down[k]);
+            put1(gy_rsrc, (oky ? gy_first : kDropped) - k * kSize, left[k]);
+          }
         }
       };
       auto tile = [&](auto up_c, auto down_c) __attribute__((always_inline)) {
@@ -641,10 +769,9 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
         for (int c4 = 0; c4 < kTileSteps / kChunk; ++c4) {
           const int e0 = m * kTileSteps + c4 * kChunk;
           if (e0 < g.nsteps && alive) {
-            // interior: every lane of a full wave is inside the window, below the
-            // top row and right of column 0 for all of the chunk's steps
-            const bool interior = g.nrows == kWave && g.row0 + kWave - 1 < NS &&
-                                  e0 >= kWave - 1 && e0 + kChunk <= NT;
+            // interior: every lane that has a row has started and stays right of
+            // column 0 for all of the chunk's steps
+            const bool interior = e0 >= g.nrows - 1 && e0 + kChunk <= NT;
             if (interior)
               chunk(up_c, down_c, std::false_type{}, c4, e0);
             else
@@ -665,7 +792,7 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
       }
       if (!alive) return;
     }
-    if (row_ok && r == NS && overwrite_ans_grad && ans_grad) ans_grad[b] = g_origin;
+    if (lane == fin_lane && overwrite_ans_grad && ans_grad) ans_grad[b] = g_origin;
     tile_base += g.ntiles;
   }
 }
@@ -677,7 +804,7 @@ int pick_sweep_waves(int S, int T, size_t elem, int arrays) {
   int n = (S + 1 + kWave - 1) / kWave;
   n = n < 1 ? 1 : (n > kMaxSweep ? kMaxSweep : n);
   auto bytes = [&](int k) {
-    return (size_t)k * ((size_t)(T + 1) + (size_t)arrays * 2 * kTileElems) * elem;
+    return (size_t)k * ((size_t)(T + 1 + 2 * kSeamPad) + (size_t)arrays * 2 * kTileElems) * elem;
   };
   while (n > 1 && bytes(n) > kLdsBudget) --n;
   return n;
@@ -689,8 +816,10 @@ int forward_impl(const R *px, const R *py, const int64_t *boundary, R *p, R *ans
   if (B < 0 || S < 0 || T < 0) return fail(FRNNT_EINVAL, "mi_forward: negative size");
   if (B == 0) return FRNNT_OK;
   if (!px || !py || !p || !ans) return fail(FRNNT_EINVAL, "mi_forward: null pointer");
+  if ((size_t)(S + 1) * (T + 1) * sizeof(R) >= ((size_t)1 << 30))
+    return fail(FRNNT_ELIMIT, "mi_forward: one utterance's lattice exceeds 1 GiB");
   const int n = pick_sweep_waves(S, T, sizeof(R), 2);
-  const size_t lds = (size_t)n * ((size_t)(T + 1) + 4 * kTileElems) * sizeof(R);
+  const size_t lds = (size_t)n * ((size_t)(T + 1 + 2 * kSeamPad) + 4 * kTileElems) * sizeof(R);
   if (lds > kLdsBudget)
     return fail(FRNNT_ELIMIT, "mi_forward: T=%d needs %zu bytes of LDS", T, lds);
   auto kernel = n <= 2 ? (modified ? mi_forward_kernel<R, true, 2> : mi_forward_kernel<R, false, 2>)
@@ -714,8 +843,10 @@ int backward_impl(const R *px, const R *py, const int64_t *boundary, const R *p,
   if (B == 0) return FRNNT_OK;
   if (!px || !p || !px_grad || !py_grad)
     return fail(FRNNT_EINVAL, "mi_backward: null pointer");
+  if ((size_t)(S + 1) * (T + 1) * sizeof(R) >= ((size_t)1 << 30))
+    return fail(FRNNT_ELIMIT, "mi_backward: one utterance's lattice exceeds 1 GiB");
   const int n = pick_sweep_waves(S, T, sizeof(R), 2);
-  const size_t lds = (size_t)n * ((size_t)(T + 1) + 4 * kTileElems) * sizeof(R);
+  const size_t lds = (size_t)n * ((size_t)(T + 1 + 2 * kSeamPad) + 4 * kTileElems) * sizeof(R);
   if (lds > kLdsBudget)
     return fail(FRNNT_ELIMIT, "mi_backward: T=%d needs %zu bytes of LDS", T, lds);
   auto kernel = n <= 2 ? (modified ? mi_backward_kernel<R, true, 2> : mi_backward_kernel<R, false, 2>)
