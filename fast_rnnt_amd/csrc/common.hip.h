@@ -82,6 +82,33 @@ __device__ __forceinline__ double from_lane_below_zero(double v) {
   return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
 }
 
+// Shift right by one in which lane 0 keeps the value it holds in `first` (a DPP move
+// leaves lanes without a source lane at their old contents).
+__device__ __forceinline__ float from_lane_below_or(float v, float first) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(first), __float_as_int(v),
+                                                    0x138, 0xf, 0xf, false));
+}
+__device__ __forceinline__ double from_lane_below_or(double v, double first) {
+  const long long vi = __double_as_longlong(v), fi = __double_as_longlong(first);
+  const int lo = __builtin_amdgcn_update_dpp((int)(fi & 0xffffffffLL), (int)(vi & 0xffffffffLL),
+                                             0x138, 0xf, 0xf, false);
+  const int hi = __builtin_amdgcn_update_dpp((int)(fi >> 32), (int)(vi >> 32), 0x138, 0xf, 0xf,
+                                             false);
+  return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+
+// Value held by lane+1 (whole-wave shift left by one, DPP wave_shl:1); lane 63 receives 0.
+__device__ __forceinline__ float from_lane_above(float v) {
+  return __int_as_float(
+      __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x130, 0xf, 0xf, true));
+}
+__device__ __forceinline__ double from_lane_above(double v) {
+  const long long vi = __double_as_longlong(v);
+  const int lo = __builtin_amdgcn_update_dpp(0, (int)(vi & 0xffffffffLL), 0x130, 0xf, 0xf, true);
+  const int hi = __builtin_amdgcn_update_dpp(0, (int)(vi >> 32), 0x130, 0xf, 0xf, true);
+  return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+
 // Broadcast of lane `src`'s value (src wave-uniform).
 __device__ __forceinline__ float lane_value(float v, int src) {
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src));

@@ -31,7 +31,7 @@ namespace {
 constexpr int kMaxSweep = 4;           // sweep waves per workgroup
 constexpr int kChunk = 8;              // steps per seam hand-over
 constexpr int kTileSteps = 32;         // steps per staged tile
-constexpr int kTilePitch = kTileSteps + 1;
+constexpr int kTilePitch = kTileSteps + 4;  // rows start 16-byte aligned and spread over the banks
 constexpr int kTileElems = kWave * kTilePitch;
 constexpr int kSeamPad = kChunk;        // slack on either side of a seam row, so that a whole
                                        // chunk of seam values is written without bounds tests
@@ -136,6 +136,20 @@ __device__ __forceinline__ void put4(__amdgpu_buffer_rsrc_t rs, int off, double 
       intx4{(int)cb, (int)(cb >> 32), (int)db, (int)(db >> 32)}, rs, off == kDropped ? off : off + 16,
       0, 0);
 }
+// One lane's kTileSteps staged values, 16 bytes per LDS read.
+template <typename R>
+__device__ __forceinline__ void pull_row(R (&dst)[kTileSteps], const R *src) {
+  constexpr int kPer = 16 / (int)sizeof(R);
+  typedef R Piece __attribute__((ext_vector_type(kPer)));
+  const Piece *s = reinterpret_cast<const Piece *>(src);
+#pragma unroll
+  for (int i = 0; i < kTileSteps / kPer; ++i) {
+    const Piece v = s[i];
+#pragma unroll
+    for (int e = 0; e < kPer; ++e) dst[i * kPer + e] = v[e];
+  }
+}
+
 struct Counters {
   int ready[kMaxSweep];                   // seam columns published by sweep wave w
   int consumed[kMaxSweep];                // tiles sweep wave w has finished
@@ -171,7 +185,7 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
 
   const int b = blockIdx.x;
   const int nsweep = blockDim.x / (kWave * (1 + kFwdStagers));
-  const int wave = threadIdx.x / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // in a scalar register
   const int lane = threadIdx.x % kWave;
   const int T1 = kModified ? T : T + 1;
   const int TP = T + 1;
@@ -193,7 +207,7 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
   R *pb = p + (size_t)b * (S + 1) * TP;
   const __amdgpu_buffer_rsrc_t p_rsrc = buffer_of(pb, (size_t)(S + 1) * TP);
   R *seam = reinterpret_cast<R *>(dyn_lds);
-  const int seam_pitch = TP + 2 * kSeamPad;
+  const int seam_pitch = (TP + 2 * kSeamPad + 3) & ~3;  // keeps the tiles 16-byte aligned
   R *tiles = seam + (size_t)nsweep * seam_pitch;  // [nsweep][2 arrays][2 buffers][kTileElems]
   const int band_rows = kWave * nsweep;
 
@@ -299,13 +313,8 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
       // the staging waves may refill the buffer
       R xq[kTileSteps], yq[kTileSteps];
       {
-        const R *xs = xt + (gt & 1) * kTileElems + lane * kTilePitch;
-        const R *ys = yt + (gt & 1) * kTileElems + lane * kTilePitch;
-#pragma unroll
-        for (int kk = 0; kk < kTileSteps; ++kk) {
-          xq[kk] = xs[kk];
-          yq[kk] = ys[kk];
-        }
+        pull_row(xq, xt + (gt & 1) * kTileElems + lane * kTilePitch);
+        pull_row(yq, yt + (gt & 1) * kTileElems + lane * kTilePitch);
       }
       if (lane == 0) publish(&cnt.consumed[w], gt + 1);
 
@@ -347,10 +356,13 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
           const int kk = c4 * kChunk + k;
           // lane 0 of a wave without a seam owns lattice row 0, whose x is -inf,
           // so the 0 it receives from the shift never matters
-          R up = from_lane_below_zero(kModified ? own2 : own);
+          R up;
           if (kUp) {
-            const R first = lane_value(handed, k);
-            up = (lane == 0) ? first : up;
+            // lane 0 takes the seam value of this step, which then moves on
+            up = from_lane_below_or(kModified ? own2 : own, handed);
+            handed = from_lane_above(handed);
+          } else {
+            up = from_lane_below_zero(kModified ? own2 : own);
           }
           const R v = chain_log_add(up + xq[kk], own + yq[kk]);
           vals[k] = v;
@@ -441,7 +453,7 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
   const int b = blockIdx.x;
   const int nsweep = blockDim.x / (kWave * (1 + kBwdStagers));
   const int nwaves = blockDim.x / kWave;
-  const int wave = threadIdx.x / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // in a scalar register
   const int lane = threadIdx.x % kWave;
   const int T1 = kModified ? T : T + 1;
   const int TP = T + 1;
@@ -506,7 +518,7 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
   const R *pxb = px + (size_t)b * S * T1;
   const R *pb = p + (size_t)b * (S + 1) * TP;
   R *seam = reinterpret_cast<R *>(dyn_lds);
-  const int seam_pitch = TP + 2 * kSeamPad;
+  const int seam_pitch = (TP + 2 * kSeamPad + 3) & ~3;  // keeps the tiles 16-byte aligned
   R *tiles = seam + (size_t)nsweep * seam_pitch;  // per sweep wave: d1[2], d2[2] tiles
   const int band_rows = kWave * nsweep;
 
@@ -668,13 +680,8 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
           return;
       R d1q[kTileSteps], d2q[kTileSteps];
       {
-        const R *d1s = base + (gt & 1) * kTileElems + lane * kTilePitch;
-        const R *d2s = base + (2 + (gt & 1)) * kTileElems + lane * kTilePitch;
-#pragma unroll
-        for (int kk = 0; kk < kTileSteps; ++kk) {
-          d1q[kk] = d1s[kk];
-          d2q[kk] = d2s[kk];
-        }
+        pull_row(d1q, base + (gt & 1) * kTileElems + lane * kTilePitch);
+        pull_row(d2q, base + (2 + (gt & 1)) * kTileElems + lane * kTilePitch);
       }
       if (lane == 0) publish(&cnt.consumed[w], gt + 1);
 
@@ -711,10 +718,12 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
 #pragma unroll
         for (int k = 0; k < kChunk; ++k) {
           const int kk = c4 * kChunk + k;
-          R from_above = from_lane_below_zero(kModified ? to_below2 : to_below);
+          R from_above;
           if (kUp) {
-            const R first = lane_value(handed, k);
-            from_above = (lane == 0) ? first : from_above;
+            from_above = from_lane_below_or(kModified ? to_below2 : to_below, handed);
+            handed = from_lane_above(handed);
+          } else {
+            from_above = from_lane_below_zero(kModified ? to_below2 : to_below);
           }
           // cells outside the window carry d1 = d2 = 0, so nothing leaks in or out
           cell[k] = from_above + to_left;
@@ -804,7 +813,7 @@ int pick_sweep_waves(int S, int T, size_t elem, int arrays) {
   int n = (S + 1 + kWave - 1) / kWave;
   n = n < 1 ? 1 : (n > kMaxSweep ? kMaxSweep : n);
   auto bytes = [&](int k) {
-    return (size_t)k * ((size_t)(T + 1 + 2 * kSeamPad) + (size_t)arrays * 2 * kTileElems) * elem;
+    return (size_t)k * ((size_t)((T + 1 + 2 * kSeamPad + 3) & ~3) + (size_t)arrays * 2 * kTileElems) * elem;
   };
   while (n > 1 && bytes(n) > kLdsBudget) --n;
   return n;
@@ -819,7 +828,7 @@ int forward_impl(const R *px, const R *py, const int64_t *boundary, R *p, R *ans
   if ((size_t)(S + 1) * (T + 1) * sizeof(R) >= ((size_t)1 << 30))
     return fail(FRNNT_ELIMIT, "mi_forward: one utterance's lattice exceeds 1 GiB");
   const int n = pick_sweep_waves(S, T, sizeof(R), 2);
-  const size_t lds = (size_t)n * ((size_t)(T + 1 + 2 * kSeamPad) + 4 * kTileElems) * sizeof(R);
+  const size_t lds = (size_t)n * ((size_t)((T + 1 + 2 * kSeamPad + 3) & ~3) + 4 * kTileElems) * sizeof(R);
   if (lds > kLdsBudget)
     return fail(FRNNT_ELIMIT, "mi_forward: T=%d needs %zu bytes of LDS", T, lds);
   auto kernel = n <= 2 ? (modified ? mi_forward_kernel<R, true, 2> : mi_forward_kernel<R, false, 2>)
@@ -846,7 +855,7 @@ int backward_impl(const R *px, const R *py, const int64_t *boundary, const R *p,
   if ((size_t)(S + 1) * (T + 1) * sizeof(R) >= ((size_t)1 << 30))
     return fail(FRNNT_ELIMIT, "mi_backward: one utterance's lattice exceeds 1 GiB");
   const int n = pick_sweep_waves(S, T, sizeof(R), 2);
-  const size_t lds = (size_t)n * ((size_t)(T + 1 + 2 * kSeamPad) + 4 * kTileElems) * sizeof(R);
+  const size_t lds = (size_t)n * ((size_t)((T + 1 + 2 * kSeamPad + 3) & ~3) + 4 * kTileElems) * sizeof(R);
   if (lds > kLdsBudget)
     return fail(FRNNT_ELIMIT, "mi_backward: T=%d needs %zu bytes of LDS", T, lds);
   auto kernel = n <= 2 ? (modified ? mi_backward_kernel<R, true, 2> : mi_backward_kernel<R, false, 2>)
