@@ -119,6 +119,15 @@ __device__ __forceinline__ void put1(__amdgpu_buffer_rsrc_t rs, int off, double 
   const long long bits = __double_as_longlong(v);
   __builtin_amdgcn_raw_buffer_store_b64(intx2{(int)bits, (int)(bits >> 32)}, rs, off, 0, 0);
 }
+// Range-checked load: an offset outside the resource (negative ones included, they are
+// huge when read as unsigned) reads as 0 and touches no memory.
+__device__ __forceinline__ float get1(__amdgpu_buffer_rsrc_t rs, int off, float) {
+  return __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(rs, off, 0, 0));
+}
+__device__ __forceinline__ double get1(__amdgpu_buffer_rsrc_t rs, int off, double) {
+  const intx2 v = __builtin_amdgcn_raw_buffer_load_b64(rs, off, 0, 0);
+  return __longlong_as_double(((long long)v[1] << 32) | (unsigned int)v[0]);
+}
 // four consecutive elements (the address only needs element alignment)
 __device__ __forceinline__ void put4(__amdgpu_buffer_rsrc_t rs, int off, float a, float b, float c,
                                      float d) {
@@ -224,22 +233,26 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
     };
     // Global fetches of a tile go to registers and do not need the LDS buffer, so
     // the fetch of tile m+1 is issued before this wave waits for the buffer of tile
-    // m to be released: the memory latency overlaps the sweep.
+    // m to be released: the memory latency overlaps the sweep.  The loads are
+    // range-checked and otherwise unconditional: what a lane reads for cells outside
+    // the window is either replaced at staging time (row 0, column 0: the -inf that
+    // closes the lattice) or never reaches a cell of the window (columns before a
+    // row's start or beyond its end only feed cells at least as far out).
+    const __amdgpu_buffer_rsrc_t px_rsrc = buffer_of(const_cast<R *>(pxb), (size_t)S * T1);
+    const __amdgpu_buffer_rsrc_t py_rsrc = buffer_of(const_cast<R *>(pyb), (size_t)(S + 1) * T);
+    constexpr int kStep = 2 * kFwdStagers;
+    constexpr int kSize = (int)sizeof(R);
+    const int r_first = 2 * l + half;
     auto fetch = [&](Staged &in, const Band &g, int m) {
+      const int s_first = win.s0 + g.row0 + r_first;
+      const int j_first = m * kTileSteps + q - r_first;
+      const int x0 = ((s_first - 1) * T1 + win.t0 + j_first - shift) * kSize;
+      const int y0 = (s_first * T + win.t0 + j_first - 1) * kSize;
 #pragma unroll
       for (int u = 0; u < kRows; ++u) {
-        const int r = 2 * l + half + 2 * kFwdStagers * u;
-        const int i = g.row0 + r, s = win.s0 + i;
-        const int j = m * kTileSteps + q - r;
-        const int jj = j - shift;
-        R x = ninf, y = ninf;
-        if (r < g.nrows) {
-          if (i >= 1 && jj >= 0 && j <= NT) x = pxb[(long)(s - 1) * T1 + win.t0 + jj];
-          if (j >= 1 && j <= NT) y = pyb[(long)s * T + win.t0 + j - 1];
-          if (i == 0 && j == 0) y = 0;
-        }
-        in.x[u] = x;
-        in.y[u] = y;
+        // kStep rows further up: as many rows down in memory, as many columns left
+        in.x[u] = get1(px_rsrc, x0 + u * (kStep * (T1 - 1) * kSize), R());
+        in.y[u] = get1(py_rsrc, y0 + u * (kStep * (T - 1) * kSize), R());
       }
     };
     int tile_base = 0;
@@ -253,13 +266,23 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
         if (m + 1 < g.ntiles) fetch(nxt, g, m + 1);
         if (gt >= 2 && !wait_for(&cnt.consumed[w], gt - 1)) return;
         R *xdst = xt + (gt & 1) * kTileElems, *ydst = yt + (gt & 1) * kTileElems;
+        // only the first tiles hold a column 0 (local step = row), and only the first
+        // band holds row 0
+        const bool starts = m * kTileSteps <= kWave - 1 + shift;
 #pragma unroll
         for (int u = 0; u < kRows; ++u) {
-          const int r = 2 * l + half + 2 * kFwdStagers * u;
-          if (r < g.nrows) {
-            xdst[r * kTilePitch + q] = cur.x[u];
-            ydst[r * kTilePitch + q] = cur.y[u];
+          const int r = r_first + kStep * u;
+          if (r >= kWave) continue;
+          R x = cur.x[u], y = cur.y[u];
+          const int i = g.row0 + r;
+          if (starts) {
+            const int j = m * kTileSteps + q - r;
+            if (j <= 0) y = (j == 0 && i == 0) ? (R)0 : ninf;
+            if (j < shift) x = ninf;
           }
+          if (u == 0 && i == 0) x = ninf;
+          xdst[r * kTilePitch + q] = x;
+          ydst[r * kTilePitch + q] = y;
         }
         if (lane == 0) publish(&cnt.loaded[w * kFwdStagers + l], gt + 1);
         cur = nxt;
@@ -533,36 +556,28 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
     struct Staged {
       R here[kRows], below[kRows], x[kRows];
     };
-    // global fetches of tile m+1 are issued (into registers) before this wave waits
-    // for the LDS buffers of tile m, so their latency overlaps the sweep
+    // Global fetches of tile m+1 are issued (into registers) before this wave waits
+    // for the LDS buffers of tile m, so their latency overlaps the sweep.  The loads
+    // are range-checked and otherwise unconditional; staging replaces what was read
+    // for cells outside the window.
+    const __amdgpu_buffer_rsrc_t p_rsrc = buffer_of(const_cast<R *>(pb), (size_t)(S + 1) * TP);
+    const __amdgpu_buffer_rsrc_t px_rsrc = buffer_of(const_cast<R *>(pxb), (size_t)S * T1);
+    constexpr int kStep = 2 * kBwdStagers;
+    constexpr int kSize = (int)sizeof(R);
+    const int r_first = 2 * l + half;
     auto fetch = [&](Staged &in, const Band &g, int m) {
-      const bool inner_tile = g.nrows == kWave && g.row0 + kWave - 1 < NS &&
-                              m * kTileSteps - (kWave - 1) >= 0 &&
-                              m * kTileSteps + kTileSteps - 1 <= NT - 1;
-      // element offsets of row u = 0; each further u is 2*kBwdStagers rows up the
-      // reversed lattice, i.e. that many rows down in memory and as many columns right
-      const int r_first = 2 * l + half;
+      // element offsets of row u = 0; each further u is kStep rows up the reversed
+      // lattice, i.e. that many rows down in memory and as many columns right
       const int s_first = win.s0 + NS - (g.row0 + r_first);
       const int j_first = NT - (m * kTileSteps + q - r_first);
-      const int below0 = (s_first - 1) * TP + win.t0 + j_first - shift;
-      const int x0 = (s_first - 1) * T1 + win.t0 + j_first - shift;
-      const int here0 = s_first * TP + win.t0 + j_first;
-      constexpr int kStep = 2 * kBwdStagers;
+      const int below0 = ((s_first - 1) * TP + win.t0 + j_first - shift) * kSize;
+      const int x0 = ((s_first - 1) * T1 + win.t0 + j_first - shift) * kSize;
+      const int here0 = (s_first * TP + win.t0 + j_first) * kSize;
 #pragma unroll
       for (int u = 0; u < kRows; ++u) {
-        const int r = r_first + kStep * u;
-        bool ok = r < g.nrows;
-        if (!inner_tile) {
-          const int i = NS - (g.row0 + r);
-          const int c = m * kTileSteps + q - r;
-          ok = ok && c >= 0 && c <= NT && i > 0 && NT - c > 0;
-        }
-        in.here[u] = in.below[u] = in.x[u] = 0;
-        if (ok) {
-          in.below[u] = pb[below0 - u * kStep * (TP - 1)];
-          in.x[u] = pxb[x0 - u * kStep * (T1 - 1)];
-          in.here[u] = pb[here0 - u * kStep * (TP - 1)];
-        }
+        in.below[u] = get1(p_rsrc, below0 - u * (kStep * (TP - 1) * kSize), R());
+        in.x[u] = get1(px_rsrc, x0 - u * (kStep * (T1 - 1) * kSize), R());
+        in.here[u] = get1(p_rsrc, here0 - u * (kStep * (TP - 1) * kSize), R());
       }
     };
     int tile_base = 0;
@@ -576,51 +591,43 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
         if (m + 1 < g.ntiles) fetch(nxt, g, m + 1);
         if (gt >= 2 && !wait_for(&cnt.consumed[w], gt - 1)) return;
         R *d1dst = base + (gt & 1) * kTileElems, *d2dst = base + (2 + (gt & 1)) * kTileElems;
-        // A tile of a full wave whose 64 x 32 cells all lie strictly inside the window
-        // (below the top row, right of column 0) needs none of the edge cases.
-        const bool inner_tile = g.nrows == kWave && g.row0 + kWave - 1 < NS &&
-                                m * kTileSteps - (kWave - 1) >= 0 &&
-                                m * kTileSteps + kTileSteps - 1 <= NT - 1;
-        if (inner_tile) {
+        // Which of the window's borders cross this tile (wave-uniform): reversed column 0,
+        // where rows start (local step = row); column 0, where they end; the top row.
+        const bool starts = m * kTileSteps <= kWave - 1;
+        const bool ends = m * kTileSteps + kTileSteps - 1 >= NT;
+        const bool has_top = g.row0 + kWave - 1 >= NS;
 #pragma unroll
-          for (int u = 0; u < kRows; ++u) {
-            const int r = 2 * l + half + 2 * kBwdStagers * u;
-            if (r >= kWave) continue;
-            const R term1 = cur.below[u] + cur.x[u];
-            R total = cur.here[u];
-            if (total - total != 0) total = 0;
-            R d1 = Num<R>::exp_(term1 - total);
-            R d2 = (R)1 - d1;
-            if (d1 - d1 != 0) d1 = d2 = 0;
-            d1dst[r * kTilePitch + q] = d1;
-            d2dst[r * kTilePitch + q] = d2;
-          }
-        } else {
-#pragma unroll
-          for (int u = 0; u < kRows; ++u) {
-            const int r = 2 * l + half + 2 * kBwdStagers * u;
-            const int i = NS - (g.row0 + r);
-            const int c = m * kTileSteps + q - r;
+        for (int u = 0; u < kRows; ++u) {
+          const int r = r_first + kStep * u;
+          if (r >= kWave) continue;
+          // mutual_information_cpu.cu:196-212
+          const R term1 = cur.below[u] + cur.x[u];
+          R total = cur.here[u];
+          if (total - total != 0) total = 0;
+          R d1 = Num<R>::exp_(term1 - total);
+          R d2 = (R)1 - d1;
+          if (d1 - d1 != 0) d1 = d2 = 0;
+          const int c = m * kTileSteps + q - r;
+          if (starts && c < 0) d1 = d2 = 0;
+          if (ends) {
+            // column 0 hands everything down (mutual_information_cpu.cu:219-226), or
+            // nothing at all in the modified lattice; beyond it nothing is defined
             const int j = NT - c;
-            if (r >= g.nrows) continue;
-            R d1 = 0, d2 = 0;
-            if (c >= 0 && c <= NT) {
-              if (i > 0 && j > 0) {
-                const R term1 = cur.below[u] + cur.x[u];
-                R total = cur.here[u];
-                if (total - total != 0) total = 0;
-                d1 = Num<R>::exp_(term1 - total);
-                d2 = (R)1 - d1;
-                if (d1 - d1 != 0) d1 = d2 = 0;
-              } else if (i == 0 && j > 0) {
-                d2 = 1;
-              } else if (i > 0 && j == 0 && !kModified) {
-                d1 = 1;
-              }
+            if (j <= 0) {
+              d1 = (j == 0 && !kModified) ? (R)1 : (R)0;
+              d2 = 0;
             }
-            d1dst[r * kTilePitch + q] = d1;
-            d2dst[r * kTilePitch + q] = d2;
           }
+          if (has_top) {
+            // the top row hands everything left (mutual_information_cpu.cu:228-235)
+            const int i = NS - (g.row0 + r);
+            if (i <= 0) {
+              d1 = 0;
+              d2 = (i == 0 && c >= 0 && c < NT) ? (R)1 : (R)0;
+            }
+          }
+          d1dst[r * kTilePitch + q] = d1;
+          d2dst[r * kTilePitch + q] = d2;
         }
         // every lane's LDS writes precede the release by lane 0 of the same wave
         if (lane == 0) publish(my_loaded, gt + 1);
