@@ -20,6 +20,9 @@ constexpr int kWave = 64;
 char *error_buffer();
 int fail(int code, const char *fmt, ...);
 int check_launch(const char *what);
+// Makes `bytes` of dynamic LDS available to `kernel` on the current device (needed
+// above 64 KB); remembers what it has granted, so the runtime is asked once.
+bool allow_lds(const void *kernel, size_t bytes);
 
 // ---- device side -----------------------------------------------------------------
 template <typename R>

@@ -841,9 +841,7 @@ int forward_impl(const R *px, const R *py, const int64_t *boundary, R *p, R *ans
   auto kernel = n <= 2 ? (modified ? mi_forward_kernel<R, true, 2> : mi_forward_kernel<R, false, 2>)
                        : (modified ? mi_forward_kernel<R, true, kMaxSweep>
                                    : mi_forward_kernel<R, false, kMaxSweep>);
-  if (lds > 64 * 1024 &&
-      hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+  if (!allow_lds(reinterpret_cast<const void *>(kernel), lds))
     return check_launch("mi_forward: hipFuncSetAttribute");
   hipLaunchKernelGGL(kernel, dim3(B), dim3(n * (1 + kFwdStagers) * kWave), lds,
                      static_cast<hipStream_t>(stream), px, py, boundary, p, ans, S, T);
@@ -868,9 +866,7 @@ int backward_impl(const R *px, const R *py, const int64_t *boundary, const R *p,
   auto kernel = n <= 2 ? (modified ? mi_backward_kernel<R, true, 2> : mi_backward_kernel<R, false, 2>)
                        : (modified ? mi_backward_kernel<R, true, kMaxSweep>
                                    : mi_backward_kernel<R, false, kMaxSweep>);
-  if (lds > 64 * 1024 &&
-      hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+  if (!allow_lds(reinterpret_cast<const void *>(kernel), lds))
     return check_launch("mi_backward: hipFuncSetAttribute");
   hipLaunchKernelGGL(kernel, dim3(B), dim3(n * (1 + kBwdStagers) * kWave), lds,
                      static_cast<hipStream_t>(stream), px, boundary, p, ans_grad, px_grad,

@@ -138,9 +138,7 @@ int ranges_impl(const R *px_grad, const R *py_grad, const int64_t *boundary, int
   const size_t lds = (size_t)T * sizeof(int);
   if (lds > 150 * 1024) return fail(FRNNT_ELIMIT, "prune_ranges: T=%d exceeds the LDS table", T);
   auto kernel = prune_ranges_kernel<R>;
-  if (lds > 64 * 1024 &&
-      hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+  if (!allow_lds(reinterpret_cast<const void *>(kernel), lds))
     return check_launch("prune_ranges: hipFuncSetAttribute");
   hipLaunchKernelGGL(kernel, dim3(B), dim3(kWave), lds, static_cast<hipStream_t>(stream), px_grad,
                      py_grad, boundary, ranges, S, T, modified ? T : T + 1, s_range);

@@ -366,6 +366,24 @@ __global__ void __launch_bounds__(256)
 }
 
 
+// four consecutive floats at any element-aligned address (global memory takes
+// unaligned 16-byte accesses); `valid` (0..4) leading elements are read, the rest is 0
+typedef float floatx4u __attribute__((ext_vector_type(4), aligned(4)));
+template <bool kVec>
+__device__ __forceinline__ dgemm::floatx4 load4_guarded(const float *base, int off, int valid,
+                                                        float fill = 0.f) {
+  dgemm::floatx4 r = {fill, fill, fill, fill};
+  if (kVec && valid >= 4) {
+    const floatx4u t = *reinterpret_cast<const floatx4u *>(base + off);
+    r[0] = t[0], r[1] = t[1], r[2] = t[2], r[3] = t[3];
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i < valid) r[i] = base[off + i];
+  }
+  return r;
+}
+
 // ---- fp32: register-direct MFMA kernels (direct_gemm.hip.h) ------------------------
 constexpr int kFwdWaves = 4;  // K split of the forward normalizer GEMM
 constexpr int kLmWaves = 4;   // K split of the lm-gradient GEMM
@@ -492,6 +510,294 @@ __global__ void __launch_bounds__(kFwdWaves *kWave)
   // the extra column of the regular lattice: nothing can be emitted after the last frame
   if (rnnt_type == kRegular && t_tile == 0 && tid < kBM && s_tile + tid < S)
     pxb[(long)(s_tile + tid) * T1 + T] = ninf;
+}
+
+// Normalizer GEMM, wave-private LDS transposition.  Both operands are k-contiguous
+// ([rows][C]), the matrix cores want one row per lane.  Letting every lane fetch its
+// own row costs one cache-line lookup per lane and instruction, which is what bounds
+// that form; here a wave fetches a 128-row x 32-k slab with 16 coalesced 16-byte loads
+// (8 lanes per row), applies exp(x - max) in registers, writes the slab to its OWN
+// LDS region (pitch 33, conflict-free for the row-per-lane reads that follow) and
+// feeds the matrix cores from there.  The eight waves of a workgroup split k; they
+// never wait for each other in the loop (a wave's LDS writes and reads are served in
+// program order), only once at the end, when the partial sums meet.  Two waves share
+// a SIMD, so one wave's exp / LDS-write phase runs under the other's MFMA phase.
+// A workgroup covers 96 lattice rows (three 32-row tiles) x 32 frames, so at
+// S+1 <= 96 the lm operand is fetched once per 32 frames.
+constexpr int kPanS = 96;                 // lattice rows per workgroup
+constexpr int kPanT = 32;                 // frames per workgroup
+constexpr int kPanRows = kPanS + kPanT;   // rows of a slab: lm rows, then am rows
+constexpr int kPanK = 32;                 // k per slab
+constexpr int kPanPitch = kPanK + 1;
+constexpr int kPanSlab = kPanRows * kPanPitch;  // floats per slab
+constexpr int kPanWaves = 8;
+constexpr int kPanThreads = kPanWaves * kWave;
+constexpr size_t kPanLdsBytes = (size_t)kPanWaves * kPanSlab * sizeof(float);
+constexpr int kPanItems = (kPanS * kPanT / 4 + kPanThreads - 1) / kPanThreads;  // 16-byte outputs per thread
+
+template <bool kVec>
+__global__ void __launch_bounds__(kPanThreads)
+    simple_fwd_panel_kernel(const float *__restrict__ lm, const float *__restrict__ am,
+                            const int64_t *__restrict__ symbols,
+                            const int64_t *__restrict__ boundary,
+                            float *__restrict__ lm_max, float *__restrict__ am_max,
+                            float *__restrict__ px, float *__restrict__ py,
+                            float *__restrict__ norm_raw, int B, int S, int T, int C, int term,
+                            int rnnt_type) {
+  using namespace dgemm;
+  extern __shared__ float pan_lds[];
+  __shared__ float wave_max[kPanWaves][kPanRows];  // row maxima over each wave's share of k
+  __shared__ float slab_max[kPanRows];             // row maxima
+  __shared__ float row_term[kPanS], row_sym[kPanS], row_max[kPanS];  // lm[s,term], lm[s,sym[s]], lm_max[s]
+  __shared__ int row_symbol[kPanS];
+  __shared__ float col_term[kPanT], col_max[kPanT];                  // am[t,term], am_max[t]
+  const int S1 = S + 1;
+  const int t_tiles = T > 0 ? (T + kPanT - 1) / kPanT : 1, s_tiles = (S1 + kPanS - 1) / kPanS;
+  int b, tile;
+  if (!decode_block(t_tiles * s_tiles, B, b, tile)) return;
+  const int s_tile = (tile / t_tiles) * kPanS, t_tile = (tile % t_tiles) * kPanT;
+  const int T1 = rnnt_type == kRegular ? T + 1 : T;
+  const float *lmb = lm + (long)b * S1 * C;
+  const float *amb = am + (long)b * T * C;
+  const int64_t *symb = symbols + (long)b * S;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = lane >> 5, r32 = lane & 31;
+  const float ninf = -__builtin_huge_valf();
+
+  // ---- the symbols come first: the epilogue's gathers depend on them
+  // this thread's outputs: 16-byte pieces (row item / 8, frames 4 (item % 8) ..)
+  int out_sym[kPanItems];
+#pragma unroll
+  for (int j = 0; j < kPanItems; ++j) {
+    const int item = tid + kPanThreads * j, sr = s_tile + item / 8;
+    out_sym[j] = -1;
+    if (item < kPanS * 8 && sr < S) {
+      const int64_t y = symb[sr];
+      out_sym[j] = (y >= 0 && y < C) ? (int)y : -1;
+    }
+  }
+  int my_sym = -1;  // threads 0 .. 95 own a lattice row each
+  if (tid < kPanS && s_tile + tid < S) {
+    const int64_t y = symb[s_tile + tid];
+    my_sym = (y >= 0 && y < C) ? (int)y : -1;
+  }
+
+  // ---- what this lane fetches of every slab: rows sub + 8 j, k-offset 4 (lane % 8)
+  constexpr int kLoads = kPanRows / 8;
+  const int sub = lane >> 3, kq = 4 * (lane & 7);
+  int row_off[kLoads];    // element offset of (row, k = kq) in lm[b] / am[b], -1: no such row
+#pragma unroll
+  for (int j = 0; j < kLoads; ++j) {
+    const int row = sub + 8 * j;
+    if (row < kPanS) {
+      const int sr = s_tile + row;
+      row_off[j] = sr < S1 ? sr * C + kq : -1;
+    } else {
+      const int tr = t_tile + row - kPanS;
+      row_off[j] = tr < T ? tr * C + kq : -1;
+    }
+  }
+  // what lies outside the operands reads as -inf: neutral for the maximum, and
+  // exp(-inf - max) = 0 in the product
+  auto fetch = [&](floatx4 (&into)[kLoads], int k0) {
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+      const float *src = (sub + 8 * j < kPanS) ? lmb : amb;
+      const int valid = row_off[j] >= 0 ? min(4, max(C - k0 - kq, 0)) : 0;
+      into[j] = load4_guarded<kVec>(src, row_off[j] + k0, valid, ninf);
+    }
+  };
+  const int chunks = (C + kPanK - 1) / kPanK;
+
+  // ---- first pass: the row maxima (rnnt_loss.py:174-178).  Every wave scans its own
+  // slabs (they come from L2 again in the second pass), then the waves' results meet.
+  floatx4 slab[kLoads];
+  {
+    float m[kLoads];
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) m[j] = ninf;
+    // half a slab is consumed while the next half is in flight
+    constexpr int kHalf = kLoads / 2;
+    auto fetch_half = [&](floatx4 (&into)[kHalf], int first, int k0) {
+#pragma unroll
+      for (int j = 0; j < kHalf; ++j) {
+        const float *src = (sub + 8 * (first + j) < kPanS) ? lmb : amb;
+        const int valid = row_off[first + j] >= 0 ? min(4, max(C - k0 - kq, 0)) : 0;
+        into[j] = load4_guarded<kVec>(src, row_off[first + j] + k0, valid, ninf);
+      }
+    };
+    auto scan_half = [&](const floatx4 (&from)[kHalf], int first) {
+#pragma unroll
+      for (int j = 0; j < kHalf; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float v = from[j][i];
+          m[first + j] = (v > m[first + j] || v != v) ? v : m[first + j];  // NaN propagates, like torch.max
+        }
+    };
+    floatx4 lo[kHalf], hi[kHalf];
+    if (wave < chunks) fetch_half(lo, 0, wave * kPanK);
+    for (int chunk = wave; chunk < chunks; chunk += kPanWaves) {
+      fetch_half(hi, kHalf, chunk * kPanK);
+      scan_half(lo, 0);
+      if (chunk + kPanWaves < chunks) fetch_half(lo, 0, (chunk + kPanWaves) * kPanK);
+      scan_half(hi, kHalf);
+    }
+    // the second pass's first slab is requested before the maxima are exchanged
+    if (wave < chunks) fetch(slab, wave * kPanK);
+    // the eight lanes that share a row
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+#pragma unroll
+      for (int off = 1; off < 8; off <<= 1) {
+        const float o = __shfl_xor(m[j], off, kWave);
+        m[j] = (o > m[j] || o != o) ? o : m[j];
+      }
+      if ((lane & 7) == 0) wave_max[wave][sub + 8 * j] = m[j];
+    }
+  }
+  __syncthreads();
+  if (tid < kPanRows) {
+    float r = wave_max[0][tid];
+#pragma unroll
+    for (int w = 1; w < kPanWaves; ++w) {
+      const float o = wave_max[w][tid];
+      r = (o > r || o != o) ? o : r;
+    }
+    // saved for the backward pass; rows that do not exist get a harmless shift
+    bool exists;
+    if (tid < kPanS) {
+      exists = s_tile + tid < S1;
+      if (exists && t_tile == 0) lm_max[(long)b * S1 + s_tile + tid] = r;
+    } else {
+      exists = t_tile + tid - kPanS < T;
+      if (exists && s_tile == 0) am_max[(long)b * T + t_tile + tid - kPanS] = r;
+    }
+    slab_max[tid] = exists ? r : 0.f;
+  }
+  __syncthreads();
+  float shift[kLoads];    // the row's maximum
+#pragma unroll
+  for (int j = 0; j < kLoads; ++j) shift[j] = slab_max[sub + 8 * j];
+  int chunk = wave;
+
+  // ---- epilogue inputs, requested behind the first slab so that their latency hides
+  // under the loop: am[b, t, sym[b, s]] for this thread's outputs ...
+  float am_sym[kPanItems][4];
+#pragma unroll
+  for (int j = 0; j < kPanItems; ++j) {
+    const int item = tid + kPanThreads * j;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int tr = t_tile + 4 * (item % 8) + i;
+      am_sym[j][i] = (out_sym[j] >= 0 && tr < T) ? amb[tr * C + out_sym[j]] : 0.f;
+    }
+  }
+  // ... and the per-row / per-column terms (kept in registers until the loop is done)
+  float my_term = 0.f, my_symval = 0.f, my_max = 0.f;
+  if (tid < kPanS) {
+    const int sr = s_tile + tid;
+    if (sr < S1) {
+      my_term = lmb[sr * C + term];
+      my_max = slab_max[tid];
+      if (my_sym >= 0) my_symval = lmb[sr * C + my_sym];
+    }
+  } else if (tid >= 128 && tid < 128 + kPanT) {
+    const int tr = t_tile + tid - 128;
+    my_term = tr < T ? amb[tr * C + term] : 0.f;
+    my_max = slab_max[kPanS + tid - 128];
+  }
+
+  // ---- main loop over this wave's slabs
+  float *mine = pan_lds + wave * kPanSlab;
+  floatx16 acc[kPanS / 32];
+#pragma unroll
+  for (int j = 0; j < kPanS / 32; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+  for (; chunk < chunks; chunk += kPanWaves) {
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+      float *d = mine + (sub + 8 * j) * kPanPitch + kq;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) d[i] = __expf(slab[j][i] - shift[j]);
+    }
+    if (chunk + kPanWaves < chunks) fetch(slab, (chunk + kPanWaves) * kPanK);
+    const float *ap = mine + r32 * kPanPitch + half;
+    const float *bp = mine + (kPanS + r32) * kPanPitch + half;
+#pragma unroll
+    for (int i = 0; i < kPanK / 2; ++i) {
+      const float bv = bp[2 * i];
+#pragma unroll
+      for (int j = 0; j < kPanS / 32; ++j)
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[j * 32 * kPanPitch + 2 * i], bv, acc[j],
+                                                      0, 0, 0);
+    }
+  }
+
+  // ---- the partial sums meet: [wave][96][33] in the slab space
+  __syncthreads();
+  if (tid < kPanS) {
+    row_term[tid] = my_term;
+    row_sym[tid] = my_symval;
+    row_max[tid] = my_max;
+    row_symbol[tid] = my_sym;
+  } else if (tid >= 128 && tid < 128 + kPanT) {
+    col_term[tid - 128] = my_term;
+    col_max[tid - 128] = my_max;
+  }
+  float *part = pan_lds + wave * (kPanS * kPanPitch);
+#pragma unroll
+  for (int j = 0; j < kPanS / 32; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+      part[(32 * j + 8 * (v / 4) + 4 * half + (v % 4)) * kPanPitch + r32] = acc[j][v];
+  __syncthreads();
+
+  const int t_mask = (rnnt_type == kRegular && boundary) ? (int)boundary[4 * b + 3] : -1;
+  float *pxb = px + (long)b * S * T1;
+  float *pyb = py + (long)b * S1 * T;
+  float *nrb = norm_raw ? norm_raw + (long)b * S1 * T : nullptr;
+#pragma unroll
+  for (int j = 0; j < kPanItems; ++j) {
+    const int item = tid + kPanThreads * j;
+    const int m = item / 8, out_t = 4 * (item % 8), sr = s_tile + m;
+    if (item >= kPanS * 8 || sr >= S1) continue;
+    float raw[4], yv[4], xv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < kPanWaves; ++w)
+        sum += pan_lds[w * (kPanS * kPanPitch) + m * kPanPitch + out_t + i];
+      raw[i] = logf(sum + 1.17549435e-38f);
+      const float norm = raw[i] + row_max[m] + col_max[out_t + i];
+      yv[i] = (col_term[out_t + i] + row_term[m]) - norm;
+      float v = std::numeric_limits<float>::quiet_NaN();  // out-of-vocabulary symbol
+      if (row_symbol[m] >= 0) v = (am_sym[j][i] + row_sym[m]) - norm;
+      if (t_tile + out_t + i == t_mask) v = ninf;
+      xv[i] = v;
+    }
+    const int tr = t_tile + out_t;
+    if (tr + 4 <= T) {
+      if (nrb) *reinterpret_cast<floatx4u *>(nrb + sr * T + tr) = floatx4u{raw[0], raw[1], raw[2], raw[3]};
+      *reinterpret_cast<floatx4u *>(pyb + sr * T + tr) = floatx4u{yv[0], yv[1], yv[2], yv[3]};
+      if (sr < S)
+        *reinterpret_cast<floatx4u *>(pxb + sr * T1 + tr) = floatx4u{xv[0], xv[1], xv[2], xv[3]};
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (tr + i >= T) continue;
+        if (nrb) nrb[sr * T + tr + i] = raw[i];
+        pyb[sr * T + tr + i] = yv[i];
+        if (sr < S) pxb[sr * T1 + tr + i] = xv[i];
+      }
+    }
+  }
+  // the extra column of the regular lattice: nothing can be emitted after the last frame
+  if (rnnt_type == kRegular && t_tile == 0 && tid < kPanS && s_tile + tid < S)
+    pxb[(s_tile + tid) * T1 + T] = ninf;
 }
 
 // lm gradient: grid = (ceil(C/64), ceil((S+1)/32), B); k runs over frames.
@@ -660,23 +966,6 @@ constexpr int kAmPairs = kAmRows / 2;
 constexpr int kAmOutPitch = 68;  // row pitch of the result tiles staged in LDS
 constexpr int kAmQ = kAmT / 4;   // 16-byte pieces per panel row (kAmT == kAmC)
 
-// four consecutive floats at any element-aligned address (global memory takes
-// unaligned 16-byte accesses); `valid` (0..4) leading elements are read, the rest is 0
-typedef float floatx4u __attribute__((ext_vector_type(4), aligned(4)));
-template <bool kVec>
-__device__ __forceinline__ dgemm::floatx4 load4_guarded(const float *base, int off, int valid) {
-  dgemm::floatx4 r = {0.f, 0.f, 0.f, 0.f};
-  if (kVec && valid >= 4) {
-    const floatx4u t = *reinterpret_cast<const floatx4u *>(base + off);
-    r[0] = t[0], r[1] = t[1], r[2] = t[2], r[3] = t[3];
-  } else {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (i < valid) r[i] = base[off + i];
-  }
-  return r;
-}
-
 size_t am_panel_lds_bytes(int rows_cap) {
   const size_t panels = (size_t)rows_cap * (2 * kAmT + kAmC) * sizeof(float);
   const size_t staging = (size_t)2 * kAmT * kAmOutPitch * sizeof(float);
@@ -837,16 +1126,17 @@ __global__ void __launch_bounds__(256, 2)
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 void launch_fwd_gemm(const float *lm, const float *am, const int64_t *symbols,
-                     const int64_t *boundary, const float *lm_max, const float *am_max, float *px,
+                     const int64_t *boundary, float *lm_max, float *am_max, float *px,
                      float *py, float *norm_raw, int B, int S, int T, int C, int term,
                      int rnnt_type, hipStream_t stream) {
-  const int t_tiles = T > 0 ? (T + dgemm::kBN - 1) / dgemm::kBN : 1;
-  const int s_tiles = (S + 1 + dgemm::kBM - 1) / dgemm::kBM;
+  const int t_tiles = T > 0 ? (T + kPanT - 1) / kPanT : 1;
+  const int s_tiles = (S + 1 + kPanS - 1) / kPanS;
   const bool vec = (C % 4 == 0) && aligned16(lm) && aligned16(am);
-  auto kernel = vec ? simple_fwd_direct_kernel<true> : simple_fwd_direct_kernel<false>;
+  auto kernel = vec ? simple_fwd_panel_kernel<true> : simple_fwd_panel_kernel<false>;
+  (void)allow_lds(reinterpret_cast<const void *>(kernel), kPanLdsBytes);
   hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(t_tiles * s_tiles, B)),
-                     dim3(kFwdWaves * kWave), 0, stream, lm, am, symbols, boundary, lm_max, am_max,
-                     px, py, norm_raw, B, S, T, C, term, rnnt_type);
+                     dim3(kPanWaves * kWave), kPanLdsBytes, stream, lm, am, symbols, boundary,
+                     lm_max, am_max, px, py, norm_raw, B, S, T, C, term, rnnt_type);
 }
 void launch_fwd_gemm(const double *lm, const double *am, const int64_t *symbols,
                      const int64_t *boundary, const double *lm_max, const double *am_max,
@@ -888,9 +1178,7 @@ void launch_bwd_am(const float *lm, const float *am, const int64_t *symbols,
   // (the 16-byte accesses need no alignment; the scalar variant exists for checking)
   const bool vec = true;
   auto kernel = vec ? simple_bwd_am_panel_kernel<true> : simple_bwd_am_panel_kernel<false>;
-  if (lds > 64 * 1024)
-    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  (void)allow_lds(reinterpret_cast<const void *>(kernel), lds);
   hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(tiles, B)), dim3(256), lds, stream, lm, am,
                      symbols, boundary, lm_max, am_max, dmat, gpx, col_y, am_grad, B, S, T, C, ldd,
                      term, rnnt_type, rows_cap);
@@ -926,8 +1214,10 @@ int fwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   const long n_lm = (long)B * (S + 1), n_am = (long)B * T;
   const long rows = n_lm + n_am;
-  hipLaunchKernelGGL(row_max_kernel<R>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, lm,
-                     am, lm_max, am_max, n_lm, n_am, C);
+  // (the fp32 GEMM kernel finds the row maxima itself)
+  if (!std::is_same<R, float>::value)
+    hipLaunchKernelGGL(row_max_kernel<R>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream,
+                       lm, am, lm_max, am_max, n_lm, n_am, C);
   {
     // (the grid always has at least one column of tiles, so that the -inf column of
     // an empty-frame regular lattice is still written)

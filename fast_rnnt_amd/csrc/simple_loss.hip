@@ -1,0 +1,63 @@
+// rnnt_loss_simple's forward pipeline behind one call (rnnt_loss.py:230-340):
+// px/py from lm and am, the lattice recursion, optionally its backward with a
+// gradient of ones (the occupation probabilities), and the reduction of the scores.
+// It only chains the entry points of the other files on one stream; what it saves
+// is host time, which matters once a whole call takes ~100 us on the GPU.
+#include "common.hip.h"
+
+namespace frnnt {
+namespace {
+
+template <typename R, typename Logprobs, typename Forward, typename Backward, typename Reduce>
+int simple_loss_fwd(Logprobs logprobs, Forward forward, Backward backward, Reduce reduce,
+                    const R *lm, const R *am, const int64_t *symbols, const int64_t *boundary,
+                    R *px, R *py, R *lm_max, R *am_max, R *norm_raw, R *p, R *scores, R *px_grad,
+                    R *py_grad, R *loss, int B, int S, int T, int C, int term, int rnnt_type,
+                    int reduction, void *stream) {
+  if ((px_grad == nullptr) != (py_grad == nullptr))
+    return fail(FRNNT_EINVAL, "simple_loss_fwd: px_grad and py_grad go together");
+  int rc = logprobs(lm, am, symbols, boundary, px, py, lm_max, am_max, norm_raw, B, S, T, C, term,
+                    rnnt_type, stream);
+  if (rc != FRNNT_OK) return rc;
+  const int modified = rnnt_type != 0;
+  rc = forward(px, py, boundary, p, scores, B, S, T, modified, stream);
+  if (rc != FRNNT_OK) return rc;
+  if (px_grad) {
+    rc = backward(px, py, boundary, p, nullptr, px_grad, py_grad, B, S, T, modified, 0, stream);
+    if (rc != FRNNT_OK) return rc;
+  }
+  if (loss) rc = reduce(scores, loss, B, reduction, stream);
+  return rc;
+}
+
+}  // namespace
+}  // namespace frnnt
+
+extern "C" {
+
+int frnnt_simple_loss_fwd_f32(const float *lm, const float *am, const int64_t *symbols,
+                              const int64_t *boundary, float *px, float *py, float *lm_max,
+                              float *am_max, float *norm_raw, float *p, float *scores,
+                              float *px_grad, float *py_grad, float *loss, int B, int S, int T,
+                              int C, int termination_symbol, int rnnt_type, int reduction,
+                              void *stream) {
+  return frnnt::simple_loss_fwd<float>(frnnt_simple_logprobs_fwd_f32, frnnt_mi_forward_f32,
+                                       frnnt_mi_backward_f32, frnnt_loss_reduce_f32, lm, am,
+                                       symbols, boundary, px, py, lm_max, am_max, norm_raw, p,
+                                       scores, px_grad, py_grad, loss, B, S, T, C,
+                                       termination_symbol, rnnt_type, reduction, stream);
+}
+int frnnt_simple_loss_fwd_f64(const double *lm, const double *am, const int64_t *symbols,
+                              const int64_t *boundary, double *px, double *py, double *lm_max,
+                              double *am_max, double *norm_raw, double *p, double *scores,
+                              double *px_grad, double *py_grad, double *loss, int B, int S, int T,
+                              int C, int termination_symbol, int rnnt_type, int reduction,
+                              void *stream) {
+  return frnnt::simple_loss_fwd<double>(frnnt_simple_logprobs_fwd_f64, frnnt_mi_forward_f64,
+                                        frnnt_mi_backward_f64, frnnt_loss_reduce_f64, lm, am,
+                                        symbols, boundary, px, py, lm_max, am_max, norm_raw, p,
+                                        scores, px_grad, py_grad, loss, B, S, T, C,
+                                        termination_symbol, rnnt_type, reduction, stream);
+}
+
+}  // extern "C"

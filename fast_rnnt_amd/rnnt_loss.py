@@ -14,6 +14,8 @@ and ``"constrained"`` (modified, plus a forced blank after each symbol).
 """
 from typing import Optional, Tuple, Union
 
+import contextlib
+
 import torch
 from torch import Tensor
 
@@ -173,6 +175,23 @@ def _recursion_and_reduce(px, py, boundary, rnnt_type, delay_penalty, reduction,
 _REDUCTIONS = {"none": 0, "mean": 1, "sum": 2}
 
 
+def _on_device(device):
+    """Device guard that costs nothing when `device` is already current."""
+    if torch.cuda.current_device() == device.index:
+        return contextlib.nullcontext()
+    return torch.cuda.device(device)
+
+
+def _carve(sizes):
+    """Element offsets of consecutive buffers, each starting 16-byte aligned (for
+    4- and 8-byte elements), and the total element count."""
+    offsets, total = [], 0
+    for n in sizes:
+        offsets.append(total)
+        total += (n + 3) & ~3
+    return offsets, total
+
+
 class _SimpleLoss(torch.autograd.Function):
     """rnnt_loss_simple's whole device pipeline behind one autograd node:
     px/py (row maxima + MFMA contraction), the lattice recursion forward, the
@@ -181,8 +200,8 @@ class _SimpleLoss(torch.autograd.Function):
     of ones, whose result both is handed out as (px_grad, py_grad) and is what
     backward() scales in place and pushes through the two gradient GEMMs.  Same
     arithmetic as get_rnnt_logprobs, mutual_information_recursion and the
-    reduction of rnnt_loss.py:330-340; it only saves Python, launch and
-    elementwise-kernel overhead."""
+    reduction of rnnt_loss.py:330-340; it only saves host time (one library call,
+    one workspace allocation) and elementwise kernels."""
 
     @staticmethod
     def forward(ctx, lm, am, symbols, boundary, termination_symbol, rnnt_type, delay_penalty,
@@ -199,38 +218,47 @@ class _SimpleLoss(torch.autograd.Function):
         need_grad = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
         # gradients of the non-differentiable outputs are not wanted as zero tensors
         ctx.set_materialize_grads(False)
-        with torch.cuda.device(am.device):
+        n_px, n_py = B * S * T1, B * (S + 1) * T
+        # internal buffers live in one allocation: px | py | lm_max | am_max | norm_raw | p | scores
+        (o_px, o_py, o_lmx, o_amx, o_nr, o_p, o_sc), total = _carve(
+            [n_px, n_py, B * (S + 1), B * T, n_py if need_grad else 0, B * (S + 1) * (T + 1), B])
+        with _on_device(am.device):
             stream = _lib.stream_of(am)
-            px = torch.empty(B, S, T1, **opts)
-            py = torch.empty(B, S + 1, T, **opts)
-            lm_max = torch.empty(B, S + 1, **opts)
-            am_max = torch.empty(B, T, **opts)
-            norm_raw = torch.empty(B, S + 1, T, **opts) if need_grad else None
-            _lib.call("frnnt_simple_logprobs_fwd_" + sfx, lm_c.data_ptr(), am_c.data_ptr(),
-                      sym_c.data_ptr(), _lib.ptr(bnd_c), px.data_ptr(), py.data_ptr(),
-                      lm_max.data_ptr(), am_max.data_ptr(), _lib.ptr(norm_raw), B, S, T, C,
-                      int(termination_symbol), kind, stream)
-            if delay_penalty > 0.0:
-                _apply_delay_penalty(px, boundary, rnnt_type, delay_penalty)
-            p = torch.empty(B, S + 1, T + 1, **opts)
-            scores = torch.empty(B, **opts)
-            modified = int(kind != 0)
-            _lib.call("frnnt_mi_forward_" + sfx, px.data_ptr(), py.data_ptr(), _lib.ptr(bnd_c),
-                      p.data_ptr(), scores.data_ptr(), B, S, T, modified, stream)
+            work = torch.empty(total, **opts)
+            base, item = work.data_ptr(), work.element_size()
+            at = lambda off: base + off * item  # noqa: E731
             px_grad = py_grad = None
             if want_grads or need_grad:
-                px_grad = torch.empty_like(px)
-                py_grad = torch.empty_like(py)
-                _lib.call("frnnt_mi_backward_" + sfx, px.data_ptr(), py.data_ptr(),
-                          _lib.ptr(bnd_c), p.data_ptr(), None, px_grad.data_ptr(),
-                          py_grad.data_ptr(), B, S, T, modified, 0, stream)
+                px_grad = torch.empty(B, S, T1, **opts)
+                py_grad = torch.empty(B, S + 1, T, **opts)
             loss = torch.empty((B,) if reduction == 0 else (), **opts)
-            _lib.call("frnnt_loss_reduce_" + sfx, scores.data_ptr(), loss.data_ptr(), B,
-                      reduction, stream)
+            if delay_penalty > 0.0:
+                # the penalty is applied to px between the two stages (rnnt_loss.py:311-326)
+                px = work[o_px:o_px + n_px].view(B, S, T1)
+                _lib.call("frnnt_simple_logprobs_fwd_" + sfx, lm_c.data_ptr(), am_c.data_ptr(),
+                          sym_c.data_ptr(), _lib.ptr(bnd_c), at(o_px), at(o_py), at(o_lmx),
+                          at(o_amx), at(o_nr) if need_grad else None, B, S, T, C,
+                          int(termination_symbol), kind, stream)
+                _apply_delay_penalty(px, boundary, rnnt_type, delay_penalty)
+                modified = int(kind != 0)
+                _lib.call("frnnt_mi_forward_" + sfx, at(o_px), at(o_py), _lib.ptr(bnd_c), at(o_p),
+                          at(o_sc), B, S, T, modified, stream)
+                if px_grad is not None:
+                    _lib.call("frnnt_mi_backward_" + sfx, at(o_px), at(o_py), _lib.ptr(bnd_c),
+                              at(o_p), None, px_grad.data_ptr(), py_grad.data_ptr(), B, S, T,
+                              modified, 0, stream)
+                _lib.call("frnnt_loss_reduce_" + sfx, at(o_sc), loss.data_ptr(), B, reduction,
+                          stream)
+            else:
+                _lib.call("frnnt_simple_loss_fwd_" + sfx, lm_c.data_ptr(), am_c.data_ptr(),
+                          sym_c.data_ptr(), _lib.ptr(bnd_c), at(o_px), at(o_py), at(o_lmx),
+                          at(o_amx), at(o_nr) if need_grad else None, at(o_p), at(o_sc),
+                          _lib.ptr(px_grad), _lib.ptr(py_grad), loss.data_ptr(), B, S, T, C,
+                          int(termination_symbol), kind, reduction, stream)
         if need_grad:
-            ctx.save_for_backward(lm_c, am_c, sym_c, bnd_c, lm_max, am_max, norm_raw, px_grad,
-                                  py_grad)
-            ctx.meta = (B, S, T, C, int(termination_symbol), kind, sfx, reduction)
+            ctx.save_for_backward(lm_c, am_c, sym_c, bnd_c, work, px_grad, py_grad)
+            ctx.meta = (B, S, T, C, int(termination_symbol), kind, sfx, reduction,
+                        o_lmx, o_amx, o_nr)
         if px_grad is None:
             return loss, None, None
         ctx.mark_non_differentiable(px_grad, py_grad)
@@ -240,28 +268,30 @@ class _SimpleLoss(torch.autograd.Function):
     def backward(ctx, g_loss, _gx, _gy):
         if g_loss is None:
             return (None,) * 9
-        lm, am, sym, bnd, lm_max, am_max, norm_raw, px_grad, py_grad = ctx.saved_tensors
-        B, S, T, C, term, kind, sfx, reduction = ctx.meta
+        lm, am, sym, bnd, work, px_grad, py_grad = ctx.saved_tensors
+        B, S, T, C, term, kind, sfx, reduction, o_lmx, o_amx, o_nr = ctx.meta
         opts = dict(dtype=am.dtype, device=am.device)
-        with torch.cuda.device(am.device):
+        with _on_device(am.device):
             # d loss / d scores[b] = scale * g_loss[b * stride]
             g = g_loss.contiguous()
             stride = 1 if reduction == 0 else 0
             scale = -1.0 / B if reduction == 1 else -1.0
-            dmat = torch.empty(B, S + 1, (T + 3) // 4 * 4, **opts)
-            row_x = torch.empty(B, S + 1, **opts)
-            row_y = torch.empty(B, S + 1, **opts)
-            col_y = torch.empty(B, T, **opts)
+            ldd = (T + 3) // 4 * 4
+            # scratch in one allocation: dmat | row_x | row_y | col_y
+            (o_d, o_rx, o_ry, o_cy), total = _carve(
+                [B * (S + 1) * ldd, B * (S + 1), B * (S + 1), B * T])
+            scratch = torch.empty(total, **opts)
+            sbase, wbase, item = scratch.data_ptr(), work.data_ptr(), work.element_size()
             lm_grad = torch.empty_like(lm) if ctx.needs_input_grad[0] else None
             am_grad = torch.empty_like(am) if ctx.needs_input_grad[1] else None
             # px_grad / py_grad are scaled in place by the scores' gradient, exactly as
             # MutualInformationRecursionFunction.backward does to the tensors it handed out
             _lib.call("frnnt_simple_logprobs_bwd_" + sfx, lm.data_ptr(), am.data_ptr(),
-                      sym.data_ptr(), _lib.ptr(bnd), lm_max.data_ptr(), am_max.data_ptr(),
-                      norm_raw.data_ptr(), g.data_ptr(), stride, scale, px_grad.data_ptr(),
-                      py_grad.data_ptr(), dmat.data_ptr(), row_x.data_ptr(), row_y.data_ptr(),
-                      col_y.data_ptr(), _lib.ptr(lm_grad), _lib.ptr(am_grad), B, S, T, C, term,
-                      kind, _lib.stream_of(am))
+                      sym.data_ptr(), _lib.ptr(bnd), wbase + o_lmx * item, wbase + o_amx * item,
+                      wbase + o_nr * item, g.data_ptr(), stride, scale, px_grad.data_ptr(),
+                      py_grad.data_ptr(), sbase + o_d * item, sbase + o_rx * item,
+                      sbase + o_ry * item, sbase + o_cy * item, _lib.ptr(lm_grad),
+                      _lib.ptr(am_grad), B, S, T, C, term, kind, _lib.stream_of(am))
         return lm_grad, am_grad, None, None, None, None, None, None, None
 
 

@@ -142,6 +142,27 @@ int frnnt_simple_logprobs_bwd_f64(const double *lm, const double *am, const int6
                                   double *lm_grad, double *am_grad, int B, int S, int T, int C,
                                   int termination_symbol, int rnnt_type, void *stream);
 /*
+ * Forward pipeline of rnnt_loss_simple (rnnt_loss.py:230-340) in one call:
+ * frnnt_simple_logprobs_fwd, frnnt_mi_forward, then -- when px_grad / py_grad are
+ * given -- frnnt_mi_backward with a gradient of ones (what the recursion's autograd
+ * wrapper computes eagerly, mutual_information.py:159-168), then -- when loss is
+ * given -- frnnt_loss_reduce.  Arguments as in those entry points; p [B][S+1][T+1]
+ * and scores [B] are outputs as well.  It exists to save host time per call.
+ */
+int frnnt_simple_loss_fwd_f32(const float *lm, const float *am, const int64_t *symbols,
+                              const int64_t *boundary, float *px, float *py, float *lm_max,
+                              float *am_max, float *norm_raw, float *p, float *scores,
+                              float *px_grad, float *py_grad, float *loss, int B, int S, int T,
+                              int C, int termination_symbol, int rnnt_type, int reduction,
+                              void *stream);
+int frnnt_simple_loss_fwd_f64(const double *lm, const double *am, const int64_t *symbols,
+                              const int64_t *boundary, double *px, double *py, double *lm_max,
+                              double *am_max, double *norm_raw, double *p, double *scores,
+                              double *px_grad, double *py_grad, double *loss, int B, int S, int T,
+                              int C, int termination_symbol, int rnnt_type, int reduction,
+                              void *stream);
+
+/*
  * The reduction at the end of every loss function (rnnt_loss.py:160-169, :330-340):
  * loss = -scores (reduction 0, [B]), -mean(scores) (1, one value) or -sum(scores)
  * (2, one value), summed in a fixed order by one workgroup.
