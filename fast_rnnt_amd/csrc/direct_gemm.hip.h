@@ -67,10 +67,6 @@ __device__ __forceinline__ void load_rowfast(Frag &f, const float *base, int ld,
   for (int i = 0; i < 16; ++i) f.v[i] = (ok && k0 + i < K) ? base[(k0 + i) * ld + col] : fill;
 }
 
-__device__ __forceinline__ void exp_shift_scalar(Frag &f, float shift) {
-#pragma unroll
-  for (int i = 0; i < 16; ++i) f.v[i] = __expf(f.v[i] - shift);
-}
 __device__ __forceinline__ void exp_shift_each(Frag &f, const Frag &shift) {
 #pragma unroll
   for (int i = 0; i < 16; ++i) f.v[i] = __expf(f.v[i] - shift.v[i]);
@@ -127,25 +123,6 @@ __device__ __forceinline__ void reduce_and_emit(const Acc &acc, float *lds, Pre 
     for (int w = 0; w < kW; ++w) sum += lds[w * kBM * kBN + e];
     post(e / kBN, e % kBN, sum, fetched[j]);
   }
-}
-
-// The same for a wave's own tile, straight from the accumulators (consecutive
-// lanes walk consecutive columns).
-template <typename Pre, typename Post>
-__device__ __forceinline__ void emit_own(const Acc &acc, Pre pre, Post post) {
-  const int lane = threadIdx.x & 63;
-  const int half = lane >> 5, col = lane & 31;
-  float fetched[32];
-#pragma unroll
-  for (int v = 0; v < 16; ++v)
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-      fetched[2 * v + t] = pre(8 * (v / 4) + 4 * half + (v % 4), 32 * t + col);
-#pragma unroll
-  for (int v = 0; v < 16; ++v)
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-      post(8 * (v / 4) + 4 * half + (v % 4), 32 * t + col, acc.c[t][v], fetched[2 * v + t]);
 }
 
 // XCD-aware decode of a 1-D grid: all tiles of batch element b run on XCD b % 8,

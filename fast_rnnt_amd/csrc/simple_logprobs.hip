@@ -385,132 +385,6 @@ __device__ __forceinline__ dgemm::floatx4 load4_guarded(const float *base, int o
 }
 
 // ---- fp32: register-direct MFMA kernels (direct_gemm.hip.h) ------------------------
-constexpr int kFwdWaves = 4;  // K split of the forward normalizer GEMM
-constexpr int kLmWaves = 4;   // K split of the lm-gradient GEMM
-
-// 1-D XCD-aware grid over (b, s-tile, t-tile); 8 waves split C between them.
-template <bool kVec>
-__global__ void __launch_bounds__(kFwdWaves *kWave)
-    simple_fwd_direct_kernel(const float *__restrict__ lm, const float *__restrict__ am,
-                             const int64_t *__restrict__ symbols,
-                             const int64_t *__restrict__ boundary,
-                             const float *__restrict__ lm_max, const float *__restrict__ am_max,
-                             float *__restrict__ px, float *__restrict__ py,
-                             float *__restrict__ norm_raw, int B, int S, int T, int C, int term,
-                             int rnnt_type) {
-  using namespace dgemm;
-  __shared__ float lds[kFwdWaves * kBM * kBN];
-  __shared__ float row_term[kBM], row_sym[kBM], row_max[kBM];  // lm[s,term], lm[s,sym[s]], lm_max[s]
-  __shared__ int row_symbol[kBM];
-  __shared__ float col_term[kBN], col_max[kBN];                // am[t,term], am_max[t]
-  const int S1 = S + 1;
-  const int t_tiles = T > 0 ? (T + kBN - 1) / kBN : 1, s_tiles = (S1 + kBM - 1) / kBM;
-  int b, tile;
-  if (!decode_block(t_tiles * s_tiles, B, b, tile)) return;
-  const int s_tile = (tile / t_tiles) * kBM, t_tile = (tile % t_tiles) * kBN;
-  const int T1 = rnnt_type == kRegular ? T + 1 : T;
-  const float *lmb = lm + (long)b * S1 * C;
-  const float *amb = am + (long)b * T * C;
-  const float *lmx = lm_max + (long)b * S1;
-  const float *amx = am_max + (long)b * T;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int half = lane >> 5, r32 = lane & 31;
-  const float ninf = -__builtin_huge_valf();
-
-  const int s_row = s_tile + r32, t_row0 = t_tile + r32, t_row1 = t_tile + 32 + r32;
-  const bool a_ok = s_row < S1, b_ok0 = t_row0 < T, b_ok1 = t_row1 < T;
-
-  Acc acc;
-  acc.clear();
-  Frag a, b0, b1, an, b0n, b1n;
-  auto fetch = [&](Frag &fa, Frag &f0, Frag &f1, int kb) {
-    const int k0 = kb + 16 * half;
-    load_kfast<kVec>(fa, lmb, s_row * C, a_ok, k0, C, ninf);
-    load_kfast<kVec>(f0, amb, t_row0 * C, b_ok0, k0, C, ninf);
-    load_kfast<kVec>(f1, amb, t_row1 * C, b_ok1, k0, C, ninf);
-  };
-  int kb = wave * kBK;
-  if (kb < C) fetch(an, b0n, b1n, kb);
-
-  // Everything the epilogue needs from global memory is requested now, behind the
-  // first operand fetch, so that its latency hides under the GEMM loop:
-  // am[b, t, sym[b, s]] for this thread's output elements ...
-  constexpr int kPer = kBM * kBN / (kFwdWaves * kWave);
-  float am_sym[kPer];
-#pragma unroll
-  for (int j = 0; j < kPer; ++j) {
-    const int e = j * (kFwdWaves * kWave) + tid;
-    const int s = s_tile + e / kBN, t = t_tile + e % kBN;
-    am_sym[j] = 0.f;
-    if (s < S && t < T) {
-      const int64_t y = symbols[(long)b * S + s];
-      if (y >= 0 && y < C) am_sym[j] = amb[(long)t * C + y];
-    }
-  }
-  // ... and the per-row / per-column terms, shared through LDS
-  if (tid < kBM) {
-    const int s = s_tile + tid;
-    float vt = 0.f, vs = 0.f, vm = 0.f;
-    int sym = -1;
-    if (s < S1) {
-      vt = lmb[(long)s * C + term];
-      vm = lmx[s];
-      if (s < S) {
-        const int64_t y = symbols[(long)b * S + s];
-        sym = (y >= 0 && y < C) ? (int)y : -1;
-        if (sym >= 0) vs = lmb[(long)s * C + sym];
-      }
-    }
-    row_term[tid] = vt;
-    row_sym[tid] = vs;
-    row_max[tid] = vm;
-    row_symbol[tid] = sym;
-  } else if (tid >= 64 && tid < 64 + kBN) {
-    const int t = t_tile + tid - 64;
-    col_term[tid - 64] = t < T ? amb[(long)t * C + term] : 0.f;
-    col_max[tid - 64] = t < T ? amx[t] : 0.f;
-  }
-  const float a_shift = a_ok ? lmx[s_row] : 0.f;
-  const float b_shift0 = b_ok0 ? amx[t_row0] : 0.f;
-  const float b_shift1 = b_ok1 ? amx[t_row1] : 0.f;
-
-  for (; kb < C; kb += kFwdWaves * kBK) {
-    a = an;
-    b0 = b0n;
-    b1 = b1n;
-    if (kb + kFwdWaves * kBK < C) fetch(an, b0n, b1n, kb + kFwdWaves * kBK);
-    exp_shift_scalar(a, a_shift);
-    exp_shift_scalar(b0, b_shift0);
-    exp_shift_scalar(b1, b_shift1);
-    acc.mma(a, b0, b1);
-  }
-
-  const int t_mask = (rnnt_type == kRegular && boundary) ? (int)boundary[4 * b + 3] : -1;
-  float *pxb = px + (long)b * S * T1;
-  float *pyb = py + (long)b * S1 * T;
-  float *nrb = norm_raw ? norm_raw + (long)b * S1 * T : nullptr;
-  // (the barrier inside reduce_and_emit also publishes row_* / col_* to all waves)
-  int slot = 0;
-  reduce_and_emit<kFwdWaves>(
-      acc, lds, [&](int, int) -> float { return am_sym[slot++]; },
-      [&](int m, int n, float sum, float am_at_sym) {
-        const int s = s_tile + m, t = t_tile + n;
-        if (s >= S1 || t >= T) return;
-        const float raw = logf(sum + 1.17549435e-38f);
-        if (nrb) nrb[(long)s * T + t] = raw;
-        const float norm = raw + row_max[m] + col_max[n];
-        pyb[(long)s * T + t] = (col_term[n] + row_term[m]) - norm;
-        if (s < S) {
-          float v = std::numeric_limits<float>::quiet_NaN();  // out-of-vocabulary symbol
-          if (row_symbol[m] >= 0) v = (am_at_sym + row_sym[m]) - norm;
-          if (t == t_mask) v = ninf;
-          pxb[(long)s * T1 + t] = v;
-        }
-      });
-  // the extra column of the regular lattice: nothing can be emitted after the last frame
-  if (rnnt_type == kRegular && t_tile == 0 && tid < kBM && s_tile + tid < S)
-    pxb[(long)(s_tile + tid) * T1 + T] = ninf;
-}
 
 // Normalizer GEMM, wave-private LDS transposition.  Both operands are k-contiguous
 // ([rows][C]), the matrix cores want one row per lane.  Letting every lane fetch its
@@ -800,147 +674,154 @@ __global__ void __launch_bounds__(kPanThreads)
     pxb[(s_tile + tid) * T1 + T] = ninf;
 }
 
-// lm gradient: grid = (ceil(C/64), ceil((S+1)/32), B); k runs over frames.
-template <bool kVec>
-__global__ void __launch_bounds__(kLmWaves *kWave)
-    simple_bwd_lm_direct_kernel(const float *__restrict__ lm, const float *__restrict__ am,
-                                const int64_t *__restrict__ symbols,
-                                const float *__restrict__ lm_max,
-                                const float *__restrict__ am_max, const float *__restrict__ dmat,
-                                const float *__restrict__ row_x, const float *__restrict__ row_y,
-                                float *__restrict__ lm_grad, int B, int S, int T, int C,
-                                int ldd, int term) {
+// lm gradient:  lm.grad[s,c] = exp(lm[s,c] - max[s]) * sum_t D[s,t] exp(am[t,c] - max[t])
+// + [c = sym[s]] row_x[s] + [c = term] row_y[s].  Same scheme as the normalizer GEMM:
+// k runs over frames and is split between the waves of a workgroup; a wave turns its
+// 32-frame slabs -- D[96 rows][32 k], fetched as coalesced 16-byte pieces and
+// transposed through its own LDS region, and exp(am[32 k][32 c] - max) -- into MFMA
+// operands without waiting for any other wave; the partial sums meet once at the end.
+// A workgroup covers 96 lattice rows x 32 vocabulary entries.
+constexpr int kLmS = 96;
+constexpr int kLmC = 32;
+constexpr int kLmK = 32;
+constexpr int kLmWaves = 4;
+constexpr int kLmThreads = kLmWaves * kWave;
+constexpr int kLmPitch = kLmK + 1;
+constexpr int kLmSlab = kLmS * kLmPitch + kLmK * kLmC;  // floats per wave: D slab, then am slab
+constexpr size_t kLmLdsBytes = (size_t)kLmWaves * kLmSlab * sizeof(float);
+constexpr int kLmItems = kLmS * kLmC / 4 / kLmThreads;   // 16-byte outputs per thread
+
+__global__ void __launch_bounds__(kLmThreads, 2)
+    simple_bwd_lm_slab_kernel(const float *__restrict__ lm, const float *__restrict__ am,
+                              const int64_t *__restrict__ symbols,
+                              const float *__restrict__ lm_max,
+                              const float *__restrict__ am_max, const float *__restrict__ dmat,
+                              const float *__restrict__ row_x, const float *__restrict__ row_y,
+                              float *__restrict__ lm_grad, int B, int S, int T, int C, int ldd,
+                              int term) {
   using namespace dgemm;
-  __shared__ float lds[kLmWaves * kBM * kBN];
+  extern __shared__ float lm_lds[];
   const int S1 = S + 1;
-  const int c_tiles = (C + kBN - 1) / kBN, s_tiles = (S1 + kBM - 1) / kBM;
+  const int c_tiles = (C + kLmC - 1) / kLmC, s_tiles = (S1 + kLmS - 1) / kLmS;
   int b, tile;
   if (!decode_block(c_tiles * s_tiles, B, b, tile)) return;
-  const int s_tile = (tile / c_tiles) * kBM, c_tile = (tile % c_tiles) * kBN;
+  const int s_tile = (tile / c_tiles) * kLmS, c_tile = (tile % c_tiles) * kLmC;
   const float *lmb = lm + (long)b * S1 * C;
   const float *amb = am + (long)b * T * C;
   const float *lmx = lm_max + (long)b * S1;
   const float *amx = am_max + (long)b * T;
   const float *db = dmat + (long)b * S1 * ldd;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int half = lane >> 5, r32 = lane & 31;
   const float ninf = -__builtin_huge_valf();
 
-  const int s_row = s_tile + r32, c0 = c_tile + r32, c1 = c_tile + 32 + r32;
-  const bool a_ok = s_row < S1, b_ok0 = c0 < C, b_ok1 = c1 < C;
-
-  // this thread's lm[b, s, c] for the epilogue, requested ahead of the GEMM loop
-  constexpr int kPer = kBM * kBN / (kLmWaves * kWave);
-  float lm_sc[kPer];
+  // what this lane fetches of every slab: D rows sub + 8 j at k-offset kq; am rows
+  // (frames) sub + 8 j at vocabulary offset kq
+  constexpr int kLoadsA = kLmS / 8, kLoadsB = kLmK / 8;
+  const int sub = lane >> 3, kq = 4 * (lane & 7);
+  floatx4 sa[kLoadsA], sb[kLoadsB];
+  float shift[kLoadsB];
+  auto fetch = [&](int k0) {
 #pragma unroll
-  for (int j = 0; j < kPer; ++j) {
-    const int e = j * (kLmWaves * kWave) + (int)threadIdx.x;
-    const int s = s_tile + e / kBN, c = c_tile + e % kBN;
-    lm_sc[j] = (s < S1 && c < C) ? lmb[(long)s * C + c] : 0.f;
-  }
-  Acc acc;
-  acc.clear();
-  for (int kb = wave * kBK; kb < T; kb += kLmWaves * kBK) {
-    const int k0 = kb + 16 * half;
-    Frag a, b0, b1, mx;
-    load_kfast<kVec>(a, db, s_row * ldd, a_ok, k0, T, 0.f);
-    load_rowfast(b0, amb, C, c0, b_ok0, k0, T, ninf);
-    load_rowfast(b1, amb, C, c1, b_ok1, k0, T, ninf);
-    load_kfast<false>(mx, amx, 0, true, k0, T, 0.f);
-    exp_shift_each(b0, mx);
-    exp_shift_each(b1, mx);
-    acc.mma(a, b0, b1);
-  }
-  int slot = 0;
-  reduce_and_emit<kLmWaves>(
-      acc, lds, [&](int, int) -> float { return lm_sc[slot++]; },
-      [&](int m, int n, float sum, float lm_at) {
-        const int s = s_tile + m, c = c_tile + n;
-        if (s >= S1 || c >= C) return;
-        float g = __expf(lm_at - lmx[s]) * sum;
-        if (s < S && symbols[(long)b * S + s] == c) g += row_x[(long)b * S1 + s];
-        if (c == term) g += row_y[(long)b * S1 + s];
-        lm_grad[((long)b * S1 + s) * C + c] = g;
-      });
-}
-
-// am gradient: k runs over the S+1 lattice rows -- too short to split, so each of
-// the four waves of a workgroup owns its own 32 (frames) x 32 (vocabulary) tile;
-// small tiles keep the register count low enough for four waves per SIMD, which
-// is what hides the memory latency of this streaming kernel.
-// The per-symbol term  sum_s [c = sym[b,s]] gx[b,s,t]  is a second product on the
-// matrix core, gx^T times a one-hot matrix made in registers from the symbols: it is
-// exact (products by 0 or 1) and has a fixed summation order.
-__global__ void __launch_bounds__(256)
-    simple_bwd_am_direct_kernel(const float *__restrict__ lm, const float *__restrict__ am,
-                                const int64_t *__restrict__ symbols,
-                                const int64_t *__restrict__ boundary,
-                                const float *__restrict__ lm_max,
-                                const float *__restrict__ am_max, const float *__restrict__ dmat,
-                                const float *__restrict__ gpx, const float *__restrict__ col_y,
-                                float *__restrict__ am_grad, int B, int S, int T, int C, int ldd,
-                                int term, int rnnt_type) {
-  using namespace dgemm;
-  const int S1 = S + 1;
-  const int T1 = rnnt_type == kRegular ? T + 1 : T;
-  const int c_tiles = (C + 31) / 32, t_groups = (T + 4 * kBM - 1) / (4 * kBM);
-  int b, tile;
-  if (!decode_block(c_tiles * t_groups, B, b, tile)) return;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int t_tile = ((tile / c_tiles) * 4 + wave) * kBM, c_tile = (tile % c_tiles) * 32;
-  if (t_tile >= T) return;
-  const float *lmb = lm + (long)b * S1 * C;
-  const float *amb = am + (long)b * T * C;
-  const float *lmx = lm_max + (long)b * S1;
-  const float *amx = am_max + (long)b * T;
-  const float *db = dmat + (long)b * S1 * ldd;
-  const float *gxb = gpx + (long)b * S * T1;
-  const int64_t *symb = symbols + (long)b * S;
-  const int half = lane >> 5, r32 = lane & 31;
-  const float ninf = -__builtin_huge_valf();
-  const int t_mask = (rnnt_type == kRegular && boundary) ? (int)boundary[4 * b + 3] : -1;
-
-  const int t_row = t_tile + r32, c0 = c_tile + r32;
-  const bool a_ok = t_row < T, g_ok = t_row < T && t_row != t_mask, b_ok = c0 < C;
-
-  // epilogue inputs first: am[b, t, c] of this lane's 16 output elements
-  float am_tc[16];
+    for (int j = 0; j < kLoadsA; ++j) {
+      const int sr = s_tile + sub + 8 * j;
+      // columns at and beyond T must read as 0: the pad of a D row is not defined
+      const int valid = sr < S1 ? min(4, max(T - k0 - kq, 0)) : 0;
+      sa[j] = load4_guarded<true>(db, sr * ldd + k0 + kq, valid);
+    }
 #pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const int t = t_tile + 8 * (v / 4) + 4 * half + (v % 4);
-    am_tc[v] = (t < T && c0 < C) ? amb[(long)t * C + c0] : 0.f;
+    for (int j = 0; j < kLoadsB; ++j) {
+      const int tr = k0 + sub + 8 * j, c = c_tile + kq;
+      const int valid = tr < T ? min(4, max(C - c, 0)) : 0;
+      sb[j] = load4_guarded<true>(amb, tr * C + c, valid, ninf);
+      shift[j] = tr < T ? amx[tr] : 0.f;
+    }
+  };
+  const int chunks = (T + kLmK - 1) / kLmK;
+  int chunk = wave;
+  if (chunk < chunks) fetch(chunk * kLmK);
+
+  // epilogue inputs behind the first slab: this thread's pieces of lm (row item / 8,
+  // vocabulary entries 4 (item % 8) ..)
+  floatx4 lm_in[kLmItems];
+#pragma unroll
+  for (int j = 0; j < kLmItems; ++j) {
+    const int item = tid + kLmThreads * j;
+    const int sr = s_tile + item / 8, c = c_tile + 4 * (item % 8);
+    lm_in[j] = load4_guarded<true>(lmb, sr * C + c, sr < S1 ? min(4, max(C - c, 0)) : 0);
   }
 
-  floatx16 acc, hot;
+  float *as = lm_lds + wave * kLmSlab;
+  float *bs = as + kLmS * kLmPitch;
+  floatx16 acc[kLmS / 32];
 #pragma unroll
-  for (int v = 0; v < 16; ++v) acc[v] = hot[v] = 0.f;
-  // symbols are < C < 2^31: their low words (little endian) are enough to compare
-  const int *sym_lo = reinterpret_cast<const int *>(symb);
-#pragma unroll 1
-  for (int kb = 0; kb < S1; kb += kBK) {
-    const int k0 = kb + 16 * half;
-    Frag a, g, b0, mx;
-    load_rowfast(a, db, ldd, t_row, a_ok, k0, S1, 0.f);
-    load_rowfast(g, gxb, T1, t_row, g_ok, k0, S, 0.f);
-    load_rowfast(b0, lmb, C, c0, b_ok, k0, S1, ninf);
-    load_kfast<false>(mx, lmx, 0, true, k0, S1, 0.f);
-    exp_shift_each(b0, mx);
+  for (int j = 0; j < kLmS / 32; ++j)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int y = (k0 + i < S) ? sym_lo[2 * (k0 + i)] : -1;
-      const float h = (y == c0) ? 1.f : 0.f;
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.v[i], b0.v[i], acc, 0, 0, 0);
-      hot = __builtin_amdgcn_mfma_f32_32x32x2f32(g.v[i], h, hot, 0, 0, 0);
+    for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+  for (; chunk < chunks; chunk += kLmWaves) {
+#pragma unroll
+    for (int j = 0; j < kLoadsA; ++j) {
+      float *d = as + (sub + 8 * j) * kLmPitch + kq;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) d[i] = sa[j][i];
+    }
+#pragma unroll
+    for (int j = 0; j < kLoadsB; ++j) {
+      floatx4 e;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) e[i] = __expf(sb[j][i] - shift[j]);
+      *reinterpret_cast<floatx4 *>(bs + (sub + 8 * j) * kLmC + kq) = e;
+    }
+    if (chunk + kLmWaves < chunks) fetch((chunk + kLmWaves) * kLmK);
+    const float *ap = as + r32 * kLmPitch + half;
+    const float *bp = bs + half * kLmC + r32;
+#pragma unroll
+    for (int i = 0; i < kLmK / 2; ++i) {
+      const float bv = bp[2 * i * kLmC];
+#pragma unroll
+      for (int j = 0; j < kLmS / 32; ++j)
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[j * 32 * kLmPitch + 2 * i], bv, acc[j], 0,
+                                                      0, 0);
     }
   }
-  if (c0 >= C) return;
+
+  // the partial sums meet: [wave][96][33] in the slab space
+  __syncthreads();
+  float *part = lm_lds + wave * (kLmS * kLmPitch);
 #pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const int t = t_tile + 8 * (v / 4) + 4 * half + (v % 4);
-    if (t >= T) continue;
-    float gsum = __expf(am_tc[v] - amx[t]) * acc[v] + hot[v];
-    if (c0 == term) gsum += col_y[(long)b * T + t];
-    am_grad[((long)b * T + t) * C + c0] = gsum;
+  for (int j = 0; j < kLmS / 32; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+      part[(32 * j + 8 * (v / 4) + 4 * half + (v % 4)) * kLmPitch + r32] = acc[j][v];
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kLmItems; ++j) {
+    const int item = tid + kLmThreads * j;
+    const int m = item / 8, n = 4 * (item % 8), sr = s_tile + m, c = c_tile + n;
+    if (sr >= S1 || c >= C) continue;
+    const float mx = lmx[sr];
+    const int sym = sr < S ? (int)symbols[(long)b * S + sr] : -1;
+    const float rx = row_x[(long)b * S1 + sr], ry = row_y[(long)b * S1 + sr];
+    float g[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < kLmWaves; ++w)
+        sum += lm_lds[w * (kLmS * kLmPitch) + m * kLmPitch + n + i];
+      g[i] = __expf(lm_in[j][i] - mx) * sum;
+      if (c + i == sym) g[i] += rx;
+      if (c + i == term) g[i] += ry;
+    }
+    float *dst = lm_grad + ((long)b * S1 + sr) * C + c;
+    if (c + 4 <= C) {
+      *reinterpret_cast<floatx4u *>(dst) = floatx4u{g[0], g[1], g[2], g[3]};
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (c + i < C) dst[i] = g[i];
+    }
   }
 }
 
@@ -962,7 +843,6 @@ __global__ void __launch_bounds__(256)
 constexpr int kAmT = 64;       // frames per workgroup
 constexpr int kAmC = 64;       // vocabulary entries per workgroup
 constexpr int kAmRows = 96;    // lattice rows per LDS pass (even)
-constexpr int kAmPairs = kAmRows / 2;
 constexpr int kAmOutPitch = 68;  // row pitch of the result tiles staged in LDS
 constexpr int kAmQ = kAmT / 4;   // 16-byte pieces per panel row (kAmT == kAmC)
 
@@ -1152,12 +1032,12 @@ void launch_bwd_lm(const float *lm, const float *am, const int64_t *symbols, con
                    const float *am_max, const float *dmat, const float *row_x, const float *row_y,
                    float *lm_grad, int B, int S, int T, int C, int ldd, int term,
                    hipStream_t stream) {
-  const int tiles = ((C + dgemm::kBN - 1) / dgemm::kBN) * ((S + 1 + dgemm::kBM - 1) / dgemm::kBM);
-  const bool vec = (ldd % 4 == 0) && aligned16(dmat);
-  auto kernel = vec ? simple_bwd_lm_direct_kernel<true> : simple_bwd_lm_direct_kernel<false>;
-  hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(tiles, B)), dim3(kLmWaves * kWave), 0, stream,
-                     lm, am, symbols, lm_max, am_max, dmat, row_x, row_y, lm_grad, B, S, T, C, ldd,
-                     term);
+  const int tiles = ((C + kLmC - 1) / kLmC) * ((S + 1 + kLmS - 1) / kLmS);
+  auto kernel = simple_bwd_lm_slab_kernel;
+  (void)allow_lds(reinterpret_cast<const void *>(kernel), kLmLdsBytes);
+  hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(tiles, B)), dim3(kLmThreads), kLmLdsBytes,
+                     stream, lm, am, symbols, lm_max, am_max, dmat, row_x, row_y, lm_grad, B, S, T,
+                     C, ldd, term);
 }
 void launch_bwd_lm(const double *lm, const double *am, const int64_t *symbols,
                    const double *lm_max, const double *am_max, const double *dmat,
@@ -1175,9 +1055,8 @@ void launch_bwd_am(const float *lm, const float *am, const int64_t *symbols,
   // rows of k held in LDS per pass: all of them when they fit
   const int rows_cap = std::min(kAmRows, (S + 2) & ~1);
   const size_t lds = am_panel_lds_bytes(rows_cap);
-  // (the 16-byte accesses need no alignment; the scalar variant exists for checking)
-  const bool vec = true;
-  auto kernel = vec ? simple_bwd_am_panel_kernel<true> : simple_bwd_am_panel_kernel<false>;
+  // (the 16-byte accesses need no alignment)
+  auto kernel = simple_bwd_am_panel_kernel<true>;
   (void)allow_lds(reinterpret_cast<const void *>(kernel), lds);
   hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(tiles, B)), dim3(256), lds, stream, lm, am,
                      symbols, boundary, lm_max, am_max, dmat, gpx, col_y, am_grad, B, S, T, C, ldd,
