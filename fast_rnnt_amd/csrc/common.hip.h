@@ -56,23 +56,9 @@ __device__ __forceinline__ R log_add(R a, R b) {
   return hi + Num<R>::log1p_(Num<R>::exp_(gap));
 }
 
-// Value held by lane-1 (whole-wave shift right by one); lane 0 receives `fill`.
-// DPP wave_shr:1 is a full-rate VALU modifier on gfx9-family parts, no LDS trip.
-__device__ __forceinline__ float from_lane_below(float v, float fill) {
-  const int r = __builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(v), 0x138, 0xf,
-                                            0xf, false);
-  return __int_as_float(r);
-}
-__device__ __forceinline__ double from_lane_below(double v, double fill) {
-  const long long vi = __double_as_longlong(v), fi = __double_as_longlong(fill);
-  const int lo = __builtin_amdgcn_update_dpp((int)(fi & 0xffffffffLL), (int)(vi & 0xffffffffLL),
-                                             0x138, 0xf, 0xf, false);
-  const int hi = __builtin_amdgcn_update_dpp((int)(fi >> 32), (int)(vi >> 32), 0x138, 0xf, 0xf,
-                                             false);
-  return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
-}
-
-// Same shift with lane 0 receiving 0: in this form the compiler can fold the
+// Whole-wave shift right by one (DPP wave_shr:1, a full-rate VALU modifier on
+// gfx9-family parts, no LDS trip): lane L receives the value held by lane L-1.
+// With lane 0 receiving 0 the compiler can fold the
 // shift into the consuming VALU instruction.
 __device__ __forceinline__ float from_lane_below_zero(float v) {
   return __int_as_float(
@@ -109,17 +95,6 @@ __device__ __forceinline__ double from_lane_above(double v) {
   const long long vi = __double_as_longlong(v);
   const int lo = __builtin_amdgcn_update_dpp(0, (int)(vi & 0xffffffffLL), 0x130, 0xf, 0xf, true);
   const int hi = __builtin_amdgcn_update_dpp(0, (int)(vi >> 32), 0x130, 0xf, 0xf, true);
-  return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
-}
-
-// Broadcast of lane `src`'s value (src wave-uniform).
-__device__ __forceinline__ float lane_value(float v, int src) {
-  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src));
-}
-__device__ __forceinline__ double lane_value(double v, int src) {
-  const long long vi = __double_as_longlong(v);
-  const int lo = __builtin_amdgcn_readlane((int)(vi & 0xffffffffLL), src);
-  const int hi = __builtin_amdgcn_readlane((int)(vi >> 32), src);
   return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
 }
 

@@ -5,14 +5,20 @@
 // local step e lane L works on column e - L, so the neighbour in the previous
 // row is what lane L-1 produced one step earlier (regular lattice) or two steps
 // earlier (modified lattice) and arrives through a DPP wave shift, and the
-// neighbour in the same row is the lane's own previous result.  Nothing but this
-// dependent chain runs on a sweep wave: all HBM traffic is done by *staging
-// waves* of the same workgroup, which fetch px/py (forward) or p/px (backward)
-// with coalesced row loads, turn them into diagonal ("sheared") 64-row x 32-step
-// tiles in LDS, and -- for the backward sweep -- also evaluate the exp() of the
-// gradient split and write the finished gradient tiles back to HBM.  Tiles are
-// double buffered; sweep and staging waves meet only through monotone LDS
-// counters (acquire/release, bounded spinning), never at a barrier.
+// neighbour in the same row is the lane's own previous result.
+//
+// A single wave issues about one instruction every 4.5 cycles and nothing overlaps
+// within it, so a sweep wave's time is its instruction count: everything that is not
+// the dependent chain is kept off it.  *Staging waves* of the same workgroup fetch
+// px/py (forward) or p/px (backward) with coalesced, range-checked row loads, turn
+// them into diagonal ("sheared") 64-row x 32-step tiles in LDS and -- for the
+// backward sweep -- also evaluate the exp() of the gradient split; the sweep wave
+// pulls a tile into registers with 16-byte LDS reads.  Results leave the sweep wave
+// as 16-byte row segments through range-checked buffer stores (an out-of-window
+// lane's store is dropped by the hardware instead of being branched around).
+// Tiles are double buffered; sweep and staging waves meet only through monotone
+// LDS counters (acquire/release, bounded spinning), never at a barrier, and the
+// sweep wave looks at a counter one chunk (one tile) before it needs it.
 //
 // Rows beyond 64 go to further sweep waves; wave w+1 consumes the last row of
 // wave w through an LDS seam row guarded by a progress counter and simply runs a

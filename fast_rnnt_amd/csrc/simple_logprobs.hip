@@ -20,7 +20,7 @@
 //                   + sum_s [c = sym[b,s]] gx[s,t] + [c = term] sum_s gy[s,t]
 // i.e. two more GEMMs with the same fused-exp loaders (what autograd derives for
 // rnnt_loss.py:174-220; the derivatives through the two max() cancel).
-#include "direct_gemm.hip.h"
+#include "xcd_grid.hip.h"
 #include "tile_gemm.hip.h"
 
 namespace frnnt {
@@ -384,7 +384,7 @@ __device__ __forceinline__ dgemm::floatx4 load4_guarded(const float *base, int o
   return r;
 }
 
-// ---- fp32: register-direct MFMA kernels (direct_gemm.hip.h) ------------------------
+// ---- fp32: MFMA kernels with LDS slabs / panels (xcd_grid.hip.h) --------------------
 
 // Normalizer GEMM, wave-private LDS transposition.  Both operands are k-contiguous
 // ([rows][C]), the matrix cores want one row per lane.  Letting every lane fetch its
@@ -1002,7 +1002,7 @@ __global__ void __launch_bounds__(256, 2)
   }
 }
 
-// launchers: float goes to the register-direct kernels, double to the LDS-tiled ones
+// launchers: float goes to the slab / panel kernels, double to the LDS-tiled ones
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 void launch_fwd_gemm(const float *lm, const float *am, const int64_t *symbols,
