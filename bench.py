@@ -38,7 +38,7 @@ def _parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c4"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0,
                     help="budget of the CPU-baseline leg (0 disables it)")
     ap.add_argument("--kernel-reps", type=int, default=50)
@@ -76,6 +76,109 @@ def _recursion_bytes(boundary, S, T, B, backward):
     return 4 * win + 4 * (B * S * (T + 1) + B * (S + 1) * T) + 4 * B + 32 * B
 
 
+def _bench_lattice(args, w, dev):
+    """c3 (pruned pipeline) and c5 (unpruned loss on full logits): HBM-streaming
+    workloads whose dominant kernel is the logits-gradient kernel."""
+    import fast_rnnt_amd
+    from fast_rnnt_amd import _lib
+
+    sym, bnd = w.symbols.to(dev), w.boundary.to(dev)
+    if w.name == "c5":
+        logits = w.logits.to(dev).requires_grad_(True)
+
+        def step():
+            logits.grad = None
+            loss = fast_rnnt_amd.rnnt_loss(logits, sym, 0, boundary=bnd, reduction="sum")
+            loss.backward()
+            return loss
+
+        ranges, R = None, w.S + 1
+        lg = logits.detach()
+        what = (f"c5: rnnt_loss fwd+bwd on logits [B,T,S+1,C], B={w.B} T={w.T} S={w.S} C={w.C}, "
+                "ragged boundary, reduction=sum")
+    else:
+        am = w.am.to(dev).requires_grad_(True)
+        lm = w.lm.to(dev).requires_grad_(True)
+        W = w.joiner.to(dev)
+
+        def step():
+            am.grad = None
+            lm.grad = None
+            simple, (gx, gy) = fast_rnnt_amd.rnnt_loss_smoothed(
+                lm, am, sym, 0, 0.25, 0.0, boundary=bnd, reduction="sum", return_grad=True)
+            rg = fast_rnnt_amd.get_rnnt_prune_ranges(gx, gy, bnd, w.s_range)
+            am_p, lm_p = fast_rnnt_amd.do_rnnt_pruning(am, lm, rg)
+            loss = fast_rnnt_amd.rnnt_loss_pruned(torch.tanh(am_p + lm_p) @ W, sym, rg, 0,
+                                                  boundary=bnd, reduction="sum")
+            (simple + loss).backward()
+            return loss
+
+        with torch.no_grad():
+            _, (gx, gy) = fast_rnnt_amd.rnnt_loss_smoothed(
+                lm, am, sym, 0, 0.25, 0.0, boundary=bnd, reduction="sum", return_grad=True)
+            ranges = fast_rnnt_amd.get_rnnt_prune_ranges(gx, gy, bnd, w.s_range)
+            am_p, lm_p = fast_rnnt_amd.do_rnnt_pruning(am, lm, ranges)
+            lg = (torch.tanh(am_p + lm_p) @ W).contiguous()
+        R = w.s_range
+        what = (f"c3: rnnt_loss_smoothed -> get_rnnt_prune_ranges -> do_rnnt_pruning -> joiner -> "
+                f"rnnt_loss_pruned fwd+bwd, B={w.B} T={w.T} S={w.S} C={w.C} s_range={w.s_range}")
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    # the two logits kernels alone, through the C ABI, with events on the launch stream
+    B, S, T, C = w.B, w.S, w.T, w.C
+    T1 = T + 1
+    f32 = dict(dtype=torch.float32, device=dev)
+    px, py = torch.empty(B, S, T1, **f32), torch.empty(B, S + 1, T, **f32)
+    norm, xr, yr = (torch.empty(B, T, R, **f32) for _ in range(3))
+    gpx, gpy = torch.rand(B, S, T1, **f32), torch.rand(B, S + 1, T, **f32)
+    grad = torch.empty_like(lg)
+    stream = torch.cuda.current_stream().cuda_stream
+    rp = _lib.ptr(ranges)
+
+    def fwd():
+        _lib.call("frnnt_lattice_logprobs_fwd_f32", lg.data_ptr(), sym.data_ptr(), rp,
+                  bnd.data_ptr(), px.data_ptr(), py.data_ptr(), norm.data_ptr(), xr.data_ptr(),
+                  yr.data_ptr(), B, S, T, R, C, 0, 0, stream)
+
+    def bwd():
+        _lib.call("frnnt_lattice_logprobs_bwd_f32", lg.data_ptr(), sym.data_ptr(), rp,
+                  bnd.data_ptr(), norm.data_ptr(), gpx.data_ptr(), gpy.data_ptr(), grad.data_ptr(),
+                  B, S, T, R, C, 0, 0, stream)
+
+    t_f = _event_time_ms(fwd, args.kernel_reps)
+    t_b = _event_time_ms(bwd, args.kernel_reps)
+    nbytes = lg.numel() * 4
+
+    def line(kernel, b, t_ms):
+        a = b / (t_ms * 1e-3) / 1e9
+        return {"kernel": kernel, "bound": "hbm", "achieved": round(a, 1), "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(a / HBM_PEAK_GBS, 4), "traffic": None,
+                "algorithmic_bytes": b, "avg_launch_us": round(1e3 * t_ms, 2)}
+
+    out = {
+        "metric": "fwd+bwd loss calls/sec + achieved HBM GB/s",
+        "value": round(args.steps / elapsed, 2), "unit": "calls/sec", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(1e3 * elapsed / args.steps, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": what, "logits_bytes": nbytes},
+        # one read and one write of the logits (gradient kernel); one read (normalizer kernel,
+        # whose entry point also runs the small px/py assembly kernel)
+        "roofline": line("row_grad_kernel<float>", 2 * nbytes, t_b),
+        "roofline_other_kernels": [line("row_norm_kernel<float> (+ assemble_kernel)", nbytes, t_f)],
+        "cpu_baseline": None,
+    }
+    print(json.dumps(out))
+
+
 def main():
     args = _parse()
     if args.gpus != 1:
@@ -94,6 +197,9 @@ def main():
     _lib.load()
     dev = torch.device("cuda", 0)
     w = workloads.make(args.workload)
+    if w.name in ("c3", "c5"):
+        _bench_lattice(args, w, dev)
+        return
     am = w.am.to(dev).requires_grad_(True)
     lm = w.lm.to(dev).requires_grad_(True)
     sym = w.symbols.to(dev)

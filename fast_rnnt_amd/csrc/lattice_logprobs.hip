@@ -100,6 +100,79 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// The same with the row held in registers (fp32, C a multiple of 4, at most
+// 256 * kVecs entries): the logits are read once, 16 bytes per lane and load.
+typedef float floatx4u __attribute__((ext_vector_type(4), aligned(4)));
+template <int kVecs>
+__global__ void __launch_bounds__(256)
+    row_norm_regs_kernel(const float *__restrict__ logits, const int64_t *__restrict__ symbols,
+                         const int64_t *__restrict__ ranges, float *__restrict__ norm,
+                         float *__restrict__ xr, float *__restrict__ yr, long rows, int T, int Rr,
+                         int S, int C, int term) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const float *x = logits + row * C;
+  const float ninf = -__builtin_huge_valf();
+  floatx4u v[kVecs];
+#pragma unroll
+  for (int i = 0; i < kVecs; ++i) {
+    const int c = 4 * (lane + kWave * i);
+    v[i] = floatx4u{ninf, ninf, ninf, ninf};
+    if (c < C) v[i] = *reinterpret_cast<const floatx4u *>(x + c);
+  }
+  float m = ninf;
+#pragma unroll
+  for (int i = 0; i < kVecs; ++i)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) m = (v[i][e] > m || v[i][e] != v[i][e]) ? v[i][e] : m;
+  m = wave_max_all(m);
+  const float shift = (m - m == 0) ? m : 0.f;  // torch.logsumexp: infinite max -> shift by 0
+  float sum = 0;
+#pragma unroll
+  for (int i = 0; i < kVecs; ++i)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sum += __expf(v[i][e] - shift);  // padding is -inf: adds 0
+  sum = wave_sum_all(sum);
+  const float lse = logf(sum) + shift;
+  if (lane == 0) {
+    const int j = (int)(row % Rr);
+    const int b = (int)(row / ((long)Rr * T));
+    const int64_t sym = row_symbol(symbols, ranges, row, b, j, S, term);
+    norm[row] = lse;
+    xr[row] = (sym >= 0 && sym < C) ? x[sym] - lse : std::numeric_limits<float>::quiet_NaN();
+    yr[row] = x[term] - lse;
+  }
+}
+
+template <typename R>
+bool launch_row_norm_regs(const R *, const int64_t *, const int64_t *, R *, R *, R *, long, int, int,
+                          int, int, int, hipStream_t) {
+  return false;
+}
+template <>
+bool launch_row_norm_regs<float>(const float *logits, const int64_t *symbols, const int64_t *ranges,
+                                 float *norm, float *xr, float *yr, long rows, int T, int Rr, int S,
+                                 int C, int term, hipStream_t stream) {
+  if (C % 4 != 0 || C > 256 * 16) return false;
+  const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+#define FRNNT_ROW_NORM(V)                                                                        \
+  hipLaunchKernelGGL(row_norm_regs_kernel<V>, grid, block, 0, stream, logits, symbols, ranges,   \
+                     norm, xr, yr, rows, T, Rr, S, C, term)
+  if (C <= 256)
+    FRNNT_ROW_NORM(1);
+  else if (C <= 512)
+    FRNNT_ROW_NORM(2);
+  else if (C <= 1024)
+    FRNNT_ROW_NORM(4);
+  else if (C <= 2048)
+    FRNNT_ROW_NORM(8);
+  else
+    FRNNT_ROW_NORM(16);
+#undef FRNNT_ROW_NORM
+  return true;
+}
+
 // One thread per px / py element, t fastest (coalesced stores).
 template <typename R>
 __global__ void __launch_bounds__(256)
@@ -200,8 +273,10 @@ int fwd_impl(const R *logits, const int64_t *symbols, const int64_t *ranges,
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   const long rows = (long)B * T * Rr;
   if (rows > 0)
-    hipLaunchKernelGGL(row_norm_kernel<R>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream,
-                       logits, symbols, ranges, norm, xr, yr, rows, T, Rr, S, C, term);
+    if (!launch_row_norm_regs<R>(logits, symbols, ranges, norm, xr, yr, rows, T, Rr, S, C, term,
+                                 stream))
+      hipLaunchKernelGGL(row_norm_kernel<R>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                         stream, logits, symbols, ranges, norm, xr, yr, rows, T, Rr, S, C, term);
   const int T1 = rnnt_type == kRegular ? T + 1 : T;
   const long total = (long)B * S * T1 + (long)B * (S + 1) * T;
   if (total > 0)

@@ -7,8 +7,9 @@
 // ties resolved to the first maximum, replace the starts of frames at or beyond
 // T_b - 1 by max(S_b - R + 1, 0), then make the starts non-decreasing, starting
 // at 0, with steps smaller than r (r = R for the regular lattice, 2 otherwise)
-// by two suffix-minimum passes.  One wave per utterance; the per-frame starts
-// live in LDS and the suffix minima are a chunked wave scan.
+// by two suffix-minimum passes.  Two kernels: one lane per frame for the window
+// starts (left in ranges[b][t][0]), then one wave per utterance for the two passes,
+// with the starts in LDS and the suffix minima as a chunked wave scan.
 //
 // prune_gather (rnnt_loss.py:780-818): lm_pruned[b,t,j,:] = lm[b, ranges[b,t,j], :]
 // and its adjoint, a deterministic segmented sum (one block per lm row).
@@ -46,37 +47,58 @@ __device__ __forceinline__ void suffix_min_inplace(int *v, int n, int lane) {
   __syncthreads();
 }
 
+// Step 1, one lane per frame: the best window start of frame (b, t), left in
+// ranges[b][t][0].
 template <typename R>
 __global__ void __launch_bounds__(kWave)
-    prune_ranges_kernel(const R *__restrict__ px_grad, const R *__restrict__ py_grad,
+    prune_starts_kernel(const R *__restrict__ px_grad, const R *__restrict__ py_grad,
                         const int64_t *__restrict__ boundary, int64_t *__restrict__ ranges, int S,
                         int T, int T1, int Rr) {
-  extern __shared__ int start[];  // [T]
-  const int b = blockIdx.x, lane = threadIdx.x;
-  const R *gx = px_grad + (long)b * S * T1;
-  const R *gy = py_grad + (long)b * (S + 1) * T;
+  const int b = blockIdx.y, t = blockIdx.x * kWave + threadIdx.x;
+  if (t >= T) return;
+  const R *gx = px_grad + (long)b * S * T1 + t;
+  const R *gy = py_grad + (long)b * (S + 1) * T + t;
   const int n = S + 2 - Rr;  // candidate window starts
   const int64_t Sb = boundary[4 * b + 2], Tb = boundary[4 * b + 3];
   int64_t tail = Sb - Rr + 1;
   if (tail < 0) tail = 0;
-  for (int t = lane; t < T; t += kWave) {
-    int best = 0;
-    R best_score = 0;
-    for (int s = 0; s < n; ++s) {
-      R sum = gy[(long)s * T + t];
-      for (int j = 1; j < Rr; ++j) sum = sum + gy[(long)(s + j) * T + t];
-      const R below = s >= 1 ? gx[(long)(s - 1) * T1 + t] : (R)0;
-      const R score = sum - below;
-      // first maximum wins; a NaN score counts as the maximum, like torch.argmax
-      if (s == 0 || score > best_score || (score != score && best_score == best_score)) {
-        best = s;
-        best_score = score;
-      }
+  int best = 0;
+  R best_score = 0;
+  // first maximum wins; a NaN score counts as the maximum, like torch.argmax
+  auto consider = [&](int s, R score) {
+    if (s == 0 || score > best_score || (score != score && best_score == best_score)) {
+      best = s;
+      best_score = score;
     }
-    start[t] = ((int64_t)t < Tb - 1) ? best : (int)tail;
+  };
+  auto score_of = [&](int s) {
+    R sum = gy[(long)s * T];
+    for (int j = 1; j < Rr; ++j) sum = sum + gy[(long)(s + j) * T];
+    const R below = s >= 1 ? gx[(long)(s - 1) * T1] : (R)0;
+    return sum - below;
+  };
+  int s = 0;
+  for (; s + 4 <= n; s += 4) {
+    // four independent windows in flight
+    const R a0 = score_of(s), a1 = score_of(s + 1), a2 = score_of(s + 2), a3 = score_of(s + 3);
+    consider(s, a0);
+    consider(s + 1, a1);
+    consider(s + 2, a2);
+    consider(s + 3, a3);
   }
+  for (; s < n; ++s) consider(s, score_of(s));
+  ranges[((long)b * T + t) * Rr] = ((int64_t)t < Tb - 1) ? (int64_t)best : tail;
+}
+
+// Step 2, one wave per utterance: the starts are made non-decreasing with bounded
+// steps by two suffix-minimum passes and expanded to the R entries of each frame.
+__global__ void __launch_bounds__(kWave)
+    prune_monotone_kernel(int64_t *__restrict__ ranges, int T, int r, int Rr) {
+  extern __shared__ int start[];  // [T]
+  const int b = blockIdx.x, lane = threadIdx.x;
+  int64_t *rb = ranges + (long)b * T * Rr;
+  for (int t = lane; t < T; t += kWave) start[t] = (int)rb[(long)t * Rr];
   __syncthreads();
-  const int r = (T1 != T) ? Rr : 2;
   suffix_min_inplace(start, T, lane);
   for (int t = lane; t < T; t += kWave) start[t] = (r - 1) * t - start[t];
   __syncthreads();
@@ -84,7 +106,7 @@ __global__ void __launch_bounds__(kWave)
   for (int t = lane; t < T; t += kWave) {
     const int y = max(start[t], 0);
     const int64_t s0 = (int64_t)(r - 1) * t - y;
-    int64_t *out = ranges + ((long)b * T + t) * Rr;
+    int64_t *out = rb + (long)t * Rr;
     for (int j = 0; j < Rr; ++j) out[j] = s0 + j;
   }
 }
@@ -108,22 +130,72 @@ __global__ void __launch_bounds__(256)
   for (int c = lane; c < C; c += kWave) dst[c] = src[c];
 }
 
-// adjoint: one block per lm row (b, s); frames are visited in order, so the sum
-// is deterministic
+// adjoint: one block per lm row (b, s).  The block first lists, in order, the entries
+// of ranges[b] that point at s (an ordered compaction through LDS; only a few dozen of
+// the T * R entries match), then sums those rows of the incoming gradient -- in that
+// order, so the result is deterministic -- with coalesced loads.
+constexpr int kHitCapacity = 4096;  // matches listed per round
+
 template <typename R>
 __global__ void __launch_bounds__(256)
     prune_scatter_kernel(const R *__restrict__ grad, const int64_t *__restrict__ ranges,
                          R *__restrict__ lm_grad, int TR, int S1, int C) {
+  __shared__ int hits[kHitCapacity];
+  __shared__ int wave_count[4];
+  __shared__ int listed;
   const int b = blockIdx.x / S1, s = blockIdx.x % S1;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t *rb = ranges + (long)b * TR;
   const R *gb = grad + (long)b * TR * C;
-  for (int c0 = 0; c0 < C; c0 += 256) {
-    const int c = c0 + threadIdx.x;
-    R acc = 0;
-    for (int k = 0; k < TR; ++k)
-      if (rb[k] == s && c < C) acc += gb[(long)k * C + c];
-    if (c < C) lm_grad[((long)b * S1 + s) * C + c] = acc;
-  }
+  R *dst = lm_grad + ((long)b * S1 + s) * C;
+  bool first_round = true;
+  int k_next = 0;
+  // rounds only repeat when more than kHitCapacity entries point at s
+  do {
+    if (tid == 0) listed = 0;
+    __syncthreads();
+    int k0 = k_next;
+    for (; k0 < TR; k0 += 256) {
+      const int k = k0 + tid;
+      const bool hit = k < TR && rb[k] == s;
+      const unsigned long long mask = __ballot(hit);
+      if (lane == 0) wave_count[wave] = __popcll(mask);
+      __syncthreads();
+      const int base = listed;
+      int before = 0, total = 0;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        if (w < wave) before += wave_count[w];
+        total += wave_count[w];
+      }
+      if (base + total > kHitCapacity) break;  // (uniform) this chunk waits for the next round
+      if (hit) hits[base + before + __popcll(mask & ((1ull << lane) - 1ull))] = k;
+      __syncthreads();
+      if (tid == 0) listed = base + total;
+      __syncthreads();
+    }
+    k_next = k0;
+    __syncthreads();
+    const int n = listed;
+    for (int c0 = 0; c0 < C; c0 += 256) {
+      const int c = c0 + tid;
+      if (c >= C) continue;
+      R acc = first_round ? (R)0 : dst[c];
+      int i = 0;
+      for (; i + 4 <= n; i += 4) {
+        const R g0 = gb[(long)hits[i] * C + c], g1 = gb[(long)hits[i + 1] * C + c];
+        const R g2 = gb[(long)hits[i + 2] * C + c], g3 = gb[(long)hits[i + 3] * C + c];
+        acc += g0;
+        acc += g1;
+        acc += g2;
+        acc += g3;
+      }
+      for (; i < n; ++i) acc += gb[(long)hits[i] * C + c];
+      dst[c] = acc;
+    }
+    first_round = false;
+    __syncthreads();
+  } while (k_next < TR);
 }
 
 template <typename R>
@@ -137,11 +209,14 @@ int ranges_impl(const R *px_grad, const R *py_grad, const int64_t *boundary, int
     return fail(FRNNT_EINVAL, "prune_ranges: null pointer");
   const size_t lds = (size_t)T * sizeof(int);
   if (lds > 150 * 1024) return fail(FRNNT_ELIMIT, "prune_ranges: T=%d exceeds the LDS table", T);
-  auto kernel = prune_ranges_kernel<R>;
-  if (!allow_lds(reinterpret_cast<const void *>(kernel), lds))
+  if (!allow_lds(reinterpret_cast<const void *>(prune_monotone_kernel), lds))
     return check_launch("prune_ranges: hipFuncSetAttribute");
-  hipLaunchKernelGGL(kernel, dim3(B), dim3(kWave), lds, static_cast<hipStream_t>(stream), px_grad,
-                     py_grad, boundary, ranges, S, T, modified ? T : T + 1, s_range);
+  const int T1 = modified ? T : T + 1;
+  hipLaunchKernelGGL(prune_starts_kernel<R>, dim3((T + kWave - 1) / kWave, B), dim3(kWave), 0,
+                     static_cast<hipStream_t>(stream), px_grad, py_grad, boundary, ranges, S, T,
+                     T1, s_range);
+  hipLaunchKernelGGL(prune_monotone_kernel, dim3(B), dim3(kWave), lds,
+                     static_cast<hipStream_t>(stream), ranges, T, modified ? 2 : s_range, s_range);
   return check_launch("prune_ranges");
 }
 

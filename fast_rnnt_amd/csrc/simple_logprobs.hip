@@ -583,7 +583,8 @@ __global__ void __launch_bounds__(kPanThreads)
     my_max = slab_max[kPanS + tid - 128];
   }
 
-  // ---- main loop over this wave's slabs
+  // ---- main loop over this wave's slabs (32-row tiles without lattice rows are skipped)
+  const int live_tiles = min(kPanS / 32, (S1 - s_tile + 31) / 32);
   float *mine = pan_lds + wave * kPanSlab;
   floatx16 acc[kPanS / 32];
 #pragma unroll
@@ -605,8 +606,9 @@ __global__ void __launch_bounds__(kPanThreads)
       const float bv = bp[2 * i];
 #pragma unroll
       for (int j = 0; j < kPanS / 32; ++j)
-        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[j * 32 * kPanPitch + 2 * i], bv, acc[j],
-                                                      0, 0, 0);
+        if (j < live_tiles)
+          acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[j * 32 * kPanPitch + 2 * i], bv, acc[j],
+                                                        0, 0, 0);
     }
   }
 
@@ -752,6 +754,7 @@ __global__ void __launch_bounds__(kLmThreads, 2)
     lm_in[j] = load4_guarded<true>(lmb, sr * C + c, sr < S1 ? min(4, max(C - c, 0)) : 0);
   }
 
+  const int live_tiles = min(kLmS / 32, (S1 - s_tile + 31) / 32);  // 32-row tiles with lattice rows
   float *as = lm_lds + wave * kLmSlab;
   float *bs = as + kLmS * kLmPitch;
   floatx16 acc[kLmS / 32];
@@ -781,8 +784,9 @@ __global__ void __launch_bounds__(kLmThreads, 2)
       const float bv = bp[2 * i * kLmC];
 #pragma unroll
       for (int j = 0; j < kLmS / 32; ++j)
-        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[j * 32 * kLmPitch + 2 * i], bv, acc[j], 0,
-                                                      0, 0);
+        if (j < live_tiles)
+          acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[j * 32 * kLmPitch + 2 * i], bv, acc[j],
+                                                        0, 0, 0);
     }
   }
 
