@@ -172,8 +172,8 @@ def _bench_lattice(args, w, dev):
         "config": {"workload": what, "logits_bytes": nbytes},
         # one read and one write of the logits (gradient kernel); one read (normalizer kernel,
         # whose entry point also runs the small px/py assembly kernel)
-        "roofline": line("row_grad_kernel<float>", 2 * nbytes, t_b),
-        "roofline_other_kernels": [line("row_norm_kernel<float> (+ assemble_kernel)", nbytes, t_f)],
+        "roofline": line("row_grad_regs_kernel", 2 * nbytes, t_b),
+        "roofline_other_kernels": [line("row_norm_regs_kernel (+ assemble_kernel)", nbytes, t_f)],
         "cpu_baseline": None,
     }
     print(json.dumps(out))

@@ -256,6 +256,95 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// The same with the row held in registers (fp32, C a multiple of 4, at most
+// 256 * kVecs entries): the logits are requested first, 16 bytes per lane and load,
+// so that they travel while the row's scalars (range, gradients, normalizer) are
+// looked up; the gradient leaves as 16-byte stores.
+template <int kVecs>
+__global__ void __launch_bounds__(256)
+    row_grad_regs_kernel(const float *__restrict__ logits, const int64_t *__restrict__ symbols,
+                         const int64_t *__restrict__ ranges, const int64_t *__restrict__ boundary,
+                         const float *__restrict__ norm, const float *__restrict__ gpx,
+                         const float *__restrict__ gpy, float *__restrict__ glogits, long rows,
+                         int S, int T, int Rr, int C, int term, int rnnt_type) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const float *x = logits + row * C;
+  floatx4u v[kVecs];
+#pragma unroll
+  for (int i = 0; i < kVecs; ++i) {
+    const int c = 4 * (lane + kWave * i);
+    v[i] = floatx4u{0.f, 0.f, 0.f, 0.f};
+    if (c < C) v[i] = *reinterpret_cast<const floatx4u *>(x + c);
+  }
+  const int S1 = S + 1;
+  const int T1 = rnnt_type == kRegular ? T + 1 : T;
+  const int j = (int)(row % Rr);
+  const long frame = row / Rr;
+  const int t = (int)(frame % T), b = (int)(frame / T);
+  const int64_t r0 = ranges ? ranges[frame * Rr] : 0;
+  int64_t s64 = ((int64_t)j + r0) % S1;
+  if (s64 < 0) s64 += S1;
+  const int s = (int)s64;
+  const bool masked = rnnt_type == kRegular && boundary && boundary[4 * b + 3] == t;
+  auto gx_at = [&](int ss) -> float {
+    if (ss < 0 || ss >= S || masked) return 0.f;
+    return gpx[((long)b * S + ss) * T1 + t];
+  };
+  const float gx = gx_at(s);
+  float gy = gpy[((long)b * S1 + s) * T + t];
+  if (rnnt_type == kConstrained) gy += gx_at(s - 1);
+  const int sym = (int)row_symbol(symbols, ranges, row, b, j, S, term);
+  const float lse = norm[row];
+  const float w = -(gx + gy);
+  float *g = glogits + row * C;
+#pragma unroll
+  for (int i = 0; i < kVecs; ++i) {
+    const int c = 4 * (lane + kWave * i);
+    if (c >= C) continue;
+    floatx4u o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float r = __expf(v[i][e] - lse) * w;
+      if (c + e == sym) r += gx;
+      if (c + e == term) r += gy;
+      o[e] = r;
+    }
+    *reinterpret_cast<floatx4u *>(g + c) = o;
+  }
+}
+
+template <typename R>
+bool launch_row_grad_regs(const R *, const int64_t *, const int64_t *, const int64_t *, const R *,
+                          const R *, const R *, R *, long, int, int, int, int, int, int,
+                          hipStream_t) {
+  return false;
+}
+template <>
+bool launch_row_grad_regs<float>(const float *logits, const int64_t *symbols, const int64_t *ranges,
+                                 const int64_t *boundary, const float *norm, const float *gpx,
+                                 const float *gpy, float *glogits, long rows, int S, int T, int Rr,
+                                 int C, int term, int rnnt_type, hipStream_t stream) {
+  if (C % 4 != 0 || C > 256 * 16) return false;
+  const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+#define FRNNT_ROW_GRAD(V)                                                                        \
+  hipLaunchKernelGGL(row_grad_regs_kernel<V>, grid, block, 0, stream, logits, symbols, ranges,   \
+                     boundary, norm, gpx, gpy, glogits, rows, S, T, Rr, C, term, rnnt_type)
+  if (C <= 256)
+    FRNNT_ROW_GRAD(1);
+  else if (C <= 512)
+    FRNNT_ROW_GRAD(2);
+  else if (C <= 1024)
+    FRNNT_ROW_GRAD(4);
+  else if (C <= 2048)
+    FRNNT_ROW_GRAD(8);
+  else
+    FRNNT_ROW_GRAD(16);
+#undef FRNNT_ROW_GRAD
+  return true;
+}
+
 template <typename R>
 int fwd_impl(const R *logits, const int64_t *symbols, const int64_t *ranges,
              const int64_t *boundary, R *px, R *py, R *norm, R *xr, R *yr, int B, int S, int T,
@@ -298,9 +387,12 @@ int bwd_impl(const R *logits, const int64_t *symbols, const int64_t *ranges,
   if (!logits || (!symbols && S > 0) || !norm || !px_grad || !py_grad || !logits_grad)
     return fail(FRNNT_EINVAL, "lattice_logprobs_bwd: null pointer");
   const long rows = (long)B * T * Rr;
-  hipLaunchKernelGGL(row_grad_kernel<R>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
-                     static_cast<hipStream_t>(stream_), logits, symbols, ranges, boundary, norm,
-                     px_grad, py_grad, logits_grad, rows, S, T, Rr, C, term, rnnt_type);
+  if (!launch_row_grad_regs<R>(logits, symbols, ranges, boundary, norm, px_grad, py_grad,
+                               logits_grad, rows, S, T, Rr, C, term, rnnt_type,
+                               static_cast<hipStream_t>(stream_)))
+    hipLaunchKernelGGL(row_grad_kernel<R>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream_), logits, symbols, ranges, boundary, norm,
+                       px_grad, py_grad, logits_grad, rows, S, T, Rr, C, term, rnnt_type);
   return check_launch("lattice_logprobs_bwd");
 }
 
