@@ -600,8 +600,9 @@ def get_rnnt_logprobs_smoothed(
     lm_probs = (lm - lm_max).exp()
     lmonly_normalizers = lm_probs.sum(dim=2, keepdim=True)  # [B][S+1][1]
     unigram_lm = torch.mean(lm_probs / lmonly_normalizers, dim=(0, 1), keepdim=True) + tiny
-    amonly_normalizers = (torch.mv(am_probs.reshape(-1, C), unigram_lm.reshape(C))
-                          .reshape(B, T, 1).log() + am_max).transpose(1, 2)  # [B][1][T]
+    # ([B*T, C] x [C] as a broadcast product and a row sum: rocBLAS' gemv is slow here)
+    amonly_normalizers = ((am_probs * unigram_lm).sum(dim=2, keepdim=True).log()
+                          + am_max).transpose(1, 2)  # [B][1][T]
     unigram_lm = unigram_lm.log()
     lmonly_normalizers = lmonly_normalizers.log() + lm_max
 
