@@ -1,0 +1,478 @@
+// The lm-only / am-only smoothing of get_rnnt_logprobs_smoothed
+// (fast_rnnt/python/fast_rnnt/rnnt_loss.py:1135-1369) and its backward.
+//
+// With pj / qj the joint px / py (from frnnt_simple_logprobs_fwd) and
+//   sigma[b,s,c] = softmax_c lm[b,s,:]            Ln[b,s]  = logsumexp_c lm[b,s,:]
+//   U[c]         = mean_{b,s} sigma[b,s,c] + tiny                      ("unigram lm")
+//   An[b,t]      = log sum_c exp(am[b,t,c]) U[c]
+// the reference forms, left to right,
+//   px = pj * k + (lm[b,s,sym] - Ln[b,s]) * l + ((am[b,t,sym] + log U[sym]) - An[b,t]) * a
+//   py = qj * k + (lm[b,s,term] - Ln[b,s]) * l + ((am[b,t,term] + log U[term]) - An[b,t]) * a
+// (k = 1 - l - a; for the regular lattice the am-only part of column T is -inf).
+//
+// Everything here is row-wise streaming work (one wave per lm or am row) plus two
+// reductions over the whole batch -- U over the lm rows, and in the backward pass the
+// gradient of U over the am rows -- which run in two deterministic stages (per-block
+// partial sums, then a sum over blocks).  The gradients follow from the formulas above:
+//   d/d lm[b,s,c] = l ([c=sym] rx + [c=term] ry) - l (rx + ry) sigma
+//                   + sigma (gU[c] - sum_c' sigma[c'] gU[c']) / N
+//   d/d am[b,t,c] = a (sum_s [c=sym_s] gx[b,s,t] + [c=term] cy[b,t]) - a G[b,t] q[b,t,c]
+//   gU[c] = a (sum_{(b,s): sym=c} rx[b,s] + [c=term] sum_{b,s} ry[b,s]) / U[c]
+//           - a sum_{b,t} G[b,t] exp(am[b,t,c] - max) / Z[b,t]
+// with rx / ry the row sums of the incoming px / py gradients, cy / G the column sums of
+// gy / gx + gy, q = exp(am - max) U / Z the am-only posterior and Z = exp(An - max).
+#include "common.hip.h"
+
+namespace frnnt {
+namespace {
+
+constexpr int kRowsPerBlock = 16;  // rows summed by one block of the batch reductions
+
+template <typename R>
+__device__ __forceinline__ R wave_max_nan(R v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const R o = __shfl_xor(v, off, 64);
+    v = (o > v || o != o) ? o : v;
+  }
+  return v;
+}
+template <typename R>
+__device__ __forceinline__ R wave_total(R v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+template <typename R>
+__device__ __forceinline__ R tiny_value();
+template <>
+__device__ __forceinline__ float tiny_value<float>() {
+  return 1.17549435e-38f;
+}
+template <>
+__device__ __forceinline__ double tiny_value<double>() {
+  return 2.2250738585072014e-308;
+}
+
+// ---- forward ------------------------------------------------------------------------
+
+// one wave per lm row: maximum and sum of exp(x - max)
+template <typename R>
+__global__ void __launch_bounds__(256)
+    lm_row_stats_kernel(const R *__restrict__ lm, R *__restrict__ row_max, R *__restrict__ row_sum,
+                        long rows, int C) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const R *x = lm + row * C;
+  R m = Num<R>::neg_inf();
+  for (int c = lane; c < C; c += kWave) {
+    const R v = x[c];
+    m = (v > m || v != v) ? v : m;
+  }
+  m = wave_max_nan(m);
+  R sum = 0;
+  for (int c = lane; c < C; c += kWave) sum += Num<R>::exp_(x[c] - m);
+  sum = wave_total(sum);
+  if (lane == 0) {
+    row_max[row] = m;
+    row_sum[row] = sum;
+  }
+}
+
+// partial[block][c] = sum over the block's rows of weight[row] * exp(x[row][c] - max[row]) * scale[row]
+// (scale = 1 / row_sum for the unigram, weight absent; for the backward reduction over am
+// rows weight[row] / z[row]).  Threads walk c, rows are visited in order.
+template <typename R>
+__global__ void __launch_bounds__(256)
+    weighted_column_partial_kernel(const R *__restrict__ x, const R *__restrict__ row_max,
+                                   const R *__restrict__ numer, const R *__restrict__ denom,
+                                   R *__restrict__ partial, long rows, int C) {
+  const long row0 = (long)blockIdx.x * kRowsPerBlock;
+  for (int c = threadIdx.x; c < C; c += 256) {
+    R acc = 0;
+    for (int k = 0; k < kRowsPerBlock; ++k) {
+      const long row = row0 + k;
+      if (row >= rows) break;
+      const R w = (numer ? numer[row] : (R)1) / denom[row];
+      acc += Num<R>::exp_(x[row * C + c] - row_max[row]) * w;
+    }
+    partial[(long)blockIdx.x * C + c] = acc;
+  }
+}
+
+// unigram[c] = (sum of the partials) / N + tiny
+template <typename R>
+__global__ void __launch_bounds__(256)
+    unigram_final_kernel(const R *__restrict__ partial, R *__restrict__ unigram, int blocks, long N,
+                         int C) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  R acc = 0;
+  for (int k = 0; k < blocks; ++k) acc += partial[(long)k * C + c];
+  unigram[c] = acc / (R)N + tiny_value<R>();
+}
+
+// one wave per am row: maximum and z = sum_c exp(x - max) unigram[c]
+template <typename R>
+__global__ void __launch_bounds__(256)
+    am_row_stats_kernel(const R *__restrict__ am, const R *__restrict__ unigram,
+                        R *__restrict__ row_max, R *__restrict__ row_z, long rows, int C) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const R *x = am + row * C;
+  R m = Num<R>::neg_inf();
+  for (int c = lane; c < C; c += kWave) {
+    const R v = x[c];
+    m = (v > m || v != v) ? v : m;
+  }
+  m = wave_max_nan(m);
+  R z = 0;
+  for (int c = lane; c < C; c += kWave) z += Num<R>::exp_(x[c] - m) * unigram[c];
+  z = wave_total(z);
+  if (lane == 0) {
+    row_max[row] = m;
+    row_z[row] = z;
+  }
+}
+
+// one thread per px / py element, t fastest
+template <typename R>
+__global__ void __launch_bounds__(256)
+    smoothed_combine_kernel(const R *__restrict__ lm, const R *__restrict__ am,
+                            const int64_t *__restrict__ symbols, const R *__restrict__ pxj,
+                            const R *__restrict__ pyj, const R *__restrict__ lm_max,
+                            const R *__restrict__ lm_sum, const R *__restrict__ am_max,
+                            const R *__restrict__ am_z, const R *__restrict__ unigram,
+                            R *__restrict__ px, R *__restrict__ py, int B, int S, int T, int C,
+                            int term, int regular, R k_joint, R k_lm, R k_am) {
+  const int T1 = regular ? T + 1 : T;
+  const int S1 = S + 1;
+  const long n_px = (long)B * S * T1, n_py = (long)B * S1 * T;
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx < n_px) {
+    const int t = (int)(idx % T1);
+    const long bs = idx / T1;
+    const int s = (int)(bs % S), b = (int)(bs / S);
+    const long lrow = (long)b * S1 + s;
+    const int64_t sym = symbols[(long)b * S + s];
+    const bool in = sym >= 0 && sym < C;
+    const R nan = std::numeric_limits<R>::quiet_NaN();
+    const R ln = log(lm_sum[lrow]) + lm_max[lrow];
+    const R lm_only = (in ? lm[lrow * C + sym] : nan) - ln;
+    R am_only = Num<R>::neg_inf();
+    if (t < T) {
+      const long arow = (long)b * T + t;
+      const R an = log(am_z[arow]) + am_max[arow];
+      am_only = ((in ? am[arow * C + sym] : nan) + (in ? log(unigram[sym]) : nan)) - an;
+    }
+    px[idx] = pxj[idx] * k_joint + lm_only * k_lm + am_only * k_am;
+  } else if (idx < n_px + n_py) {
+    const long j = idx - n_px;
+    const int t = (int)(j % T);
+    const long lrow = j / T;
+    const int b = (int)(lrow / S1);
+    const long arow = (long)b * T + t;
+    const R ln = log(lm_sum[lrow]) + lm_max[lrow];
+    const R an = log(am_z[arow]) + am_max[arow];
+    const R lm_only = lm[lrow * C + term] - ln;
+    const R am_only = (am[arow * C + term] + log(unigram[term])) - an;
+    py[j] = pyj[j] * k_joint + lm_only * k_lm + am_only * k_am;
+  }
+}
+
+// ---- backward -----------------------------------------------------------------------
+
+// Row sums rx, ry (one wave per lattice row; rx over all T1 columns) and column sums
+// cy = sum_s gy, G = sum_s (gx + gy) over the frames (64 frames per block, waves split
+// the rows); also the gradients of the joint inputs, k * (gx, gy).
+template <typename R>
+__global__ void __launch_bounds__(256)
+    smoothed_bwd_sums_kernel(const R *__restrict__ gpx, const R *__restrict__ gpy,
+                             R *__restrict__ gxj, R *__restrict__ gyj, R *__restrict__ row_x,
+                             R *__restrict__ row_y, R *__restrict__ col_y, R *__restrict__ col_g,
+                             int B, int S, int T, int T1, R k_joint) {
+  __shared__ R part[2][4][kWave];
+  const int S1 = S + 1;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long n_rows = (long)B * S1;
+  const long row_blocks = (n_rows + 3) / 4;
+  if (blockIdx.x < row_blocks) {
+    const long row = (long)blockIdx.x * 4 + wave;
+    if (row >= n_rows) return;
+    const int b = (int)(row / S1), s = (int)(row % S1);
+    R sx = 0, sy = 0;
+    if (s < S) {
+      const long o = ((long)b * S + s) * T1;
+      for (int t = lane; t < T1; t += kWave) {
+        const R v = gpx[o + t];
+        gxj[o + t] = v * k_joint;
+        sx += v;
+      }
+    }
+    const long o = row * T;
+    for (int t = lane; t < T; t += kWave) {
+      const R v = gpy[o + t];
+      gyj[o + t] = v * k_joint;
+      sy += v;
+    }
+    sx = wave_total(sx);
+    sy = wave_total(sy);
+    if (lane == 0) {
+      row_x[row] = sx;
+      row_y[row] = sy;
+    }
+  } else {
+    const int tiles = (T + kWave - 1) / kWave;
+    const long cb = blockIdx.x - row_blocks;
+    const int b = (int)(cb / tiles), t = (int)(cb % tiles) * kWave + lane;
+    const bool ok = t < T;
+    R ax = 0, ay = 0;
+    for (int s = wave; s < S1; s += 4) {
+      if (ok) {
+        ay += gpy[((long)b * S1 + s) * T + t];
+        if (s < S) ax += gpx[((long)b * S + s) * T1 + t];
+      }
+    }
+    part[0][wave][lane] = ax;
+    part[1][wave][lane] = ay;
+    __syncthreads();
+    if (wave == 0 && ok) {
+      const R x = (part[0][0][lane] + part[0][1][lane]) + (part[0][2][lane] + part[0][3][lane]);
+      const R y = (part[1][0][lane] + part[1][1][lane]) + (part[1][2][lane] + part[1][3][lane]);
+      col_y[(long)b * T + t] = y;
+      col_g[(long)b * T + t] = x + y;
+    }
+  }
+}
+
+// gU[c] = a (sum_{(b,s): sym=c} rx + [c=term] sum ry) / U[c] - a sum of the partials,
+// the partials being sum_rows G[row] exp(am - max) / z[row]
+template <typename R>
+__global__ void __launch_bounds__(256)
+    unigram_grad_kernel(const R *__restrict__ partial, const int64_t *__restrict__ symbols,
+                        const R *__restrict__ row_x, const R *__restrict__ row_y,
+                        const R *__restrict__ unigram, R *__restrict__ g_unigram, int blocks,
+                        int B, int S, int C, int term, R k_am) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  R acc = 0;
+  for (int k = 0; k < blocks; ++k) acc += partial[(long)k * C + c];
+  R direct = 0;
+  const int S1 = S + 1;
+  for (int b = 0; b < B; ++b)
+    for (int s = 0; s < S1; ++s) {
+      if (s < S && symbols[(long)b * S + s] == c) direct += row_x[(long)b * S1 + s];
+      if (c == term) direct += row_y[(long)b * S1 + s];
+    }
+  g_unigram[c] = k_am * direct / unigram[c] - k_am * acc;
+}
+
+// one wave per lm row
+template <typename R>
+__global__ void __launch_bounds__(256)
+    smoothed_bwd_lm_kernel(const R *__restrict__ lm, const int64_t *__restrict__ symbols,
+                           const R *__restrict__ lm_max, const R *__restrict__ lm_sum,
+                           const R *__restrict__ row_x, const R *__restrict__ row_y,
+                           const R *__restrict__ g_unigram, R *__restrict__ lm_grad, long rows,
+                           int S, int C, int term, R k_lm, R inv_n) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const int S1 = S + 1;
+  const int b = (int)(row / S1), s = (int)(row % S1);
+  const R *x = lm + row * C;
+  const R m = lm_max[row], inv = (R)1 / lm_sum[row];
+  R dot = 0;
+  for (int c = lane; c < C; c += kWave) dot += Num<R>::exp_(x[c] - m) * inv * g_unigram[c];
+  dot = wave_total(dot);
+  const R rx = row_x[row], ry = row_y[row];
+  const int64_t sym = s < S ? symbols[(long)b * S + s] : -1;
+  R *g = lm_grad + row * C;
+  for (int c = lane; c < C; c += kWave) {
+    const R sigma = Num<R>::exp_(x[c] - m) * inv;
+    R v = sigma * ((g_unigram[c] - dot) * inv_n - k_lm * (rx + ry));
+    if (c == sym) v += k_lm * rx;
+    if (c == term) v += k_lm * ry;
+    g[c] = v;
+  }
+}
+
+// one wave per am row: everything but the per-symbol terms
+template <typename R>
+__global__ void __launch_bounds__(256)
+    smoothed_bwd_am_kernel(const R *__restrict__ am, const R *__restrict__ am_max,
+                           const R *__restrict__ am_z, const R *__restrict__ unigram,
+                           const R *__restrict__ col_y, const R *__restrict__ col_g,
+                           R *__restrict__ am_grad, long rows, int C, int term, R k_am) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const R *x = am + row * C;
+  const R m = am_max[row];
+  const R w = -k_am * col_g[row] / am_z[row];
+  const R cy = k_am * col_y[row];
+  R *g = am_grad + row * C;
+  for (int c = lane; c < C; c += kWave) {
+    R v = w * Num<R>::exp_(x[c] - m) * unigram[c];
+    if (c == term) v += cy;
+    g[c] = v;
+  }
+}
+
+// am_grad[b,t,sym] += a * sum over the rows s' >= s with the same symbol of gx[b,s',t]:
+// one block per (b, s); only the first row of each symbol works, so a column of
+// am_grad[b] has one owner and the rows are added in order.
+template <typename R>
+__global__ void __launch_bounds__(256)
+    smoothed_bwd_symbols_kernel(const R *__restrict__ gpx, const int64_t *__restrict__ symbols,
+                                R *__restrict__ am_grad, int S, int T, int T1, int C, R k_am) {
+  const int b = blockIdx.x / S, s = blockIdx.x % S;
+  const int64_t *sym_b = symbols + (long)b * S;
+  const int64_t sym = sym_b[s];
+  if (sym < 0 || sym >= C) return;
+  for (int k = 0; k < s; ++k)
+    if (sym_b[k] == sym) return;  // an earlier row owns this symbol
+  for (int t = threadIdx.x; t < T; t += 256) {
+    R acc = 0;
+    for (int k = s; k < S; ++k)
+      if (sym_b[k] == sym) acc += gpx[((long)b * S + k) * T1 + t];
+    am_grad[((long)b * T + t) * C + sym] += k_am * acc;
+  }
+}
+
+template <typename R>
+int fwd_impl(const R *lm, const R *am, const int64_t *symbols, const R *pxj, const R *pyj, R *px,
+             R *py, R *lm_max, R *lm_sum, R *am_max, R *am_z, R *unigram, R *partial, int B, int S,
+             int T, int C, int term, int regular, double lm_only_scale, double am_only_scale,
+             void *stream_) {
+  if (B < 0 || S < 0 || T < 0 || C < 1) return fail(FRNNT_EINVAL, "smoothed_logprobs_fwd: bad size");
+  if (term < 0 || term >= C)
+    return fail(FRNNT_EINVAL, "smoothed_logprobs_fwd: termination symbol outside [0, C)");
+  if (B == 0) return FRNNT_OK;
+  if (!lm || !am || (!symbols && S > 0) || !pxj || !pyj || !px || !py || !lm_max || !lm_sum ||
+      !am_max || !am_z || !unigram || !partial)
+    return fail(FRNNT_EINVAL, "smoothed_logprobs_fwd: null pointer");
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  const long n_lm = (long)B * (S + 1), n_am = (long)B * T;
+  const int blocks = (int)((n_lm + kRowsPerBlock - 1) / kRowsPerBlock);
+  hipLaunchKernelGGL(lm_row_stats_kernel<R>, dim3((unsigned)((n_lm + 3) / 4)), dim3(256), 0, stream,
+                     lm, lm_max, lm_sum, n_lm, C);
+  hipLaunchKernelGGL(weighted_column_partial_kernel<R>, dim3(blocks), dim3(256), 0, stream, lm,
+                     lm_max, (const R *)nullptr, lm_sum, partial, n_lm, C);
+  hipLaunchKernelGGL(unigram_final_kernel<R>, dim3((C + 255) / 256), dim3(256), 0, stream, partial,
+                     unigram, blocks, n_lm, C);
+  if (n_am > 0)
+    hipLaunchKernelGGL(am_row_stats_kernel<R>, dim3((unsigned)((n_am + 3) / 4)), dim3(256), 0,
+                       stream, am, unigram, am_max, am_z, n_am, C);
+  const int T1 = regular ? T + 1 : T;
+  const long total = (long)B * S * T1 + (long)B * (S + 1) * T;
+  const R k_lm = (R)lm_only_scale, k_am = (R)am_only_scale;
+  const R k_joint = (R)(1.0 - lm_only_scale - am_only_scale);
+  if (total > 0)
+    hipLaunchKernelGGL(smoothed_combine_kernel<R>, dim3((unsigned)((total + 255) / 256)),
+                       dim3(256), 0, stream, lm, am, symbols, pxj, pyj, lm_max, lm_sum, am_max,
+                       am_z, unigram, px, py, B, S, T, C, term, regular, k_joint, k_lm, k_am);
+  return check_launch("smoothed_logprobs_fwd");
+}
+
+template <typename R>
+int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const R *lm_max, const R *lm_sum,
+             const R *am_max, const R *am_z, const R *unigram, const R *px_grad, const R *py_grad,
+             R *pxj_grad, R *pyj_grad, R *lm_grad, R *am_grad, R *row_x, R *row_y, R *col_y,
+             R *col_g, R *g_unigram, R *partial, int B, int S, int T, int C, int term, int regular,
+             double lm_only_scale, double am_only_scale, void *stream_) {
+  if (B < 0 || S < 0 || T < 0 || C < 1) return fail(FRNNT_EINVAL, "smoothed_logprobs_bwd: bad size");
+  if (term < 0 || term >= C)
+    return fail(FRNNT_EINVAL, "smoothed_logprobs_bwd: termination symbol outside [0, C)");
+  if (B == 0) return FRNNT_OK;
+  if (!lm || !am || (!symbols && S > 0) || !lm_max || !lm_sum || !am_max || !am_z || !unigram ||
+      !px_grad || !py_grad || !pxj_grad || !pyj_grad || !lm_grad || !am_grad || !row_x ||
+      !row_y || !col_y || !col_g || !g_unigram || !partial)
+    return fail(FRNNT_EINVAL, "smoothed_logprobs_bwd: null pointer");
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  const int T1 = regular ? T + 1 : T;
+  const long n_lm = (long)B * (S + 1), n_am = (long)B * T;
+  const R k_lm = (R)lm_only_scale, k_am = (R)am_only_scale;
+  const R k_joint = (R)(1.0 - lm_only_scale - am_only_scale);
+  const long sums_blocks = (n_lm + 3) / 4 + (long)B * ((T + kWave - 1) / kWave);
+  hipLaunchKernelGGL(smoothed_bwd_sums_kernel<R>, dim3((unsigned)sums_blocks), dim3(256), 0, stream,
+                     px_grad, py_grad, pxj_grad, pyj_grad, row_x, row_y, col_y, col_g, B, S, T, T1,
+                     k_joint);
+  const int blocks = (int)((n_am + kRowsPerBlock - 1) / kRowsPerBlock);
+  if (n_am > 0)
+    hipLaunchKernelGGL(weighted_column_partial_kernel<R>, dim3(blocks), dim3(256), 0, stream, am,
+                       am_max, col_g, am_z, partial, n_am, C);
+  hipLaunchKernelGGL(unigram_grad_kernel<R>, dim3((C + 255) / 256), dim3(256), 0, stream, partial,
+                     symbols, row_x, row_y, unigram, g_unigram, n_am > 0 ? blocks : 0, B, S, C, term,
+                     k_am);
+  hipLaunchKernelGGL(smoothed_bwd_lm_kernel<R>, dim3((unsigned)((n_lm + 3) / 4)), dim3(256), 0,
+                     stream, lm, symbols, lm_max, lm_sum, row_x, row_y, g_unigram, lm_grad, n_lm, S, C,
+                     term, k_lm, (R)(1.0 / (double)n_lm));
+  if (n_am > 0) {
+    hipLaunchKernelGGL(smoothed_bwd_am_kernel<R>, dim3((unsigned)((n_am + 3) / 4)), dim3(256), 0,
+                       stream, am, am_max, am_z, unigram, col_y, col_g, am_grad, n_am, C, term, k_am);
+    if (S > 0)
+      hipLaunchKernelGGL(smoothed_bwd_symbols_kernel<R>, dim3((unsigned)(B * S)), dim3(256), 0,
+                         stream, px_grad, symbols, am_grad, S, T, T1, C, k_am);
+  }
+  return check_launch("smoothed_logprobs_bwd");
+}
+
+}  // namespace
+}  // namespace frnnt
+
+extern "C" {
+
+int frnnt_smoothed_logprobs_fwd_f32(const float *lm, const float *am, const int64_t *symbols,
+                                    const float *px_joint, const float *py_joint, float *px,
+                                    float *py, float *lm_max, float *lm_sum, float *am_max,
+                                    float *am_z, float *unigram, float *partial, int B, int S,
+                                    int T, int C, int termination_symbol, int regular,
+                                    double lm_only_scale, double am_only_scale, void *stream) {
+  return frnnt::fwd_impl<float>(lm, am, symbols, px_joint, py_joint, px, py, lm_max, lm_sum, am_max,
+                                am_z, unigram, partial, B, S, T, C, termination_symbol, regular,
+                                lm_only_scale, am_only_scale, stream);
+}
+int frnnt_smoothed_logprobs_fwd_f64(const double *lm, const double *am, const int64_t *symbols,
+                                    const double *px_joint, const double *py_joint, double *px,
+                                    double *py, double *lm_max, double *lm_sum, double *am_max,
+                                    double *am_z, double *unigram, double *partial, int B, int S,
+                                    int T, int C, int termination_symbol, int regular,
+                                    double lm_only_scale, double am_only_scale, void *stream) {
+  return frnnt::fwd_impl<double>(lm, am, symbols, px_joint, py_joint, px, py, lm_max, lm_sum,
+                                 am_max, am_z, unigram, partial, B, S, T, C, termination_symbol,
+                                 regular, lm_only_scale, am_only_scale, stream);
+}
+int frnnt_smoothed_logprobs_bwd_f32(const float *lm, const float *am, const int64_t *symbols,
+                                    const float *lm_max, const float *lm_sum, const float *am_max,
+                                    const float *am_z, const float *unigram, const float *px_grad,
+                                    const float *py_grad, float *px_joint_grad,
+                                    float *py_joint_grad, float *lm_grad, float *am_grad,
+                                    float *row_x, float *row_y, float *col_y, float *col_g,
+                                    float *g_unigram, float *partial, int B, int S, int T, int C,
+                                    int termination_symbol, int regular, double lm_only_scale,
+                                    double am_only_scale, void *stream) {
+  return frnnt::bwd_impl<float>(lm, am, symbols, lm_max, lm_sum, am_max, am_z, unigram, px_grad,
+                                py_grad, px_joint_grad, py_joint_grad, lm_grad, am_grad, row_x,
+                                row_y, col_y, col_g, g_unigram, partial, B, S, T, C,
+                                termination_symbol, regular, lm_only_scale, am_only_scale, stream);
+}
+int frnnt_smoothed_logprobs_bwd_f64(const double *lm, const double *am, const int64_t *symbols,
+                                    const double *lm_max, const double *lm_sum,
+                                    const double *am_max, const double *am_z,
+                                    const double *unigram, const double *px_grad,
+                                    const double *py_grad, double *px_joint_grad,
+                                    double *py_joint_grad, double *lm_grad, double *am_grad,
+                                    double *row_x, double *row_y, double *col_y, double *col_g,
+                                    double *g_unigram, double *partial, int B, int S, int T, int C,
+                                    int termination_symbol, int regular, double lm_only_scale,
+                                    double am_only_scale, void *stream) {
+  return frnnt::bwd_impl<double>(lm, am, symbols, lm_max, lm_sum, am_max, am_z, unigram, px_grad,
+                                 py_grad, px_joint_grad, py_joint_grad, lm_grad, am_grad, row_x,
+                                 row_y, col_y, col_g, g_unigram, partial, B, S, T, C,
+                                 termination_symbol, regular, lm_only_scale, am_only_scale, stream);
+}
+
+}  // extern "C"

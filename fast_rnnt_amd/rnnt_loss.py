@@ -563,6 +563,65 @@ def rnnt_loss_pruned(
                                  return_grad)
 
 
+class _SmoothedCombine(torch.autograd.Function):
+    """Interpolation of the joint (px, py) with the lm-only and am-only models
+    (rnnt_loss.py:1264-1355): frnnt_smoothed_logprobs_fwd/bwd."""
+
+    @staticmethod
+    def forward(ctx, pxj, pyj, lm, am, symbols, termination_symbol, regular, k_lm, k_am):
+        B, T, C = am.shape
+        S = lm.shape[1] - 1
+        sfx = _lib.suffix(am.dtype)
+        lm_c, am_c, sym_c = lm.contiguous(), am.contiguous(), symbols.contiguous()
+        pxj_c, pyj_c = pxj.contiguous(), pyj.contiguous()
+        opts = dict(dtype=am.dtype, device=am.device)
+        n_lm, n_am = B * (S + 1), B * T
+        # kept for the backward: lm_max | lm_sum | am_max | am_z | unigram
+        (o_lmx, o_lms, o_amx, o_amz, o_u), total = _carve([n_lm, n_lm, n_am, n_am, C])
+        with _on_device(am.device):
+            px = torch.empty_like(pxj_c)
+            py = torch.empty_like(pyj_c)
+            stats = torch.empty(total, **opts)
+            partial = torch.empty((n_lm + 15) // 16 * C, **opts)
+            base, item = stats.data_ptr(), stats.element_size()
+            _lib.call("frnnt_smoothed_logprobs_fwd_" + sfx, lm_c.data_ptr(), am_c.data_ptr(),
+                      sym_c.data_ptr(), pxj_c.data_ptr(), pyj_c.data_ptr(), px.data_ptr(),
+                      py.data_ptr(), base + o_lmx * item, base + o_lms * item,
+                      base + o_amx * item, base + o_amz * item, base + o_u * item,
+                      partial.data_ptr(), B, S, T, C, int(termination_symbol), int(regular),
+                      k_lm, k_am, _lib.stream_of(am))
+        ctx.save_for_backward(lm_c, am_c, sym_c, stats)
+        ctx.meta = (B, S, T, C, int(termination_symbol), int(regular), k_lm, k_am, sfx,
+                    (o_lmx, o_lms, o_amx, o_amz, o_u))
+        return px, py
+
+    @staticmethod
+    def backward(ctx, gpx, gpy):
+        lm, am, sym, stats = ctx.saved_tensors
+        B, S, T, C, term, regular, k_lm, k_am, sfx, (o_lmx, o_lms, o_amx, o_amz, o_u) = ctx.meta
+        opts = dict(dtype=am.dtype, device=am.device)
+        T1 = T + 1 if regular else T
+        n_lm, n_am = B * (S + 1), B * T
+        with _on_device(am.device):
+            gpx = torch.zeros(B, S, T1, **opts) if gpx is None else gpx.contiguous()
+            gpy = torch.zeros(B, S + 1, T, **opts) if gpy is None else gpy.contiguous()
+            gxj, gyj = torch.empty_like(gpx), torch.empty_like(gpy)
+            lm_grad, am_grad = torch.empty_like(lm), torch.empty_like(am)
+            # scratch: row_x | row_y | col_y | col_g | g_unigram | partial
+            (o_rx, o_ry, o_cy, o_cg, o_gu, o_p), total = _carve(
+                [n_lm, n_lm, n_am, n_am, C, (n_am + 15) // 16 * C])
+            scratch = torch.empty(total, **opts)
+            sb, wb, item = scratch.data_ptr(), stats.data_ptr(), stats.element_size()
+            _lib.call("frnnt_smoothed_logprobs_bwd_" + sfx, lm.data_ptr(), am.data_ptr(),
+                      sym.data_ptr(), wb + o_lmx * item, wb + o_lms * item, wb + o_amx * item,
+                      wb + o_amz * item, wb + o_u * item, gpx.data_ptr(), gpy.data_ptr(),
+                      gxj.data_ptr(), gyj.data_ptr(), lm_grad.data_ptr(), am_grad.data_ptr(),
+                      sb + o_rx * item, sb + o_ry * item, sb + o_cy * item, sb + o_cg * item,
+                      sb + o_gu * item, sb + o_p * item, B, S, T, C, term, regular, k_lm, k_am,
+                      _lib.stream_of(am))
+        return gxj, gyj, lm_grad, am_grad, None, None, None, None, None
+
+
 def get_rnnt_logprobs_smoothed(
     lm: Tensor, am: Tensor, symbols: Tensor, termination_symbol: int,
     lm_only_scale: float = 0.1, am_only_scale: float = 0.1,
@@ -575,8 +634,8 @@ def get_rnnt_logprobs_smoothed(
                                                     + am_only_scale * am_only
 
     The joint part -- the [B,S+1,C] x [B,C,T] contraction and its px / py -- comes
-    from the fused MFMA kernel; the lm-only / am-only corrections are small
-    tensors handled with torch ops in the reference's order.
+    from the fused MFMA kernel; the lm-only / am-only models, the unigram over the
+    whole batch and the interpolation come from frnnt_smoothed_logprobs_fwd/bwd.
     """
     assert lm.ndim == 3, lm.ndim
     assert am.ndim == 3, am.ndim
@@ -593,42 +652,14 @@ def get_rnnt_logprobs_smoothed(
     base_type = "regular" if rnnt_type == "regular" else "modified"
     px, py = _SimpleLogprobs.apply(lm, am, symbols, None, termination_symbol, base_type)
 
-    tiny = torch.finfo(lm.dtype).tiny
-    am_max, _ = torch.max(am, dim=2, keepdim=True)
-    lm_max, _ = torch.max(lm, dim=2, keepdim=True)
-    am_probs = (am - am_max).exp()
-    lm_probs = (lm - lm_max).exp()
-    lmonly_normalizers = lm_probs.sum(dim=2, keepdim=True)  # [B][S+1][1]
-    unigram_lm = torch.mean(lm_probs / lmonly_normalizers, dim=(0, 1), keepdim=True) + tiny
-    # ([B*T, C] x [C] as a broadcast product and a row sum: rocBLAS' gemv is slow here)
-    amonly_normalizers = ((am_probs * unigram_lm).sum(dim=2, keepdim=True).log()
-                          + am_max).transpose(1, 2)  # [B][1][T]
-    unigram_lm = unigram_lm.log()
-    lmonly_normalizers = lmonly_normalizers.log() + lm_max
-
-    rows = torch.arange(B, device=am.device).reshape(B, 1)
-    px_am = am[rows, :, symbols]  # [B][S][T]
-    if rnnt_type == "regular":
-        px_am = torch.cat((px_am, px_am.new_full((B, S, 1), float("-inf"))), dim=2)
-    px_lm = torch.gather(lm[:, :S], dim=2, index=symbols.unsqueeze(-1))  # [B][S][1]
-    px_lm_unigram = unigram_lm.reshape(C)[symbols].unsqueeze(-1)  # [B][S][1]
-    px_amonly = px_am + px_lm_unigram
-    px_amonly[:, :, :T] -= amonly_normalizers
-    px_lmonly = px_lm - lmonly_normalizers[:, :S, :]
-
-    py_am = am[:, :, termination_symbol].unsqueeze(1)
-    py_lm = lm[:, :, termination_symbol].unsqueeze(2)
-    py_amonly = py_am + unigram_lm[0][0][termination_symbol] - amonly_normalizers
-    py_lmonly = py_lm - lmonly_normalizers
-
-    combined_scale = 1.0 - lm_only_scale - am_only_scale
     # exact zeros would turn -inf * 0 into nan
     if lm_only_scale == 0.0:
         lm_only_scale = 1.0e-20
     if am_only_scale == 0.0:
         am_only_scale = 1.0e-20
-    px_interp = px * combined_scale + px_lmonly * lm_only_scale + px_amonly * am_only_scale
-    py_interp = py * combined_scale + py_lmonly * lm_only_scale + py_amonly * am_only_scale
+    px_interp, py_interp = _SmoothedCombine.apply(
+        px, py, lm, am, symbols, termination_symbol, rnnt_type == "regular",
+        float(lm_only_scale), float(am_only_scale))
 
     if rnnt_type == "regular":
         px_interp = fix_for_boundary(px_interp, boundary)

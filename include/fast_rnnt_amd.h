@@ -142,6 +142,54 @@ int frnnt_simple_logprobs_bwd_f64(const double *lm, const double *am, const int6
                                   double *lm_grad, double *am_grad, int B, int S, int T, int C,
                                   int termination_symbol, int rnnt_type, void *stream);
 /*
+ * The lm-only / am-only smoothing of get_rnnt_logprobs_smoothed (rnnt_loss.py:1135-1369)
+ * applied to joint px / py (px_joint, py_joint: outputs of frnnt_simple_logprobs_fwd
+ * without a boundary, regular or modified layout):
+ *   px = px_joint * (1 - l - a) + lm_only_px * l + am_only_px * a     (same for py)
+ * with l = lm_only_scale, a = am_only_scale, the lm-only model log_softmax(lm) and the
+ * am-only model am + log(unigram) normalised per frame, unigram = mean over all
+ * (b, s) of softmax(lm[b,s,:]) + tiny.  The boundary / constrained post-processing of
+ * the reference (rnnt_loss.py:1357-1367) is left to the caller.
+ *   lm_max, lm_sum [B][S+1], am_max, am_z [B][T], unigram [C]: out, kept for the backward
+ *   partial [ceil(B*(S+1)/16)][C] (forward), [ceil(B*T/16)][C] (backward): scratch
+ * Backward: px_grad / py_grad are the gradients of px / py; out are the gradients of
+ * the joint inputs ((1 - l - a) * px_grad, ...) and the smoothing terms' own
+ * contributions to lm_grad [B][S+1][C] and am_grad [B][T][C] (fully written);
+ * row_x, row_y [B][S+1], col_y, col_g [B][T], g_unigram [C]: scratch.
+ */
+int frnnt_smoothed_logprobs_fwd_f32(const float *lm, const float *am, const int64_t *symbols,
+                                    const float *px_joint, const float *py_joint, float *px,
+                                    float *py, float *lm_max, float *lm_sum, float *am_max,
+                                    float *am_z, float *unigram, float *partial, int B, int S,
+                                    int T, int C, int termination_symbol, int regular,
+                                    double lm_only_scale, double am_only_scale, void *stream);
+int frnnt_smoothed_logprobs_fwd_f64(const double *lm, const double *am, const int64_t *symbols,
+                                    const double *px_joint, const double *py_joint, double *px,
+                                    double *py, double *lm_max, double *lm_sum, double *am_max,
+                                    double *am_z, double *unigram, double *partial, int B, int S,
+                                    int T, int C, int termination_symbol, int regular,
+                                    double lm_only_scale, double am_only_scale, void *stream);
+int frnnt_smoothed_logprobs_bwd_f32(const float *lm, const float *am, const int64_t *symbols,
+                                    const float *lm_max, const float *lm_sum, const float *am_max,
+                                    const float *am_z, const float *unigram, const float *px_grad,
+                                    const float *py_grad, float *px_joint_grad,
+                                    float *py_joint_grad, float *lm_grad, float *am_grad,
+                                    float *row_x, float *row_y, float *col_y, float *col_g,
+                                    float *g_unigram, float *partial, int B, int S, int T, int C,
+                                    int termination_symbol, int regular, double lm_only_scale,
+                                    double am_only_scale, void *stream);
+int frnnt_smoothed_logprobs_bwd_f64(const double *lm, const double *am, const int64_t *symbols,
+                                    const double *lm_max, const double *lm_sum,
+                                    const double *am_max, const double *am_z,
+                                    const double *unigram, const double *px_grad,
+                                    const double *py_grad, double *px_joint_grad,
+                                    double *py_joint_grad, double *lm_grad, double *am_grad,
+                                    double *row_x, double *row_y, double *col_y, double *col_g,
+                                    double *g_unigram, double *partial, int B, int S, int T, int C,
+                                    int termination_symbol, int regular, double lm_only_scale,
+                                    double am_only_scale, void *stream);
+
+/*
  * Forward pipeline of rnnt_loss_simple (rnnt_loss.py:230-340) in one call:
  * frnnt_simple_logprobs_fwd, frnnt_mi_forward, then -- when px_grad / py_grad are
  * given -- frnnt_mi_backward with a gradient of ones (what the recursion's autograd
