@@ -301,7 +301,7 @@ def main():
             cpu_loss = cpu_step()
             n += 1
             spent = time.perf_counter() - t_start
-            if spent > args.cpu_seconds or n >= 200:
+            if spent > args.cpu_seconds or n >= 5000:
                 break
         gpu_loss = step().item()
         cpu = {

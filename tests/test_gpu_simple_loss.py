@@ -119,7 +119,7 @@ def test_delay_penalty_and_only_one_input_needs_grad(gpu_device):
         fast_rnnt_amd.rnnt_loss_simple(dl, am.to(dev), sym.to(dev), 0, reduction="bogus")
 
 
-@pytest.mark.parametrize("name", ["c1", "c2"])
+@pytest.mark.parametrize("name", ["c1", "c2", "c4"])
 def test_baseline_configs(gpu_device, name):
     dev = gpu_device
     w = workloads.make(name)
