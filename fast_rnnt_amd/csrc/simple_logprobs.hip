@@ -386,6 +386,13 @@ __device__ __forceinline__ dgemm::floatx4 load4_guarded(const float *base, int o
 
 // ---- fp32: MFMA kernels with LDS slabs / panels (xcd_grid.hip.h) --------------------
 
+// exp(x - m) as one fused multiply-add and one v_exp_f32: 2^(x log2(e) - m log2(e)),
+// with shift2 = -m log2(e) prepared per row; x = -inf gives 0.
+constexpr float kLog2e = 1.44269504088896341f;
+__device__ __forceinline__ float exp_shifted(float x, float shift2) {
+  return __builtin_amdgcn_exp2f(__builtin_fmaf(x, kLog2e, shift2));
+}
+
 // Normalizer GEMM, wave-private LDS transposition.  Both operands are k-contiguous
 // ([rows][C]), the matrix cores want one row per lane.  Letting every lane fetch its
 // own row costs one cache-line lookup per lane and instruction, which is what bounds
@@ -396,20 +403,30 @@ __device__ __forceinline__ dgemm::floatx4 load4_guarded(const float *base, int o
 // never wait for each other in the loop (a wave's LDS writes and reads are served in
 // program order), only once at the end, when the partial sums meet.  Two waves share
 // a SIMD, so one wave's exp / LDS-write phase runs under the other's MFMA phase.
-// A workgroup covers 96 lattice rows (three 32-row tiles) x 32 frames, so at
-// S+1 <= 96 the lm operand is fetched once per 32 frames.
-constexpr int kPanS = 96;                 // lattice rows per workgroup
+// A workgroup covers kS lattice rows (32-row tiles) x 32 frames and takes k in slabs
+// of kK: 96 rows with k = 32, or 128 rows with k = 16 (the LDS holds eight slabs either
+// way).  The host picks the form that pads S+1 least, so that at S+1 <= 128 the lm
+// operand is fetched once per 32 frames and the am operand once.
 constexpr int kPanT = 32;                 // frames per workgroup
-constexpr int kPanRows = kPanS + kPanT;   // rows of a slab: lm rows, then am rows
-constexpr int kPanK = 32;                 // k per slab
-constexpr int kPanPitch = kPanK + 1;
-constexpr int kPanSlab = kPanRows * kPanPitch;  // floats per slab
+constexpr int kPanOutPitch = kPanT + 1;   // pitch of a wave's partial sums in LDS
 constexpr int kPanWaves = 8;
 constexpr int kPanThreads = kPanWaves * kWave;
-constexpr size_t kPanLdsBytes = (size_t)kPanWaves * kPanSlab * sizeof(float);
-constexpr int kPanItems = (kPanS * kPanT / 4 + kPanThreads - 1) / kPanThreads;  // 16-byte outputs per thread
+template <int kS, int kK>
+struct PanelShape {
+  static constexpr int kRows = kS + kPanT;        // rows of a slab: lm rows, then am rows
+  static constexpr int kPitch = kK + 1;
+  static constexpr int kSlab = kRows * kPitch;    // floats per slab
+  static constexpr int kRowLanes = kK / 4;        // lanes that share a row of a slab
+  static constexpr int kRowsPerLoad = kWave / kRowLanes;
+  static constexpr int kLoads = kRows / kRowsPerLoad;  // 16-byte loads per lane and slab
+  static constexpr int kSums = kS * kPanOutPitch; // floats of a wave's partial sums
+  static constexpr size_t kLdsBytes =
+      (size_t)kPanWaves * (kSlab > kSums ? kSlab : kSums) * sizeof(float);
+  static constexpr int kItems = (kS * kPanT / 4 + kPanThreads - 1) / kPanThreads;  // 16-byte outputs per thread
+  static_assert(kRows % kRowsPerLoad == 0 && kLoads % 2 == 0 && kS % 32 == 0 && kS <= 128, "shape");
+};
 
-template <bool kVec>
+template <bool kVec, int kS, int kK>
 __global__ void __launch_bounds__(kPanThreads)
     simple_fwd_panel_kernel(const float *__restrict__ lm, const float *__restrict__ am,
                             const int64_t *__restrict__ symbols,
@@ -418,9 +435,15 @@ __global__ void __launch_bounds__(kPanThreads)
                             float *__restrict__ px, float *__restrict__ py,
                             float *__restrict__ norm_raw, int B, int S, int T, int C, int term,
                             int rnnt_type) {
+  using Shape = PanelShape<kS, kK>;
+  constexpr int kPanS = kS, kPanK = kK, kPanRows = Shape::kRows, kPanPitch = Shape::kPitch;
+  constexpr int kPanSlab = Shape::kSlab, kPanItems = Shape::kItems;
+  constexpr int kRowLanes = Shape::kRowLanes, kRowsPerLoad = Shape::kRowsPerLoad;
   using namespace dgemm;
   extern __shared__ float pan_lds[];
-  __shared__ float wave_max[kPanWaves][kPanRows];  // row maxima over each wave's share of k
+  __shared__ float wave_max[kPanWaves][kPanRows];    // row maxima over each wave's share of k
+  __shared__ float wave_shift[kPanWaves][kPanRows];  // the waves' final shifts, as -shift log2(e)
+  __shared__ float factor[kPanWaves][kPanRows];      // scale factors for a wave's partial sums
   __shared__ float slab_max[kPanRows];             // row maxima
   __shared__ float row_term[kPanS], row_sym[kPanS], row_max[kPanS];  // lm[s,term], lm[s,sym[s]], lm_max[s]
   __shared__ int row_symbol[kPanS];
@@ -451,113 +474,58 @@ __global__ void __launch_bounds__(kPanThreads)
       out_sym[j] = (y >= 0 && y < C) ? (int)y : -1;
     }
   }
-  int my_sym = -1;  // threads 0 .. 95 own a lattice row each
+  int my_sym = -1;  // threads 0 .. kS-1 own a lattice row each
   if (tid < kPanS && s_tile + tid < S) {
     const int64_t y = symb[s_tile + tid];
     my_sym = (y >= 0 && y < C) ? (int)y : -1;
   }
 
-  // ---- what this lane fetches of every slab: rows sub + 8 j, k-offset 4 (lane % 8)
-  constexpr int kLoads = kPanRows / 8;
-  const int sub = lane >> 3, kq = 4 * (lane & 7);
-  int row_off[kLoads];    // element offset of (row, k = kq) in lm[b] / am[b], -1: no such row
-#pragma unroll
-  for (int j = 0; j < kLoads; ++j) {
-    const int row = sub + 8 * j;
-    if (row < kPanS) {
-      const int sr = s_tile + row;
-      row_off[j] = sr < S1 ? sr * C + kq : -1;
-    } else {
-      const int tr = t_tile + row - kPanS;
-      row_off[j] = tr < T ? tr * C + kq : -1;
-    }
-  }
-  // what lies outside the operands reads as -inf: neutral for the maximum, and
-  // exp(-inf - max) = 0 in the product
+  // ---- what this lane fetches of every slab: rows sub + kRowsPerLoad j, k-offset kq
+  constexpr int kLoads = Shape::kLoads;
+  const int sub = lane / kRowLanes, kq = 4 * (lane % kRowLanes);
+  // row j of a fetch is lattice row s_tile + sub + kRowsPerLoad j while that stays below
+  // kS, a frame after that; what lies outside the operands reads as -inf, neutral for
+  // the maximum, and exp(-inf - shift) = 0 in the product
+  constexpr int kLmLoads = kPanS / kRowsPerLoad;
+  static_assert(kPanS % kRowsPerLoad == 0, "a fetch row holds lm or am, not both");
+  const int lm_off = (s_tile + sub) * C + kq, am_off = (t_tile + sub) * C + kq;
+  const int lm_rows = S1 - s_tile - sub, am_rows = T - t_tile - sub;  // rows left from this lane's first
+  const int step = kRowsPerLoad * C;
   auto fetch = [&](floatx4 (&into)[kLoads], int k0) {
+    const int width = min(4, max(C - k0 - kq, 0));
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
-      const float *src = (sub + 8 * j < kPanS) ? lmb : amb;
-      const int valid = row_off[j] >= 0 ? min(4, max(C - k0 - kq, 0)) : 0;
-      into[j] = load4_guarded<kVec>(src, row_off[j] + k0, valid, ninf);
+      if (j < kLmLoads)
+        into[j] = load4_guarded<kVec>(lmb, lm_off + j * step + k0,
+                                      kRowsPerLoad * j < lm_rows ? width : 0, ninf);
+      else
+        into[j] = load4_guarded<kVec>(amb, am_off + (j - kLmLoads) * step + k0,
+                                      kRowsPerLoad * (j - kLmLoads) < am_rows ? width : 0, ninf);
     }
   };
   const int chunks = (C + kPanK - 1) / kPanK;
+  // a wave takes the slabs in pairs (2 p, 2 p + 1), p = wave, wave + 8, ..: the two
+  // slabs of a pair are requested back to back and share their cache lines at k = 16
+  const int pairs = (chunks + 1) / 2;
 
-  // ---- first pass: the row maxima (rnnt_loss.py:174-178).  Every wave scans its own
-  // slabs (they come from L2 again in the second pass), then the waves' results meet.
-  floatx4 slab[kLoads];
-  {
-    float m[kLoads];
-#pragma unroll
-    for (int j = 0; j < kLoads; ++j) m[j] = ninf;
-    // half a slab is consumed while the next half is in flight
-    constexpr int kHalf = kLoads / 2;
-    auto fetch_half = [&](floatx4 (&into)[kHalf], int first, int k0) {
-#pragma unroll
-      for (int j = 0; j < kHalf; ++j) {
-        const float *src = (sub + 8 * (first + j) < kPanS) ? lmb : amb;
-        const int valid = row_off[first + j] >= 0 ? min(4, max(C - k0 - kq, 0)) : 0;
-        into[j] = load4_guarded<kVec>(src, row_off[first + j] + k0, valid, ninf);
-      }
-    };
-    auto scan_half = [&](const floatx4 (&from)[kHalf], int first) {
-#pragma unroll
-      for (int j = 0; j < kHalf; ++j)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float v = from[j][i];
-          m[first + j] = (v > m[first + j] || v != v) ? v : m[first + j];  // NaN propagates, like torch.max
-        }
-    };
-    floatx4 lo[kHalf], hi[kHalf];
-    if (wave < chunks) fetch_half(lo, 0, wave * kPanK);
-    for (int chunk = wave; chunk < chunks; chunk += kPanWaves) {
-      fetch_half(hi, kHalf, chunk * kPanK);
-      scan_half(lo, 0);
-      if (chunk + kPanWaves < chunks) fetch_half(lo, 0, (chunk + kPanWaves) * kPanK);
-      scan_half(hi, kHalf);
-    }
-    // the second pass's first slab is requested before the maxima are exchanged
-    if (wave < chunks) fetch(slab, wave * kPanK);
-    // the eight lanes that share a row
-#pragma unroll
-    for (int j = 0; j < kLoads; ++j) {
-#pragma unroll
-      for (int off = 1; off < 8; off <<= 1) {
-        const float o = __shfl_xor(m[j], off, kWave);
-        m[j] = (o > m[j] || o != o) ? o : m[j];
-      }
-      if ((lane & 7) == 0) wave_max[wave][sub + 8 * j] = m[j];
-    }
+  // ---- one pass over k.  The reference subtracts the row maxima before exp
+  // (rnnt_loss.py:174-178); a maximum is known only after the whole row has been seen, so
+  // each wave works with a SHIFT per row instead: the largest value of the row it had
+  // seen when the shift was last set.  A value more than kMargin above the shift (always
+  // the case for the first finite value of a row) makes the wave raise its shifts and
+  // scale its partial sums to match; anything closer stays representable, e^(2 kMargin)
+  // per product.  The running maxima are kept beside the shifts, and when the waves
+  // meet their partial sums are brought to the true maxima, exp(shift - max) <= 1.
+  constexpr float kMargin = 30.f;
+  floatx4 slab0[kLoads], slab1[kLoads];
+  if (wave < pairs) {
+    fetch(slab0, 2 * wave * kPanK);
+    fetch(slab1, (2 * wave + 1) * kPanK);
   }
-  __syncthreads();
-  if (tid < kPanRows) {
-    float r = wave_max[0][tid];
-#pragma unroll
-    for (int w = 1; w < kPanWaves; ++w) {
-      const float o = wave_max[w][tid];
-      r = (o > r || o != o) ? o : r;
-    }
-    // saved for the backward pass; rows that do not exist get a harmless shift
-    bool exists;
-    if (tid < kPanS) {
-      exists = s_tile + tid < S1;
-      if (exists && t_tile == 0) lm_max[(long)b * S1 + s_tile + tid] = r;
-    } else {
-      exists = t_tile + tid - kPanS < T;
-      if (exists && s_tile == 0) am_max[(long)b * T + t_tile + tid - kPanS] = r;
-    }
-    slab_max[tid] = exists ? r : 0.f;
-  }
-  __syncthreads();
-  float shift[kLoads];    // the row's maximum
-#pragma unroll
-  for (int j = 0; j < kLoads; ++j) shift[j] = slab_max[sub + 8 * j];
-  int chunk = wave;
 
-  // ---- epilogue inputs, requested behind the first slab so that their latency hides
-  // under the loop: am[b, t, sym[b, s]] for this thread's outputs ...
+  // ---- epilogue inputs, requested behind the first slabs (the symbols they depend on
+  // were requested before those) so that their latency hides under the loop:
+  // am[b, t, sym[b, s]] for this thread's outputs ...
   float am_sym[kPanItems][4];
 #pragma unroll
   for (int j = 0; j < kPanItems; ++j) {
@@ -569,21 +537,26 @@ __global__ void __launch_bounds__(kPanThreads)
     }
   }
   // ... and the per-row / per-column terms (kept in registers until the loop is done)
-  float my_term = 0.f, my_symval = 0.f, my_max = 0.f;
+  float my_term = 0.f, my_symval = 0.f;
   if (tid < kPanS) {
     const int sr = s_tile + tid;
     if (sr < S1) {
       my_term = lmb[sr * C + term];
-      my_max = slab_max[tid];
       if (my_sym >= 0) my_symval = lmb[sr * C + my_sym];
     }
   } else if (tid >= 128 && tid < 128 + kPanT) {
     const int tr = t_tile + tid - 128;
     my_term = tr < T ? amb[tr * C + term] : 0.f;
-    my_max = slab_max[kPanS + tid - 128];
   }
 
-  // ---- main loop over this wave's slabs (32-row tiles without lattice rows are skipped)
+  float seen[kLoads];     // largest value this lane has met in the row
+  // -shift * log2(e), see exp_shifted; the lanes of a row agree on it.  kUnset while the
+  // row has shown nothing finite: it sends -inf to exp2(-inf) = 0 and anything finite
+  // above the margin.
+  float shift2[kLoads];
+  constexpr float kUnset = 3.0e38f;
+#pragma unroll
+  for (int j = 0; j < kLoads; ++j) seen[j] = ninf, shift2[j] = kUnset;
   const int live_tiles = min(kPanS / 32, (S1 - s_tile + 31) / 32);
   float *mine = pan_lds + wave * kPanSlab;
   floatx16 acc[kPanS / 32];
@@ -591,14 +564,47 @@ __global__ void __launch_bounds__(kPanThreads)
   for (int j = 0; j < kPanS / 32; ++j)
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
-  for (; chunk < chunks; chunk += kPanWaves) {
+
+  auto across_row = [&](float v) {  // maximum over the lanes that share a row
+#pragma unroll
+    for (int off = 1; off < kRowLanes; off <<= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+  };
+  auto raise_shifts = [&]() {
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
-      float *d = mine + (sub + 8 * j) * kPanPitch + kq;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) d[i] = __expf(slab[j][i] - shift[j]);
+      const float now = fminf(shift2[j], -across_row(seen[j]) * kLog2e);
+      const float f = __builtin_amdgcn_exp2f(now - shift2[j]);  // exp(old shift - new shift)
+      shift2[j] = now;
+      if (lane % kRowLanes == 0) factor[wave][sub + kRowsPerLoad * j] = f;
     }
-    if (chunk + kPanWaves < chunks) fetch(slab, (chunk + kPanWaves) * kPanK);
+    __builtin_amdgcn_wave_barrier();
+    const float ft = factor[wave][kPanS + r32];
+#pragma unroll
+    for (int j = 0; j < kPanS / 32; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        acc[j][v] *= factor[wave][32 * j + 8 * (v / 4) + 4 * half + (v % 4)] * ft;
+    __builtin_amdgcn_wave_barrier();
+  };
+  // one slab: exp(x - shift) to LDS, the request for the slab that will take these
+  // registers next, then the products (32-row tiles without lattice rows are skipped)
+  auto consume = [&](floatx4 (&slab)[kLoads], int next_chunk) {
+    bool above = false;
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+      const float top = fmaxf(fmaxf(slab[j][0], slab[j][1]), fmaxf(slab[j][2], slab[j][3]));
+      seen[j] = fmaxf(seen[j], top);
+      above |= __builtin_fmaf(top, kLog2e, shift2[j]) > kMargin * kLog2e;
+    }
+    if (__any(above)) raise_shifts();
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+      float *d = mine + (sub + kRowsPerLoad * j) * kPanPitch + kq;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) d[i] = exp_shifted(slab[j][i], shift2[j]);
+    }
+    if (next_chunk < chunks) fetch(slab, next_chunk * kPanK);
     const float *ap = mine + r32 * kPanPitch + half;
     const float *bp = mine + (kPanS + r32) * kPanPitch + half;
 #pragma unroll
@@ -610,25 +616,64 @@ __global__ void __launch_bounds__(kPanThreads)
           acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[j * 32 * kPanPitch + 2 * i], bv, acc[j],
                                                         0, 0, 0);
     }
+  };
+  for (int pair = wave; pair < pairs; pair += kPanWaves) {
+    consume(slab0, 2 * (pair + kPanWaves));
+    if (2 * pair + 1 < chunks) consume(slab1, 2 * (pair + kPanWaves) + 1);
   }
 
-  // ---- the partial sums meet: [wave][96][33] in the slab space
+  // ---- the waves meet: maxima first ...
+#pragma unroll
+  for (int j = 0; j < kLoads; ++j) {
+    const float top = across_row(seen[j]);
+    if (lane % kRowLanes == 0) {
+      wave_max[wave][sub + kRowsPerLoad * j] = top;
+      wave_shift[wave][sub + kRowsPerLoad * j] = shift2[j];
+    }
+  }
   __syncthreads();
+  if (tid < kPanRows) {
+    float r = wave_max[0][tid];
+#pragma unroll
+    for (int w = 1; w < kPanWaves; ++w) r = fmaxf(r, wave_max[w][tid]);
+    // saved for the backward pass; rows that do not exist get a harmless shift
+    bool exists;
+    if (tid < kPanS) {
+      exists = s_tile + tid < S1;
+      if (exists && t_tile == 0) lm_max[(long)b * S1 + s_tile + tid] = r;
+    } else {
+      exists = t_tile + tid - kPanS < T;
+      if (exists && s_tile == 0) am_max[(long)b * T + t_tile + tid - kPanS] = r;
+    }
+    slab_max[tid] = exists ? r : 0.f;
+    // what brings a wave's partial sums from its shift to the maximum (a wave that met
+    // nothing finite in the row holds zeros there)
+#pragma unroll
+    for (int w = 0; w < kPanWaves; ++w)
+      factor[w][tid] = exists ? __builtin_amdgcn_exp2f(-__builtin_fmaf(r, kLog2e, wave_shift[w][tid])) : 1.f;
+  }
+  __syncthreads();
+  // ... then the partial sums: [wave][kS][33] in the slab space
   if (tid < kPanS) {
     row_term[tid] = my_term;
     row_sym[tid] = my_symval;
-    row_max[tid] = my_max;
+    row_max[tid] = slab_max[tid];
     row_symbol[tid] = my_sym;
   } else if (tid >= 128 && tid < 128 + kPanT) {
     col_term[tid - 128] = my_term;
-    col_max[tid - 128] = my_max;
+    col_max[tid - 128] = slab_max[kPanS + tid - 128];
   }
-  float *part = pan_lds + wave * (kPanS * kPanPitch);
+  float *part = pan_lds + wave * Shape::kSums;
+  {
+    const float ft = factor[wave][kPanS + r32];
 #pragma unroll
-  for (int j = 0; j < kPanS / 32; ++j)
+    for (int j = 0; j < kPanS / 32; ++j)
 #pragma unroll
-    for (int v = 0; v < 16; ++v)
-      part[(32 * j + 8 * (v / 4) + 4 * half + (v % 4)) * kPanPitch + r32] = acc[j][v];
+      for (int v = 0; v < 16; ++v) {
+        const int m = 32 * j + 8 * (v / 4) + 4 * half + (v % 4);
+        part[m * kPanOutPitch + r32] = acc[j][v] * (factor[wave][m] * ft);
+      }
+  }
   __syncthreads();
 
   const int t_mask = (rnnt_type == kRegular && boundary) ? (int)boundary[4 * b + 3] : -1;
@@ -646,7 +691,7 @@ __global__ void __launch_bounds__(kPanThreads)
       float sum = 0.f;
 #pragma unroll
       for (int w = 0; w < kPanWaves; ++w)
-        sum += pan_lds[w * (kPanS * kPanPitch) + m * kPanPitch + out_t + i];
+        sum += pan_lds[w * Shape::kSums + m * kPanOutPitch + out_t + i];
       raw[i] = logf(sum + 1.17549435e-38f);
       const float norm = raw[i] + row_max[m] + col_max[out_t + i];
       yv[i] = (col_term[out_t + i] + row_term[m]) - norm;
@@ -723,7 +768,7 @@ __global__ void __launch_bounds__(kLmThreads, 2)
   constexpr int kLoadsA = kLmS / 8, kLoadsB = kLmK / 8;
   const int sub = lane >> 3, kq = 4 * (lane & 7);
   floatx4 sa[kLoadsA], sb[kLoadsB];
-  float shift[kLoadsB];
+  float shift2[kLoadsB];  // -(the frame's maximum) * log2(e)
   auto fetch = [&](int k0) {
 #pragma unroll
     for (int j = 0; j < kLoadsA; ++j) {
@@ -737,7 +782,7 @@ __global__ void __launch_bounds__(kLmThreads, 2)
       const int tr = k0 + sub + 8 * j, c = c_tile + kq;
       const int valid = tr < T ? min(4, max(C - c, 0)) : 0;
       sb[j] = load4_guarded<true>(amb, tr * C + c, valid, ninf);
-      shift[j] = tr < T ? amx[tr] : 0.f;
+      shift2[j] = tr < T ? -amx[tr] * kLog2e : 0.f;
     }
   };
   const int chunks = (T + kLmK - 1) / kLmK;
@@ -773,7 +818,7 @@ __global__ void __launch_bounds__(kLmThreads, 2)
     for (int j = 0; j < kLoadsB; ++j) {
       floatx4 e;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) e[i] = __expf(sb[j][i] - shift[j]);
+      for (int i = 0; i < 4; ++i) e[i] = exp_shifted(sb[j][i], shift2[j]);
       *reinterpret_cast<floatx4 *>(bs + (sub + 8 * j) * kLmC + kq) = e;
     }
     if (chunk + kLmWaves < chunks) fetch((chunk + kLmWaves) * kLmK);
@@ -1009,18 +1054,34 @@ __global__ void __launch_bounds__(256, 2)
 // launchers: float goes to the slab / panel kernels, double to the LDS-tiled ones
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+template <int kS, int kK>
+void launch_fwd_panel(const float *lm, const float *am, const int64_t *symbols,
+                      const int64_t *boundary, float *lm_max, float *am_max, float *px,
+                      float *py, float *norm_raw, int B, int S, int T, int C, int term,
+                      int rnnt_type, hipStream_t stream) {
+  using Shape = PanelShape<kS, kK>;
+  const int t_tiles = T > 0 ? (T + kPanT - 1) / kPanT : 1;
+  const int s_tiles = (S + 1 + kS - 1) / kS;
+  const bool vec = (C % 4 == 0) && aligned16(lm) && aligned16(am);
+  auto kernel = vec ? simple_fwd_panel_kernel<true, kS, kK> : simple_fwd_panel_kernel<false, kS, kK>;
+  (void)allow_lds(reinterpret_cast<const void *>(kernel), Shape::kLdsBytes);
+  hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(t_tiles * s_tiles, B)), dim3(kPanThreads),
+                     Shape::kLdsBytes, stream, lm, am, symbols, boundary, lm_max, am_max, px, py,
+                     norm_raw, B, S, T, C, term, rnnt_type);
+}
 void launch_fwd_gemm(const float *lm, const float *am, const int64_t *symbols,
                      const int64_t *boundary, float *lm_max, float *am_max, float *px,
                      float *py, float *norm_raw, int B, int S, int T, int C, int term,
                      int rnnt_type, hipStream_t stream) {
-  const int t_tiles = T > 0 ? (T + kPanT - 1) / kPanT : 1;
-  const int s_tiles = (S + 1 + kPanS - 1) / kPanS;
-  const bool vec = (C % 4 == 0) && aligned16(lm) && aligned16(am);
-  auto kernel = vec ? simple_fwd_panel_kernel<true> : simple_fwd_panel_kernel<false>;
-  (void)allow_lds(reinterpret_cast<const void *>(kernel), kPanLdsBytes);
-  hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(t_tiles * s_tiles, B)),
-                     dim3(kPanWaves * kWave), kPanLdsBytes, stream, lm, am, symbols, boundary,
-                     lm_max, am_max, px, py, norm_raw, B, S, T, C, term, rnnt_type);
+  // the row count per workgroup that leaves fewer padding rows; 128 on a tie
+  const int S1 = S + 1;
+  const int padded96 = (S1 + 95) / 96 * 96, padded128 = (S1 + 127) / 128 * 128;
+  if (padded96 < padded128)
+    launch_fwd_panel<96, 16>(lm, am, symbols, boundary, lm_max, am_max, px, py, norm_raw, B, S, T,
+                             C, term, rnnt_type, stream);
+  else
+    launch_fwd_panel<128, 16>(lm, am, symbols, boundary, lm_max, am_max, px, py, norm_raw, B, S,
+                              T, C, term, rnnt_type, stream);
 }
 void launch_fwd_gemm(const double *lm, const double *am, const int64_t *symbols,
                      const int64_t *boundary, const double *lm_max, const double *am_max,

@@ -1,7 +1,8 @@
 """rnnt_loss_simple / get_rnnt_logprobs on the GPU against the CPU oracle.
 
-Tolerances (float32): loss 1e-5 relative, px_grad / py_grad 1e-4 absolute,
-am.grad / lm.grad 1e-4 absolute; float64: 1e-9.
+Tolerances (float32): loss 1e-5 relative, px_grad / py_grad 1e-4 absolute
+(2.5e-4 at the large-vocabulary workload, see _GRAD_BOUND), am.grad / lm.grad the same
+absolute + 1e-4 relative; float64: 1e-9.
 """
 import sys
 
@@ -68,6 +69,65 @@ def test_logprobs_match_oracle(gpu_device, dtype, kind):
             assert _close(gy, wy, tol, tol)
 
 
+@pytest.mark.parametrize("rows", [20, 110])
+def test_normalizer_where_the_maximum_comes_late(gpu_device, rows):
+    """The float32 normalizer kernel meets a row's maximum only at the end of its pass over
+    the vocabulary: rows that keep growing along the vocabulary, rows that start with -inf,
+    rows that are -inf or hold one huge entry, and a wide spread must all come out as the
+    reference's max-then-exp form gives them (rnnt_loss.py:174-186).  The truth is the
+    float64 oracle; the tolerance is that of test_logprobs_match_oracle."""
+    dev = gpu_device
+    B, S, T, C = 2, rows, 70, 333
+    g = torch.Generator().manual_seed(7)
+    am = torch.randn(B, T, C, generator=g)
+    lm = torch.randn(B, S + 1, C, generator=g)
+    ramp = torch.arange(C, dtype=torch.float32)
+    lm[0, 0] += 0.9 * ramp - 150.0          # grows by 300 along the vocabulary
+    lm[0, 1] -= 0.9 * ramp                  # falls by 300
+    am[0, 0] += 2.5 * ramp                  # grows by 830: the shift is raised again and again
+    am[0, 1, :40] = float("-inf")           # nothing finite in the first slabs
+    lm[0, 2, :200] = float("-inf")
+    lm[0, 3, 17] = 3.0e4                    # one huge entry
+    am[0, 2, C - 1] = -2.0e4
+    am[0, 3] *= 40.0                        # wide spread
+    lm[1, 4] *= 25.0
+    am[1, 5, 1:] = float("-inf")            # a single finite entry, at the very start
+    lm[1, 6, : C - 1] = float("-inf")       # ... and at the very end
+    am[1, 7, 1:] = -1.0e4                   # the same with numerators that stay finite
+    lm[1, 8, : C - 1] = -1.0e4
+    sym = torch.randint(0, C, (B, S), generator=g)
+    term = 250
+    tx, ty = O.lattice_logprobs_simple(lm.double(), am.double(), sym, term)
+    wx, wy = O.lattice_logprobs_simple(lm, am, sym, term)
+    gx, gy = fast_rnnt_amd.get_rnnt_logprobs(lm.to(dev), am.to(dev), sym.to(dev), term)
+    gx, gy = gx.cpu(), gy.cpu()
+    # Where a steep lm row meets a steep am row every product underflows in float32 and the
+    # reference's own result is log(tiny); those cells say nothing.  Everywhere else the
+    # float32 reference agrees with float64, and so must the kernel.
+    def sound_cells(ref, truth):
+        finite = torch.isfinite(truth) & ((ref.double() - truth).abs() <= 1e-4 * (1 + truth.abs()))
+        return finite | (torch.isinf(truth) & (ref.double() == truth))
+
+    for name, got, ref, truth in (("px", gx, wx, tx), ("py", gy, wy, ty)):
+        sound = sound_cells(ref, truth)
+        _say(f"  rows={rows} {name}: {sound.float().mean().item():.3f} of the cells are sound")
+        assert sound.float().mean().item() > 0.9
+        assert not torch.isnan(got[~torch.isnan(truth)]).any()
+        assert _close(got.double()[sound], truth[sound], 2e-5, 2e-5)
+    # every special row meets the ordinary frames, and every special frame the ordinary
+    # rows, in sound cells
+    sound = sound_cells(wy, ty)
+    assert sound[0, :4, 10:].all() and sound[0, 10:, :4].all()
+    assert sound[1, [4, 6, 8], 10:].all() and sound[1, 10:, [5, 7]].all()
+    assert torch.isfinite(ty[1, 8, 10:]).all() and torch.isfinite(ty[1, 10:, 7]).all()
+    # a row without a finite entry has no normalizer: NaN, as in the reference
+    lm[1, 9] = float("-inf")
+    wx, wy = O.lattice_logprobs_simple(lm, am, sym, term)
+    gx, gy = fast_rnnt_amd.get_rnnt_logprobs(lm.to(dev), am.to(dev), sym.to(dev), term)
+    assert torch.isnan(wy[1, 9]).all() and torch.isnan(gy.cpu()[1, 9]).all()
+    assert _close(gy[1, 10:, 10:].double(), ty[1, 10:, 10:], 2e-5, 2e-5)
+
+
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 def test_loss_and_all_gradients(gpu_device, dtype, kind):
@@ -119,6 +179,17 @@ def test_delay_penalty_and_only_one_input_needs_grad(gpu_device):
         fast_rnnt_amd.rnnt_loss_simple(dl, am.to(dev), sym.to(dev), 0, reduction="bogus")
 
 
+# One float32 ulp of the lattice scores p is 2.4e-4 at |p| ~ 3000 (c2, c4 per utterance).
+# The occupation gradients are exp of differences of p, so once px / py differ in their
+# last bit between two pipelines (the normalizer's summation order differs between any two
+# GEMMs), a cell of p that rounds the other way moves the gradients around it by up to
+# one such ulp times the occupation there.  1e-4 holds at c1 and c2; at c4 the measured
+# difference is 2.1e-4 and the bound one ulp of p, 2.5e-4.  What keeps that honest is
+# the second check: against the float64 oracle the GPU's gradients must be as close as
+# the float32 CPU reference's own.
+_GRAD_BOUND = {"c1": 1e-4, "c2": 1e-4, "c4": 2.5e-4}
+
+
 @pytest.mark.parametrize("name", ["c1", "c2", "c4"])
 def test_baseline_configs(gpu_device, name):
     dev = gpu_device
@@ -130,6 +201,8 @@ def test_baseline_configs(gpu_device, name):
                                    return_grad=True)
     wx0, wy0 = wx.clone(), wy.clone()
     want.backward()
+    _, (tx, ty) = O.loss_simple(w.lm.double(), w.am.double(), w.symbols, 0, boundary=w.boundary,
+                                reduction="sum", return_grad=True)
     da = w.am.to(dev).requires_grad_(True)
     dl = w.lm.to(dev).requires_grad_(True)
     got, (gx, gy) = fast_rnnt_amd.rnnt_loss_simple(
@@ -138,11 +211,17 @@ def test_baseline_configs(gpu_device, name):
     gx0, gy0 = gx.clone(), gy.clone()
     got.backward()
     rel = abs(got.item() - want.item()) / abs(want.item())
+    gpu_off = max((gx0.cpu().double() - tx).abs().max().item(),
+                  (gy0.cpu().double() - ty).abs().max().item())
+    cpu_off = max((wx0.double() - tx).abs().max().item(), (wy0.double() - ty).abs().max().item())
     _say(f"  loss gpu={got.item():.6f} cpu={want.item():.6f} rel={rel:.2e} "
          f"px_grad maxdiff={(gx0.cpu() - wx0).abs().max().item():.2e} "
          f"py_grad maxdiff={(gy0.cpu() - wy0).abs().max().item():.2e} "
          f"am.grad maxdiff={(da.grad.cpu() - a.grad).abs().max().item():.2e} "
-         f"lm.grad maxdiff={(dl.grad.cpu() - l.grad).abs().max().item():.2e}")
+         f"lm.grad maxdiff={(dl.grad.cpu() - l.grad).abs().max().item():.2e}; "
+         f"px/py_grad against float64: gpu {gpu_off:.2e}, cpu float32 {cpu_off:.2e}")
     assert rel <= 1e-5
-    assert _close(gx0, wx0, 1e-4) and _close(gy0, wy0, 1e-4)
-    assert _close(da.grad, a.grad, 1e-4, 1e-4) and _close(dl.grad, l.grad, 1e-4, 1e-4)
+    bound = _GRAD_BOUND[name]
+    assert _close(gx0, wx0, bound) and _close(gy0, wy0, bound)
+    assert gpu_off <= 1.5 * cpu_off + 2e-5
+    assert _close(da.grad, a.grad, bound, 1e-4) and _close(dl.grad, l.grad, bound, 1e-4)
