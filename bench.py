@@ -27,7 +27,7 @@ FP32_MFMA_PEAK_TFLOPS = 157.3
 # profiles/ (FETCH_SIZE and WRITE_SIZE, scaled by what the same counters read for a
 # copy of known size); filled in for the workloads that were profiled
 MEASURED_TRAFFIC = {
-    ("c2", "simple_fwd_panel_kernel<true>"): 29494871,
+    ("c2", "simple_fwd_panel_kernel<true, 96, 16>"): 29494871,
     ("c2", "mi_forward_kernel<float, false, 2>"): 6877090,
     ("c2", "mi_backward_kernel<float, false, 2>"): 9790310,
 }
@@ -42,6 +42,8 @@ def _parse():
     ap.add_argument("--cpu-seconds", type=float, default=12.0,
                     help="budget of the CPU-baseline leg (0 disables it)")
     ap.add_argument("--kernel-reps", type=int, default=50)
+    ap.add_argument("--no-graph", dest="graph", action="store_false",
+                    help="skip the graph-replay leg")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run device-to-device copies of this size (a reference of known "
                          "traffic for hardware-counter runs)")
@@ -62,6 +64,57 @@ def _event_time_ms(fn, reps):
     stop.record()
     stop.synchronize()
     return start.elapsed_time(stop) / reps
+
+
+def _graph_replay(step, am, lm, args):
+    """Captures one step (forward and backward through autograd) in a HIP graph and times
+    `args.steps` replays; every replay recomputes the loss and both gradients in place.
+    Checked against an eager step before and after the timed replays."""
+    try:
+        # the gradient-accumulation nodes of am / lm were made on the default stream
+        # by the eager steps; autograd's note about that is not an error
+        quiet = getattr(torch.autograd.graph, "set_warn_on_accumulate_grad_stream_mismatch", None)
+        if quiet is not None:
+            quiet(False)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            loss = step()
+        g_am, g_lm = am.grad, lm.grad   # the graph's own output tensors
+
+        def differs():
+            graph.replay()
+            torch.cuda.synchronize()
+            got = (loss.clone(), g_am.clone(), g_lm.clone())
+            want_loss = step()          # eager work between replays
+            torch.cuda.synchronize()
+            same = (torch.equal(got[0], want_loss) and torch.equal(got[1], am.grad)
+                    and torch.equal(got[2], lm.grad))
+            return not same
+
+        if differs():
+            return {"error": "replay differs from the eager step"}
+        for _ in range(args.warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        if differs():
+            return {"error": "replay differs from the eager step after the timed replays"}
+        return {"value": round(args.steps / elapsed, 2), "unit": "calls/sec",
+                "ms_per_step": round(1e3 * elapsed / args.steps, 4), "steps": args.steps,
+                "checked": "loss and both gradients bit-equal to an eager step, before and after"}
+    except Exception as err:  # the eager figure stands on its own
+        return {"error": f"{type(err).__name__}: {err}"}
 
 
 def _recursion_bytes(boundary, S, T, B, backward):
@@ -231,6 +284,10 @@ def main():
     ms_per_step = 1e3 * elapsed / args.steps
     calls_per_sec = args.steps / elapsed
 
+    # ---- the same step captured once in a HIP graph and replayed: what the device
+    # sustains when the host's launch cost (nine short kernels per step) is out of the way
+    replay = _graph_replay(step, am, lm, args) if args.graph else None
+
     # ---- per-stage kernel timings (events on the launch stream) -------------------
     with torch.no_grad():
         px, py = fast_rnnt_amd.get_rnnt_logprobs(lm, am, sym, 0, boundary=bnd)
@@ -255,9 +312,10 @@ def main():
                 "avg_launch_us": round(1e3 * t_ms, 2)}
 
     # normalizer contraction exp(lm - max) . exp(am - max)^T on the fp32 matrix cores;
-    # the same kernel first scans its operands for the row maxima and assembles px/py
-    # at the end, so this figure is a lower bound on the rate of its MFMA loop
-    gemm_name = "simple_fwd_panel_kernel<true>"
+    # the same kernel finds the row maxima on the way and assembles px/py at the end,
+    # so this figure is a lower bound on the rate of its MFMA loop
+    gemm_name = "simple_fwd_panel_kernel<true, 96, 16>" if (S + 1 + 95) // 96 * 96 < (S + 1 + 127) // 128 * 128 \
+        else "simple_fwd_panel_kernel<true, 128, 16>"
     gemm_flops = 2.0 * B * (S + 1) * T * w.C
     gemm_tflops = gemm_flops / (t_logp * 1e-3) / 1e12
     lines = [
@@ -333,6 +391,7 @@ def main():
         "roofline": roofline,
         "roofline_other_kernels": other,
         "cpu_baseline": cpu,
+        "graph_replay": replay,
         "stages": {k: round(v, 4) for k, v in stages.items()},
         "whole_call_hbm_GBs": round(workloads.simple_call_bytes(w) / elapsed * args.steps / 1e9, 2),
     }

@@ -90,6 +90,58 @@ __global__ void __launch_bounds__(kWave)
   ranges[((long)b * T + t) * Rr] = ((int64_t)t < Tb - 1) ? (int64_t)best : tail;
 }
 
+// The same with the 64 frames' columns of py_grad and px_grad staged in LDS first: every
+// load of the tile is in flight at once (the kernel above walks the rows with a few loads
+// in flight), and the four waves share the candidate starts, each scanning a contiguous
+// quarter; wave 0 then takes the quarters' winners in order under the same rule, which
+// is the sequential scan's result.
+template <typename R>
+__global__ void __launch_bounds__(256)
+    prune_starts_tile_kernel(const R *__restrict__ px_grad, const R *__restrict__ py_grad,
+                             const int64_t *__restrict__ boundary, int64_t *__restrict__ ranges,
+                             int S, int T, int T1, int Rr) {
+  extern __shared__ unsigned char tile_raw[];
+  __shared__ int seg_best[4][kWave];
+  __shared__ R seg_score[4][kWave];
+  R *ty = reinterpret_cast<R *>(tile_raw);  // [S + 1][64]
+  R *tx = ty + (S + 1) * kWave;             // [S][64]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int b = blockIdx.y, t = blockIdx.x * kWave + lane;
+  const bool ok = t < T;
+  const R *gx = px_grad + (long)b * S * T1 + t;
+  const R *gy = py_grad + (long)b * (S + 1) * T + t;
+  for (int s = wave; s <= S; s += 4) ty[s * kWave + lane] = ok ? gy[(long)s * T] : (R)0;
+  for (int s = wave; s < S; s += 4) tx[s * kWave + lane] = ok ? gx[(long)s * T1] : (R)0;
+  __syncthreads();
+  const int n = S + 2 - Rr;  // candidate window starts
+  const int per = (n + 3) / 4, lo = wave * per, hi = min(n, lo + per);
+  int best = -1;
+  R best_score = 0;
+  // first maximum wins; a NaN score counts as the maximum, like torch.argmax
+  auto consider = [&](int s, R score) {
+    if (best < 0 || score > best_score || (score != score && best_score == best_score)) {
+      best = s;
+      best_score = score;
+    }
+  };
+  for (int s = lo; s < hi; ++s) {
+    R sum = ty[s * kWave + lane];
+    for (int j = 1; j < Rr; ++j) sum = sum + ty[(s + j) * kWave + lane];
+    const R below = s >= 1 ? tx[(s - 1) * kWave + lane] : (R)0;
+    consider(s, sum - below);
+  }
+  seg_best[wave][lane] = best;
+  seg_score[wave][lane] = best_score;
+  __syncthreads();
+  if (wave != 0 || !ok) return;
+  for (int w = 1; w < 4; ++w)
+    if (seg_best[w][lane] >= 0) consider(seg_best[w][lane], seg_score[w][lane]);
+  const int64_t Sb = boundary[4 * b + 2], Tb = boundary[4 * b + 3];
+  int64_t tail = Sb - Rr + 1;
+  if (tail < 0) tail = 0;
+  ranges[((long)b * T + t) * Rr] = ((int64_t)t < Tb - 1) ? (int64_t)best : tail;
+}
+
 // Step 2, one wave per utterance: the starts are made non-decreasing with bounded
 // steps by two suffix-minimum passes and expanded to the R entries of each frame.
 __global__ void __launch_bounds__(kWave)
@@ -212,9 +264,16 @@ int ranges_impl(const R *px_grad, const R *py_grad, const int64_t *boundary, int
   if (!allow_lds(reinterpret_cast<const void *>(prune_monotone_kernel), lds))
     return check_launch("prune_ranges: hipFuncSetAttribute");
   const int T1 = modified ? T : T + 1;
-  hipLaunchKernelGGL(prune_starts_kernel<R>, dim3((T + kWave - 1) / kWave, B), dim3(kWave), 0,
-                     static_cast<hipStream_t>(stream), px_grad, py_grad, boundary, ranges, S, T,
-                     T1, s_range);
+  const size_t tile_lds = (size_t)(2 * S + 1) * kWave * sizeof(R);
+  if (tile_lds <= 144 * 1024 &&
+      allow_lds(reinterpret_cast<const void *>(prune_starts_tile_kernel<R>), tile_lds))
+    hipLaunchKernelGGL(prune_starts_tile_kernel<R>, dim3((T + kWave - 1) / kWave, B), dim3(256),
+                       tile_lds, static_cast<hipStream_t>(stream), px_grad, py_grad, boundary,
+                       ranges, S, T, T1, s_range);
+  else
+    hipLaunchKernelGGL(prune_starts_kernel<R>, dim3((T + kWave - 1) / kWave, B), dim3(kWave), 0,
+                       static_cast<hipStream_t>(stream), px_grad, py_grad, boundary, ranges, S, T,
+                       T1, s_range);
   hipLaunchKernelGGL(prune_monotone_kernel, dim3(B), dim3(kWave), lds,
                      static_cast<hipStream_t>(stream), ranges, T, modified ? 2 : s_range, s_range);
   return check_launch("prune_ranges");

@@ -89,16 +89,62 @@ __global__ void __launch_bounds__(256)
                                    const R *__restrict__ numer, const R *__restrict__ denom,
                                    R *__restrict__ partial, long rows, int C) {
   const long row0 = (long)blockIdx.x * kRowsPerBlock;
+  // per-row weight and maximum (the same for every thread); rows past the end weigh nothing
+  R w[kRowsPerBlock], m[kRowsPerBlock];
+  long at[kRowsPerBlock];
+#pragma unroll
+  for (int k = 0; k < kRowsPerBlock; ++k) {
+    const bool ok = row0 + k < rows;
+    const long row = ok ? row0 + k : row0;
+    w[k] = ok ? (numer ? numer[row] : (R)1) / denom[row] : (R)0;
+    m[k] = row_max[row];
+    at[k] = row * C;
+  }
   for (int c = threadIdx.x; c < C; c += 256) {
+    R v[kRowsPerBlock];
+#pragma unroll
+    for (int k = 0; k < kRowsPerBlock; ++k) v[k] = x[at[k] + c];  // all in flight
     R acc = 0;
-    for (int k = 0; k < kRowsPerBlock; ++k) {
-      const long row = row0 + k;
-      if (row >= rows) break;
-      const R w = (numer ? numer[row] : (R)1) / denom[row];
-      acc += Num<R>::exp_(x[row * C + c] - row_max[row]) * w;
-    }
+#pragma unroll
+    for (int k = 0; k < kRowsPerBlock; ++k)
+      if (row0 + k < rows) acc += Num<R>::exp_(v[k] - m[k]) * w[k];
     partial[(long)blockIdx.x * C + c] = acc;
   }
+}
+
+// The reductions over all rows of the batch end in a sum per vocabulary entry.  A block
+// of 256 threads takes 16 entries: 16 groups of 16 threads, every group walks its share
+// of the rows (64-byte reads), and the groups' sums meet in LDS in a fixed order, so the
+// result does not depend on timing.
+constexpr int kColsPerBlock = 16;
+constexpr int kRowGroups = 16;
+
+template <typename R>
+__device__ __forceinline__ R sum_of_groups(R mine, R (*meet)[kColsPerBlock], int col, int grp) {
+  meet[grp][col] = mine;
+  __syncthreads();
+  R total = 0;
+  if (grp == 0)
+#pragma unroll
+    for (int k = 0; k < kRowGroups; ++k) total += meet[k][col];
+  return total;  // meaningful in group 0
+}
+
+// sum over this group's share of the partial rows, eight loads in flight, added in order
+template <typename R>
+__device__ __forceinline__ R sum_partials(const R *__restrict__ partial, int blocks, int C, int c,
+                                          int grp) {
+  R acc = 0;
+  int k = grp;
+  for (; k + 7 * kRowGroups < blocks; k += 8 * kRowGroups) {
+    R v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = partial[(long)(k + u * kRowGroups) * C + c];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc += v[u];
+  }
+  for (; k < blocks; k += kRowGroups) acc += partial[(long)k * C + c];
+  return acc;
 }
 
 // unigram[c] = (sum of the partials) / N + tiny
@@ -106,11 +152,12 @@ template <typename R>
 __global__ void __launch_bounds__(256)
     unigram_final_kernel(const R *__restrict__ partial, R *__restrict__ unigram, int blocks, long N,
                          int C) {
-  const int c = blockIdx.x * 256 + threadIdx.x;
-  if (c >= C) return;
-  R acc = 0;
-  for (int k = 0; k < blocks; ++k) acc += partial[(long)k * C + c];
-  unigram[c] = acc / (R)N + tiny_value<R>();
+  __shared__ R meet[kRowGroups][kColsPerBlock];
+  const int col = threadIdx.x % kColsPerBlock, grp = threadIdx.x / kColsPerBlock;
+  const int c = blockIdx.x * kColsPerBlock + col;
+  R acc = c < C ? sum_partials(partial, blocks, C, c, grp) : (R)0;
+  acc = sum_of_groups(acc, meet, col, grp);
+  if (grp == 0 && c < C) unigram[c] = acc / (R)N + tiny_value<R>();
 }
 
 // one wave per am row: maximum and z = sum_c exp(x - max) unigram[c]
@@ -248,25 +295,57 @@ __global__ void __launch_bounds__(256)
 }
 
 // gU[c] = a (sum_{(b,s): sym=c} rx + [c=term] sum ry) / U[c] - a sum of the partials,
-// the partials being sum_rows G[row] exp(am - max) / z[row]
+// the partials being sum_rows G[row] exp(am - max) / z[row].  Same layout as
+// unigram_final_kernel.  The (b, s) pairs pass through LDS in chunks -- symbol and
+// row_x, fetched once by the whole block -- and every group scans a contiguous share
+// of each chunk.
+constexpr int kPairChunk = 2048;
+
 template <typename R>
 __global__ void __launch_bounds__(256)
     unigram_grad_kernel(const R *__restrict__ partial, const int64_t *__restrict__ symbols,
                         const R *__restrict__ row_x, const R *__restrict__ row_y,
                         const R *__restrict__ unigram, R *__restrict__ g_unigram, int blocks,
                         int B, int S, int C, int term, R k_am) {
-  const int c = blockIdx.x * 256 + threadIdx.x;
-  if (c >= C) return;
-  R acc = 0;
-  for (int k = 0; k < blocks; ++k) acc += partial[(long)k * C + c];
-  R direct = 0;
-  const int S1 = S + 1;
-  for (int b = 0; b < B; ++b)
-    for (int s = 0; s < S1; ++s) {
-      if (s < S && symbols[(long)b * S + s] == c) direct += row_x[(long)b * S1 + s];
-      if (c == term) direct += row_y[(long)b * S1 + s];
+  __shared__ R meet[kRowGroups][kColsPerBlock];
+  __shared__ int pair_sym[kPairChunk];
+  __shared__ R pair_x[kPairChunk];
+  const int col = threadIdx.x % kColsPerBlock, grp = threadIdx.x / kColsPerBlock;
+  const int c = blockIdx.x * kColsPerBlock + col;
+  const int S1 = S + 1, n = B * S1;
+  R acc = c < C ? sum_partials(partial, blocks, C, c, grp) : (R)0, direct = 0;
+  for (int row0 = 0; row0 < n; row0 += kPairChunk) {
+    const int count = min(kPairChunk, n - row0);
+    __syncthreads();
+    for (int i = threadIdx.x; i < count; i += 256) {
+      const int row = row0 + i, b = row / S1, s = row - b * S1;
+      const int64_t y = s < S ? symbols[(long)b * S + s] : -1;
+      pair_sym[i] = (y >= 0 && y < C) ? (int)y : -1;
+      pair_x[i] = row_x[row];
     }
-  g_unigram[c] = k_am * direct / unigram[c] - k_am * acc;
+    __syncthreads();
+    const int share = (count + kRowGroups - 1) / kRowGroups;
+    const int first = grp * share, last = min(first + share, count);
+    for (int i = first; i < last; ++i)
+      if (pair_sym[i] == c) direct += pair_x[i];
+  }
+  if (c == term) {
+    const int share = (n + kRowGroups - 1) / kRowGroups;
+    const int first = grp * share, last = min(first + share, n);
+    int row = first;
+    for (; row + 8 <= last; row += 8) {
+      R v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = row_y[row + u];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) direct += v[u];
+    }
+    for (; row < last; ++row) direct += row_y[row];
+  }
+  acc = sum_of_groups(acc, meet, col, grp);
+  __syncthreads();
+  direct = sum_of_groups(direct, meet, col, grp);
+  if (grp == 0 && c < C) g_unigram[c] = k_am * direct / unigram[c] - k_am * acc;
 }
 
 // one wave per lm row
@@ -361,7 +440,7 @@ int fwd_impl(const R *lm, const R *am, const int64_t *symbols, const R *pxj, con
                      lm, lm_max, lm_sum, n_lm, C);
   hipLaunchKernelGGL(weighted_column_partial_kernel<R>, dim3(blocks), dim3(256), 0, stream, lm,
                      lm_max, (const R *)nullptr, lm_sum, partial, n_lm, C);
-  hipLaunchKernelGGL(unigram_final_kernel<R>, dim3((C + 255) / 256), dim3(256), 0, stream, partial,
+  hipLaunchKernelGGL(unigram_final_kernel<R>, dim3((C + kColsPerBlock - 1) / kColsPerBlock), dim3(256), 0, stream, partial,
                      unigram, blocks, n_lm, C);
   if (n_am > 0)
     hipLaunchKernelGGL(am_row_stats_kernel<R>, dim3((unsigned)((n_am + 3) / 4)), dim3(256), 0,
@@ -404,7 +483,7 @@ int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const R *lm_max, 
   if (n_am > 0)
     hipLaunchKernelGGL(weighted_column_partial_kernel<R>, dim3(blocks), dim3(256), 0, stream, am,
                        am_max, col_g, am_z, partial, n_am, C);
-  hipLaunchKernelGGL(unigram_grad_kernel<R>, dim3((C + 255) / 256), dim3(256), 0, stream, partial,
+  hipLaunchKernelGGL(unigram_grad_kernel<R>, dim3((C + kColsPerBlock - 1) / kColsPerBlock), dim3(256), 0, stream, partial,
                      symbols, row_x, row_y, unigram, g_unigram, n_am > 0 ? blocks : 0, B, S, C, term,
                      k_am);
   hipLaunchKernelGGL(smoothed_bwd_lm_kernel<R>, dim3((unsigned)((n_lm + 3) / 4)), dim3(256), 0,

@@ -124,6 +124,31 @@ def test_prune_ranges_random_bit_exact(gpu_device, dtype, kind):
             assert torch.equal(got.cpu(), want)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_prune_ranges_ties_nans_and_long_targets(gpu_device, dtype):
+    """Window scores with exact ties and NaNs (first maximum wins, NaN counts as the maximum,
+    as torch.argmax in rnnt_loss.py:735-741), on targets short enough for the kernel that
+    stages a frame tile in LDS and long enough (S = 300, and 160 in float64) for the one
+    that does not.  Bit-exact against the oracle."""
+    dev = gpu_device
+    for n, (B, S, T) in enumerate([(2, 37, 90), (1, 160, 170), (1, 300, 330)]):
+        g = torch.Generator().manual_seed(900 + n)
+        # few distinct values: many windows tie
+        gx = torch.randint(0, 3, (B, S, T + 1), generator=g).to(dtype) * 0.25
+        gy = torch.randint(0, 3, (B, S + 1, T), generator=g).to(dtype) * 0.25
+        gy[0, S // 2, 5::7] = float("nan")
+        gx[0, S // 3, 3::11] = float("nan")
+        Sb = torch.randint(S // 2, S + 1, (B,), generator=g)
+        Tb = torch.randint(T // 2, T + 1, (B,), generator=g)
+        z = torch.zeros(B, dtype=torch.int64)
+        bnd = torch.stack([z, z, Sb, Tb], 1)
+        for R in (2, 5, 9):
+            _say(f"ranges ties/NaN {dtype} B={B} S={S} T={T} R={R}")
+            want = O.prune_ranges(gx, gy, bnd, R)
+            got = fast_rnnt_amd.get_rnnt_prune_ranges(gx.to(dev), gy.to(dev), bnd.to(dev), R)
+            assert torch.equal(got.cpu(), want)
+
+
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 def test_pruned_pipeline(gpu_device, dtype, kind):
