@@ -185,8 +185,12 @@ __global__ void __launch_bounds__(256)
 // adjoint: one block per lm row (b, s).  The block first lists, in order, the entries
 // of ranges[b] that point at s (an ordered compaction through LDS; only a few dozen of
 // the T * R entries match), then sums those rows of the incoming gradient -- in that
-// order, so the result is deterministic -- with coalesced loads.
-constexpr int kHitCapacity = 4096;  // matches listed per round
+// order, so the result is deterministic -- with coalesced loads.  For the listing a
+// thread takes kScanPerThread consecutive entries (all requested at once), and one
+// prefix sum over the threads' counts places everybody's matches.
+constexpr int kHitCapacity = 4096;   // matches listed per round
+constexpr int kScanPerThread = 8;
+constexpr int kScanChunk = 256 * kScanPerThread;
 
 template <typename R>
 __global__ void __launch_bounds__(256)
@@ -194,7 +198,6 @@ __global__ void __launch_bounds__(256)
                          R *__restrict__ lm_grad, int TR, int S1, int C) {
   __shared__ int hits[kHitCapacity];
   __shared__ int wave_count[4];
-  __shared__ int listed;
   const int b = blockIdx.x / S1, s = blockIdx.x % S1;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t *rb = ranges + (long)b * TR;
@@ -204,27 +207,39 @@ __global__ void __launch_bounds__(256)
   int k_next = 0;
   // rounds only repeat when more than kHitCapacity entries point at s
   do {
-    if (tid == 0) listed = 0;
-    __syncthreads();
+    int listed = 0;  // the same in every thread
     int k0 = k_next;
-    for (; k0 < TR; k0 += 256) {
-      const int k = k0 + tid;
-      const bool hit = k < TR && rb[k] == s;
-      const unsigned long long mask = __ballot(hit);
-      if (lane == 0) wave_count[wave] = __popcll(mask);
+    for (; k0 < TR; k0 += kScanChunk) {
+      const int mine = k0 + tid * kScanPerThread;
+      int64_t v[kScanPerThread];
+#pragma unroll
+      for (int u = 0; u < kScanPerThread; ++u) v[u] = mine + u < TR ? rb[mine + u] : (int64_t)-1;
+      unsigned found = 0;
+#pragma unroll
+      for (int u = 0; u < kScanPerThread; ++u) found |= (v[u] == s ? 1u : 0u) << u;
+      const int count = __popc(found);
+      // exclusive prefix of the counts: over the wave, then over the four waves
+      int upto = count;
+#pragma unroll
+      for (int off = 1; off < kWave; off <<= 1) {
+        const int o = __shfl_up(upto, off, kWave);
+        if (lane >= off) upto += o;
+      }
+      __syncthreads();  // the previous chunk's wave_count has been read
+      if (lane == kWave - 1) wave_count[wave] = upto;
       __syncthreads();
-      const int base = listed;
       int before = 0, total = 0;
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
         if (w < wave) before += wave_count[w];
         total += wave_count[w];
       }
-      if (base + total > kHitCapacity) break;  // (uniform) this chunk waits for the next round
-      if (hit) hits[base + before + __popcll(mask & ((1ull << lane) - 1ull))] = k;
-      __syncthreads();
-      if (tid == 0) listed = base + total;
-      __syncthreads();
+      if (listed + total > kHitCapacity) break;  // (uniform) this chunk waits for the next round
+      int at = listed + before + upto - count;
+#pragma unroll
+      for (int u = 0; u < kScanPerThread; ++u)
+        if (found & (1u << u)) hits[at++] = mine + u;
+      listed += total;
     }
     k_next = k0;
     __syncthreads();
@@ -234,13 +249,20 @@ __global__ void __launch_bounds__(256)
       if (c >= C) continue;
       R acc = first_round ? (R)0 : dst[c];
       int i = 0;
-      for (; i + 4 <= n; i += 4) {
-        const R g0 = gb[(long)hits[i] * C + c], g1 = gb[(long)hits[i + 1] * C + c];
-        const R g2 = gb[(long)hits[i + 2] * C + c], g3 = gb[(long)hits[i + 3] * C + c];
-        acc += g0;
-        acc += g1;
-        acc += g2;
-        acc += g3;
+      for (; i + 8 <= n; i += 8) {
+        R g[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) g[u] = gb[(long)hits[i + u] * C + c];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc += g[u];
+      }
+      if (i + 4 <= n) {
+        R g[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) g[u] = gb[(long)hits[i + u] * C + c];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) acc += g[u];
+        i += 4;
       }
       for (; i < n; ++i) acc += gb[(long)hits[i] * C + c];
       dst[c] = acc;

@@ -798,6 +798,18 @@ __global__ void __launch_bounds__(kLmThreads, 2)
     const int sr = s_tile + item / 8, c = c_tile + 4 * (item % 8);
     lm_in[j] = load4_guarded<true>(lmb, sr * C + c, sr < S1 ? min(4, max(C - c, 0)) : 0);
   }
+  // ... and its rows' maximum, symbol and row sums
+  float row_mx[kLmItems], row_rx[kLmItems], row_ry[kLmItems];
+  int row_sym[kLmItems];
+#pragma unroll
+  for (int j = 0; j < kLmItems; ++j) {
+    const int sr = s_tile + (tid + kLmThreads * j) / 8;
+    const bool ok = sr < S1;
+    row_mx[j] = ok ? lmx[sr] : 0.f;
+    row_sym[j] = sr < S ? (int)symbols[(long)b * S + sr] : -1;
+    row_rx[j] = ok ? row_x[(long)b * S1 + sr] : 0.f;
+    row_ry[j] = ok ? row_y[(long)b * S1 + sr] : 0.f;
+  }
 
   const int live_tiles = min(kLmS / 32, (S1 - s_tile + 31) / 32);  // 32-row tiles with lattice rows
   float *as = lm_lds + wave * kLmSlab;
@@ -849,9 +861,8 @@ __global__ void __launch_bounds__(kLmThreads, 2)
     const int item = tid + kLmThreads * j;
     const int m = item / 8, n = 4 * (item % 8), sr = s_tile + m, c = c_tile + n;
     if (sr >= S1 || c >= C) continue;
-    const float mx = lmx[sr];
-    const int sym = sr < S ? (int)symbols[(long)b * S + sr] : -1;
-    const float rx = row_x[(long)b * S1 + sr], ry = row_y[(long)b * S1 + sr];
+    const float mx = row_mx[j], rx = row_rx[j], ry = row_ry[j];
+    const int sym = row_sym[j];
     float g[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {

@@ -218,6 +218,41 @@ def test_pruning_gather_and_its_gradient(gpu_device):
     assert _close(dl.grad, l.grad, 1e-5, 1e-5) and _close(da.grad, a.grad, 1e-5, 1e-5)
 
 
+def test_pruning_gradient_when_most_frames_share_a_row(gpu_device):
+    """do_rnnt_pruning's lm gradient (the adjoint of the gather, rnnt_loss.py:797-802)
+    when thousands of (frame, j) entries point at the same lm row: more than the adjoint
+    kernel lists per round (4096), in several scan chunks, plus rows nobody points at."""
+    dev = gpu_device
+    g = torch.Generator().manual_seed(5)
+    B, S, T, C, R = 2, 6, 2300, 5, 2
+    am = torch.randn(B, T, C, generator=g)
+    lm = torch.randn(B, S + 1, C, generator=g)
+    r0 = torch.full((B, T), 2, dtype=torch.int64)
+    r0[0, 2000:] = 4                     # rows 2, 3 get 2000 + 2000 entries, rows 4, 5 get 300
+    r0[1, ::3] = 0
+    ranges = r0.unsqueeze(2) + torch.arange(R)
+    w = torch.randn(B, T, R, C, generator=g)
+    l = lm.clone().requires_grad_(True)
+    _, lp = O.prune(am, l, ranges)
+    (lp * w).sum().backward()
+    dl = lm.to(dev).requires_grad_(True)
+    _, glp = fast_rnnt_amd.do_rnnt_pruning(am.to(dev), dl, ranges.to(dev))
+    (glp * w.to(dev)).sum().backward()
+    assert (l.grad[0, 6] == 0).all() and (dl.grad[0, 6].cpu() == 0).all()
+    # sums of up to 2300 terms: the order of the float32 additions may differ
+    assert _close(dl.grad, l.grad, 2e-4, 1e-5), (dl.grad.cpu() - l.grad).abs().max()
+    # ... all entries on one row
+    ranges = torch.ones(1, T, 2, dtype=torch.int64) * torch.tensor([3, 3])
+    w = torch.randn(1, T, 2, C, generator=g)
+    l = lm[:1].clone().requires_grad_(True)
+    _, lp = O.prune(am[:1], l, ranges)
+    (lp * w).sum().backward()
+    dl = lm[:1].to(dev).requires_grad_(True)
+    _, glp = fast_rnnt_amd.do_rnnt_pruning(am[:1].to(dev), dl, ranges.to(dev))
+    (glp * w.to(dev)).sum().backward()
+    assert _close(dl.grad, l.grad, 4e-4, 1e-5), (dl.grad.cpu() - l.grad).abs().max()
+
+
 def test_smoothed_golden(gpu_device):
     dev = gpu_device
     data = torch.load(os.path.join(GOLDEN, "smoothed_logprobs.pt"), weights_only=True)
