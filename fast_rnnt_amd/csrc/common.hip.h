@@ -98,4 +98,34 @@ __device__ __forceinline__ double from_lane_above(double v) {
   return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
 }
 
+// loss = -scores, -mean(scores) or -sum(scores) (rnnt_loss.py:330-340) by ONE wave: every
+// lane sums a contiguous slice, then a fixed butterfly over the lanes.
+template <typename R>
+__device__ __forceinline__ void reduce_scores(const R *__restrict__ scores, R *__restrict__ loss,
+                                              int B, int reduction, int lane) {
+  if (reduction == 0) {
+    for (int b = lane; b < B; b += kWave) loss[b] = -scores[b];
+    return;
+  }
+  const int per = (B + kWave - 1) / kWave;
+  R acc = 0;
+  for (int k = 0; k < per; ++k) {
+    const int b = lane * per + k;
+    if (b < B) acc += scores[b];
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
+  if (lane == 0) loss[0] = reduction == 1 ? -(acc / (R)B) : -acc;
+}
+
+// The recursion's backward with a gradient of ones which, on its way, also reduces the
+// forward's scores to the loss (a staging wave of the first workgroup does it once its
+// tiles are done): saves the launch of a reduction kernel.  Host side, mi_recursion.hip.
+int mi_backward_and_loss(const float *px, const int64_t *boundary, const float *p, float *px_grad,
+                         float *py_grad, const float *scores, float *loss, int B, int S, int T,
+                         int modified, int reduction, void *stream);
+int mi_backward_and_loss(const double *px, const int64_t *boundary, const double *p,
+                         double *px_grad, double *py_grad, const double *scores, double *loss,
+                         int B, int S, int T, int modified, int reduction, void *stream);
+
 }  // namespace frnnt

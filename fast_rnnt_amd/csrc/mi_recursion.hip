@@ -475,7 +475,8 @@ template <typename R, bool kModified, int kSweepCap>
 __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
     mi_backward_kernel(const R *__restrict__ px, const int64_t *__restrict__ boundary,
                        const R *__restrict__ p, R *ans_grad, R *__restrict__ px_grad,
-                       R *__restrict__ py_grad, int S, int T, int overwrite_ans_grad) {
+                       R *__restrict__ py_grad, int S, int T, int overwrite_ans_grad,
+                       const R *__restrict__ scores, R *__restrict__ loss, int B, int reduction) {
   extern __shared__ __align__(16) unsigned char dyn_lds[];
   __shared__ Counters cnt;
 
@@ -537,6 +538,7 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
   };
   if (!win.ok) {
     zero_outside(wave, nwaves);
+    if (loss && b == 0 && wave == 0) reduce_scores(scores, loss, B, reduction, lane);
     return;
   }
   if (threadIdx.x < (int)(sizeof(Counters) / sizeof(int)))
@@ -642,6 +644,9 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
       tile_base += g.ntiles;
     }
     zero_outside(wave - nsweep, nwaves - nsweep);
+    // the loss, if asked for: the scores are the forward kernel's, complete before this
+    // kernel started, and this wave has nothing left to do
+    if (loss && b == 0 && wave == nsweep) reduce_scores(scores, loss, B, reduction, lane);
     return;
   }
 
@@ -857,8 +862,11 @@ int forward_impl(const R *px, const R *py, const int64_t *boundary, R *p, R *ans
 template <typename R>
 int backward_impl(const R *px, const R *py, const int64_t *boundary, const R *p, R *ans_grad,
                   R *px_grad, R *py_grad, int B, int S, int T, int modified,
-                  int overwrite_ans_grad, void *stream) {
+                  int overwrite_ans_grad, void *stream, const R *scores = nullptr,
+                  R *loss = nullptr, int reduction = 0) {
   (void)py;  // the d2 = 1 - d1 split needs only p and px
+  if (loss && (!scores || reduction < 0 || reduction > 2))
+    return fail(FRNNT_EINVAL, "mi_backward: loss without scores, or bad reduction");
   if (B < 0 || S < 0 || T < 0) return fail(FRNNT_EINVAL, "mi_backward: negative size");
   if (B == 0) return FRNNT_OK;
   if (!px || !p || !px_grad || !py_grad)
@@ -876,11 +884,25 @@ int backward_impl(const R *px, const R *py, const int64_t *boundary, const R *p,
     return check_launch("mi_backward: hipFuncSetAttribute");
   hipLaunchKernelGGL(kernel, dim3(B), dim3(n * (1 + kBwdStagers) * kWave), lds,
                      static_cast<hipStream_t>(stream), px, boundary, p, ans_grad, px_grad,
-                     py_grad, S, T, overwrite_ans_grad);
+                     py_grad, S, T, overwrite_ans_grad, scores, loss, B, reduction);
   return check_launch("mi_backward");
 }
 
 }  // namespace
+
+int mi_backward_and_loss(const float *px, const int64_t *boundary, const float *p, float *px_grad,
+                         float *py_grad, const float *scores, float *loss, int B, int S, int T,
+                         int modified, int reduction, void *stream) {
+  return backward_impl<float>(px, nullptr, boundary, p, nullptr, px_grad, py_grad, B, S, T,
+                              modified, 0, stream, scores, loss, reduction);
+}
+int mi_backward_and_loss(const double *px, const int64_t *boundary, const double *p,
+                         double *px_grad, double *py_grad, const double *scores, double *loss,
+                         int B, int S, int T, int modified, int reduction, void *stream) {
+  return backward_impl<double>(px, nullptr, boundary, p, nullptr, px_grad, py_grad, B, S, T,
+                               modified, 0, stream, scores, loss, reduction);
+}
+
 }  // namespace frnnt
 
 extern "C" {

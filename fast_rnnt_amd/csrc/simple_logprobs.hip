@@ -264,24 +264,11 @@ __global__ void __launch_bounds__(256)
     if (first + 256 * u < n) base[first + 256 * u] = v[u] * g;
 }
 
-// loss = -scores, -mean(scores) or -sum(scores); one wave: every lane sums a
-// contiguous slice, then a fixed butterfly over the lanes
+// loss = -scores, -mean(scores) or -sum(scores); one wave
 template <typename R>
 __global__ void __launch_bounds__(kWave)
     loss_reduce_kernel(const R *__restrict__ scores, R *__restrict__ loss, int B, int reduction) {
-  const int lane = threadIdx.x;
-  if (reduction == 0) {
-    for (int b = lane; b < B; b += kWave) loss[b] = -scores[b];
-    return;
-  }
-  const int per = (B + kWave - 1) / kWave;
-  R acc = 0;
-  for (int k = 0; k < per; ++k) {
-    const int b = lane * per + k;
-    if (b < B) acc += scores[b];
-  }
-  acc = wave_sum(acc);
-  if (lane == 0) loss[0] = reduction == 1 ? -(acc / (R)B) : -acc;
+  reduce_scores(scores, loss, B, reduction, (int)threadIdx.x);
 }
 
 // lm gradient: grid = (ceil(C/64), ceil((S+1)/64), B); K runs over frames.

@@ -23,6 +23,10 @@ int simple_loss_fwd(Logprobs logprobs, Forward forward, Backward backward, Reduc
   rc = forward(px, py, boundary, p, scores, B, S, T, modified, stream);
   if (rc != FRNNT_OK) return rc;
   if (px_grad) {
+    // with a loss to form, the backward kernel reduces the scores on its way
+    if (loss && B > 0)
+      return mi_backward_and_loss(px, boundary, p, px_grad, py_grad, scores, loss, B, S, T,
+                                  modified, reduction, stream);
     rc = backward(px, py, boundary, p, nullptr, px_grad, py_grad, B, S, T, modified, 0, stream);
     if (rc != FRNNT_OK) return rc;
   }
