@@ -714,17 +714,27 @@ __global__ void __launch_bounds__(kPanThreads)
 // 32-frame slabs -- D[96 rows][32 k], fetched as coalesced 16-byte pieces and
 // transposed through its own LDS region, and exp(am[32 k][32 c] - max) -- into MFMA
 // operands without waiting for any other wave; the partial sums meet once at the end.
-// A workgroup covers 96 lattice rows x 32 vocabulary entries.
-constexpr int kLmS = 96;
+// A workgroup covers kS lattice rows x 32 vocabulary entries and takes the frames in slabs
+// of kK: 96 rows with 32 frames, or 128 rows with 16 (the form that pads S+1 less, as in
+// the normalizer kernel).
 constexpr int kLmC = 32;
-constexpr int kLmK = 32;
 constexpr int kLmWaves = 4;
 constexpr int kLmThreads = kLmWaves * kWave;
-constexpr int kLmPitch = kLmK + 1;
-constexpr int kLmSlab = kLmS * kLmPitch + kLmK * kLmC;  // floats per wave: D slab, then am slab
-constexpr size_t kLmLdsBytes = (size_t)kLmWaves * kLmSlab * sizeof(float);
-constexpr int kLmItems = kLmS * kLmC / 4 / kLmThreads;   // 16-byte outputs per thread
+constexpr int kLmOutPitch = kLmC + 1;  // pitch of a wave's partial sums in LDS
+template <int kS, int kK>
+struct LmShape {
+  static constexpr int kPitch = kK + 1;
+  static constexpr int kSlab = kS * kPitch + kK * kLmC;  // floats per wave: D slab, then am slab
+  static constexpr int kSums = kS * kLmOutPitch;         // floats of a wave's partial sums
+  static constexpr size_t kLdsBytes =
+      (size_t)kLmWaves * (kSlab > kSums ? kSlab : kSums) * sizeof(float);
+  static constexpr int kItems = kS * kLmC / 4 / kLmThreads;  // 16-byte outputs per thread
+  static constexpr int kRowLanes = kK / 4;                   // lanes that share a row of the D slab
+  static constexpr int kRowsPerLoad = kWave / kRowLanes;
+  static_assert(kS % kRowsPerLoad == 0 && kK % 8 == 0 && kS % 32 == 0, "shape");
+};
 
+template <int kS, int kK>
 __global__ void __launch_bounds__(kLmThreads, 2)
     simple_bwd_lm_slab_kernel(const float *__restrict__ lm, const float *__restrict__ am,
                               const int64_t *__restrict__ symbols,
@@ -733,6 +743,9 @@ __global__ void __launch_bounds__(kLmThreads, 2)
                               const float *__restrict__ row_x, const float *__restrict__ row_y,
                               float *__restrict__ lm_grad, int B, int S, int T, int C, int ldd,
                               int term) {
+  using Shape = LmShape<kS, kK>;
+  constexpr int kLmS = kS, kLmK = kK, kLmPitch = Shape::kPitch, kLmSlab = Shape::kSlab;
+  constexpr int kLmItems = Shape::kItems;
   using namespace dgemm;
   extern __shared__ float lm_lds[];
   const int S1 = S + 1;
@@ -750,19 +763,21 @@ __global__ void __launch_bounds__(kLmThreads, 2)
   const int half = lane >> 5, r32 = lane & 31;
   const float ninf = -__builtin_huge_valf();
 
-  // what this lane fetches of every slab: D rows sub + 8 j at k-offset kq; am rows
-  // (frames) sub + 8 j at vocabulary offset kq
-  constexpr int kLoadsA = kLmS / 8, kLoadsB = kLmK / 8;
+  // what this lane fetches of every slab: D rows sub_a + kRowsA j at k-offset kq_a; am
+  // rows (frames) sub + 8 j at vocabulary offset kq
+  constexpr int kRowsA = Shape::kRowsPerLoad;
+  constexpr int kLoadsA = kLmS / kRowsA, kLoadsB = kLmK / 8;
   const int sub = lane >> 3, kq = 4 * (lane & 7);
+  const int sub_a = lane / Shape::kRowLanes, kq_a = 4 * (lane % Shape::kRowLanes);
   floatx4 sa[kLoadsA], sb[kLoadsB];
   float shift2[kLoadsB];  // -(the frame's maximum) * log2(e)
   auto fetch = [&](int k0) {
 #pragma unroll
     for (int j = 0; j < kLoadsA; ++j) {
-      const int sr = s_tile + sub + 8 * j;
+      const int sr = s_tile + sub_a + kRowsA * j;
       // columns at and beyond T must read as 0: the pad of a D row is not defined
-      const int valid = sr < S1 ? min(4, max(T - k0 - kq, 0)) : 0;
-      sa[j] = load4_guarded<true>(db, sr * ldd + k0 + kq, valid);
+      const int valid = sr < S1 ? min(4, max(T - k0 - kq_a, 0)) : 0;
+      sa[j] = load4_guarded<true>(db, sr * ldd + k0 + kq_a, valid);
     }
 #pragma unroll
     for (int j = 0; j < kLoadsB; ++j) {
@@ -809,7 +824,7 @@ __global__ void __launch_bounds__(kLmThreads, 2)
   for (; chunk < chunks; chunk += kLmWaves) {
 #pragma unroll
     for (int j = 0; j < kLoadsA; ++j) {
-      float *d = as + (sub + 8 * j) * kLmPitch + kq;
+      float *d = as + (sub_a + kRowsA * j) * kLmPitch + kq_a;
 #pragma unroll
       for (int i = 0; i < 4; ++i) d[i] = sa[j][i];
     }
@@ -834,14 +849,14 @@ __global__ void __launch_bounds__(kLmThreads, 2)
     }
   }
 
-  // the partial sums meet: [wave][96][33] in the slab space
+  // the partial sums meet: [wave][kS][33] in the slab space
   __syncthreads();
-  float *part = lm_lds + wave * (kLmS * kLmPitch);
+  float *part = lm_lds + wave * Shape::kSums;
 #pragma unroll
   for (int j = 0; j < kLmS / 32; ++j)
 #pragma unroll
     for (int v = 0; v < 16; ++v)
-      part[(32 * j + 8 * (v / 4) + 4 * half + (v % 4)) * kLmPitch + r32] = acc[j][v];
+      part[(32 * j + 8 * (v / 4) + 4 * half + (v % 4)) * kLmOutPitch + r32] = acc[j][v];
   __syncthreads();
 #pragma unroll
   for (int j = 0; j < kLmItems; ++j) {
@@ -856,7 +871,7 @@ __global__ void __launch_bounds__(kLmThreads, 2)
       float sum = 0.f;
 #pragma unroll
       for (int w = 0; w < kLmWaves; ++w)
-        sum += lm_lds[w * (kLmS * kLmPitch) + m * kLmPitch + n + i];
+        sum += lm_lds[w * Shape::kSums + m * kLmOutPitch + n + i];
       g[i] = __expf(lm_in[j][i] - mx) * sum;
       if (c + i == sym) g[i] += rx;
       if (c + i == term) g[i] += ry;
@@ -1095,12 +1110,17 @@ void launch_bwd_lm(const float *lm, const float *am, const int64_t *symbols, con
                    const float *am_max, const float *dmat, const float *row_x, const float *row_y,
                    float *lm_grad, int B, int S, int T, int C, int ldd, int term,
                    hipStream_t stream) {
-  const int tiles = ((C + kLmC - 1) / kLmC) * ((S + 1 + kLmS - 1) / kLmS);
-  auto kernel = simple_bwd_lm_slab_kernel;
-  (void)allow_lds(reinterpret_cast<const void *>(kernel), kLmLdsBytes);
-  hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(tiles, B)), dim3(kLmThreads), kLmLdsBytes,
-                     stream, lm, am, symbols, lm_max, am_max, dmat, row_x, row_y, lm_grad, B, S, T,
-                     C, ldd, term);
+  // the row count per workgroup that leaves fewer padding rows; 128 on a tie
+  const int S1 = S + 1;
+  const bool rows96 = (S1 + 95) / 96 * 96 < (S1 + 127) / 128 * 128;
+  const int rows = rows96 ? 96 : 128;
+  const int tiles = ((C + kLmC - 1) / kLmC) * ((S1 + rows - 1) / rows);
+  auto kernel = rows96 ? simple_bwd_lm_slab_kernel<96, 32> : simple_bwd_lm_slab_kernel<128, 16>;
+  const size_t lds = rows96 ? LmShape<96, 32>::kLdsBytes : LmShape<128, 16>::kLdsBytes;
+  (void)allow_lds(reinterpret_cast<const void *>(kernel), lds);
+  hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(tiles, B)), dim3(kLmThreads), lds, stream, lm,
+                     am, symbols, lm_max, am_max, dmat, row_x, row_y, lm_grad, B, S, T, C, ldd,
+                     term);
 }
 void launch_bwd_lm(const double *lm, const double *am, const int64_t *symbols,
                    const double *lm_max, const double *am_max, const double *dmat,
