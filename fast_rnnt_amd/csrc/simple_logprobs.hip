@@ -888,10 +888,10 @@ __global__ void __launch_bounds__(kLmThreads, 2)
 }
 
 // am gradient, LDS-panel form.  k runs over the S+1 lattice rows, which is short, so
-// a workgroup brings ALL of k for its 64 (frames) x 64 (vocabulary) tile into LDS:
-// D[k][t], gx[k][t] and exp(lm[k][c] - max[k]) are all contiguous along the output
-// dimension, so the panels arrive as coalesced 16-byte loads, and the matrix cores
-// read their operands from LDS only.  What bounds this kernel is the number of
+// a workgroup brings ALL of k (up to 128 rows per pass) for its 64 (frames) x 64
+// (vocabulary) tile into LDS: D[k][t] and exp(lm[k][c] - max[k]) are both contiguous
+// along the output dimension, so the panels arrive as coalesced 16-byte loads, and the
+// matrix cores read the dense product's operands from LDS only.  What bounds this kernel is the number of
 // vector-memory INSTRUCTIONS a compute unit can retire (an instruction costs about
 // the same whether it moves 4 or 16 bytes per lane), so every global access here is
 // 16 bytes wide and row-contiguous: the am tile comes in that way too, and the
@@ -901,15 +901,19 @@ __global__ void __launch_bounds__(kLmThreads, 2)
 // The per-symbol term  sum_s [c = sym[b,s]] gx[b,s,t]  is a second product on the
 // matrix core, gx^T times a one-hot matrix made in registers from the symbols: it is
 // exact (products by 0 or 1) and has a fixed summation order; k-pairs none of whose
-// symbols falls into the wave's 32 vocabulary columns are skipped (wave-uniform).
+// symbols falls into the wave's 32 vocabulary columns are skipped (wave-uniform).  With
+// a large vocabulary almost every pair is skipped, so gx has no panel: a wave reads the
+// few 128-byte row pieces it needs straight from memory, the first eight of them
+// requested before the dense product so that they arrive under it.
 constexpr int kAmT = 64;       // frames per workgroup
 constexpr int kAmC = 64;       // vocabulary entries per workgroup
-constexpr int kAmRows = 96;    // lattice rows per LDS pass (even)
+constexpr int kAmRows = 128;   // lattice rows per LDS pass (even)
+constexpr int kAmHotAhead = 8; // per-symbol pairs whose gx values are requested ahead
 constexpr int kAmOutPitch = 68;  // row pitch of the result tiles staged in LDS
 constexpr int kAmQ = kAmT / 4;   // 16-byte pieces per panel row (kAmT == kAmC)
 
 size_t am_panel_lds_bytes(int rows_cap) {
-  const size_t panels = (size_t)rows_cap * (2 * kAmT + kAmC) * sizeof(float);
+  const size_t panels = (size_t)rows_cap * (kAmT + kAmC) * sizeof(float);
   const size_t staging = (size_t)2 * kAmT * kAmOutPitch * sizeof(float);
   return std::max(panels, staging) + (size_t)(2 * rows_cap + 2 * kAmT) * sizeof(float);
 }
@@ -931,8 +935,7 @@ __global__ void __launch_bounds__(256, 2)
   float *shift_s = lmx_s + rows_cap;              // [kAmT] am_max of the tile's frames
   float *extra_s = shift_s + kAmT;                // [kAmT] col_y of the tile's frames
   float *As = extra_s + kAmT;                     // [rows_cap][kAmT]   D[k][t]
-  float *Gs = As + rows_cap * kAmT;               // [rows_cap][kAmT]   gx[k][t]
-  float *Bs = Gs + rows_cap * kAmT;               // [rows_cap][kAmC]   exp(lm[k][c] - max[k])
+  float *Bs = As + rows_cap * kAmT;               // [rows_cap][kAmC]   exp(lm[k][c] - max[k])
   float *out_acc = As;                            // result tiles, after the last pass
   float *out_hot = As + kAmT * kAmOutPitch;
   const int S1 = S + 1;
@@ -976,13 +979,11 @@ __global__ void __launch_bounds__(256, 2)
     const int rows = min(rows_cap, S1 - k0);
     const int pairs = (rows + 1) / 2;
     constexpr int kSteps = kAmRows / 16;
-    floatx4 ra[kSteps], rg[kSteps], rb[kSteps];
+    floatx4 ra[kSteps], rb[kSteps];
 #pragma unroll
     for (int j = 0; j < kSteps; ++j) {
       const int k = q_row + 16 * j, t = t_tile + q_col, c = c_tile + q_col;
       ra[j] = load4_guarded<kVec>(db, (k0 + k) * ldd + t, (k < rows && t < ldd) ? 4 : 0);
-      rg[j] = load4_guarded<kVec>(gxb, (k0 + k) * T1 + t,
-                                  (k < rows && k0 + k < S) ? min(4, max(T - t, 0)) : 0);
       rb[j] = load4_guarded<kVec>(lmb, (k0 + k) * C + c, k < rows ? min(4, max(C - c, 0)) : 0);
     }
     if (k0 > 0) __syncthreads();  // the previous pass's readers are done with the panels
@@ -994,13 +995,34 @@ __global__ void __launch_bounds__(256, 2)
     for (int j = 0; j < kSteps; ++j) {
       const int k = q_row + 16 * j;
       if (k >= 2 * pairs) continue;
-      floatx4 gz = rg[j];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) gz[i] = (t_tile + q_col + i == t_mask) ? 0.f : gz[i];
       *reinterpret_cast<floatx4 *>(As + k * kAmT + q_col) = ra[j];
-      *reinterpret_cast<floatx4 *>(Gs + k * kAmT + q_col) = gz;
     }
-    __syncthreads();  // lmx_s is visible
+    __syncthreads();  // lmx_s and sym_s are visible
+    // per-symbol product: the pairs with a symbol among this wave's columns ...
+    bool in = false;
+    if (lane < pairs)
+      in = (unsigned)(sym_s[2 * lane] - c_lo) < 32u || (unsigned)(sym_s[2 * lane + 1] - c_lo) < 32u;
+    unsigned long long wanted = __ballot(in);
+    // ... and this lane's gx[k][t] of pair i (k = 2 i + half, t = the wave's frame r32):
+    // nothing for the masked frame, past T or past the last symbol
+    const int hot_t = t_tile + wt + r32;
+    const bool hot_ok = hot_t < T && hot_t != t_mask;
+    auto hot_value = [&](int i) {
+      const int k = k0 + 2 * i + half;
+      return (hot_ok && k < S) ? gxb[(long)k * T1 + hot_t] : 0.f;
+    };
+    int ahead[kAmHotAhead];
+    float ahead_v[kAmHotAhead];
+#pragma unroll
+    for (int u = 0; u < kAmHotAhead; ++u) {
+      ahead[u] = -1;
+      ahead_v[u] = 0.f;
+      if (wanted) {
+        ahead[u] = __builtin_ctzll(wanted);
+        wanted &= wanted - 1;
+        ahead_v[u] = hot_value(ahead[u]);
+      }
+    }
 #pragma unroll
     for (int j = 0; j < kSteps; ++j) {
       const int k = q_row + 16 * j, c = c_tile + q_col;
@@ -1018,17 +1040,18 @@ __global__ void __launch_bounds__(256, 2)
 #pragma unroll 4
     for (int i = 0; i < pairs; ++i)
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[2 * i * kAmT], bp[2 * i * kAmC], acc, 0, 0, 0);
-    // per-symbol product, only for pairs with a symbol among this wave's columns
-    bool in = false;
-    if (lane < pairs)
-      in = (unsigned)(sym_s[2 * lane] - c_lo) < 32u || (unsigned)(sym_s[2 * lane + 1] - c_lo) < 32u;
-    unsigned long long wanted = __ballot(in);
-    const float *gp = Gs + half * kAmT + wt + r32;
+    // per-symbol product
+#pragma unroll
+    for (int u = 0; u < kAmHotAhead; ++u) {
+      if (ahead[u] < 0) continue;
+      const float h = (sym_s[2 * ahead[u] + half] == c_lo + r32) ? 1.f : 0.f;
+      hot = __builtin_amdgcn_mfma_f32_32x32x2f32(ahead_v[u], h, hot, 0, 0, 0);
+    }
     while (wanted) {
       const int i = __builtin_ctzll(wanted);
       wanted &= wanted - 1;
       const float h = (sym_s[2 * i + half] == c_lo + r32) ? 1.f : 0.f;
-      hot = __builtin_amdgcn_mfma_f32_32x32x2f32(gp[2 * i * kAmT], h, hot, 0, 0, 0);
+      hot = __builtin_amdgcn_mfma_f32_32x32x2f32(hot_value(i), h, hot, 0, 0, 0);
     }
   }
   // results through LDS, so that they leave as whole row segments
