@@ -27,7 +27,7 @@ FP32_MFMA_PEAK_TFLOPS = 157.3
 # profiles/ (FETCH_SIZE and WRITE_SIZE, scaled by what the same counters read for a
 # copy of known size); filled in for the workloads that were profiled
 MEASURED_TRAFFIC = {
-    ("c2", "simple_fwd_panel_kernel<true, 96, 16>"): 29397292,
+    ("c2", "simple_fwd_panel_kernel<96, 16>"): 29397292,
     ("c2", "mi_forward_kernel<float, false, 2>"): 6877163,
     ("c2", "mi_backward_kernel<float, false, 2>"): 9790490,
 }
@@ -314,8 +314,8 @@ def main():
     # normalizer contraction exp(lm - max) . exp(am - max)^T on the fp32 matrix cores;
     # the same kernel finds the row maxima on the way and assembles px/py at the end,
     # so this figure is a lower bound on the rate of its MFMA loop
-    gemm_name = "simple_fwd_panel_kernel<true, 96, 16>" if (S + 1 + 95) // 96 * 96 < (S + 1 + 127) // 128 * 128 \
-        else "simple_fwd_panel_kernel<true, 128, 16>"
+    gemm_name = "simple_fwd_panel_kernel<96, 16>" if (S + 1 + 95) // 96 * 96 < (S + 1 + 127) // 128 * 128 \
+        else "simple_fwd_panel_kernel<128, 16>"
     gemm_flops = 2.0 * B * (S + 1) * T * w.C
     gemm_tflops = gemm_flops / (t_logp * 1e-3) / 1e12
     lines = [

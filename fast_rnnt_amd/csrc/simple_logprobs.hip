@@ -413,7 +413,7 @@ struct PanelShape {
   static_assert(kRows % kRowsPerLoad == 0 && kLoads % 2 == 0 && kS % 32 == 0 && kS <= 128, "shape");
 };
 
-template <bool kVec, int kS, int kK>
+template <int kS, int kK>
 __global__ void __launch_bounds__(kPanThreads)
     simple_fwd_panel_kernel(const float *__restrict__ lm, const float *__restrict__ am,
                             const int64_t *__restrict__ symbols,
@@ -471,29 +471,39 @@ __global__ void __launch_bounds__(kPanThreads)
   constexpr int kLoads = Shape::kLoads;
   const int sub = lane / kRowLanes, kq = 4 * (lane % kRowLanes);
   // row j of a fetch is lattice row s_tile + sub + kRowsPerLoad j while that stays below
-  // kS, a frame after that; what lies outside the operands reads as -inf, neutral for
-  // the maximum, and exp(-inf - shift) = 0 in the product
+  // kS, a frame after that.  The loads go through buffer resources that cover lm[b] and
+  // am[b]: one instruction each, no branch, any alignment; a row past the last one lies
+  // past the resource and reads as 0 -- such rows only feed outputs that are never
+  // written.  Columns at and past C (the last slab) belong to the next row and are
+  // replaced by -inf, exp(-inf - shift) = 0 in the product.
   constexpr int kLmLoads = kPanS / kRowsPerLoad;
   static_assert(kPanS % kRowsPerLoad == 0, "a fetch row holds lm or am, not both");
-  const int lm_off = (s_tile + sub) * C + kq, am_off = (t_tile + sub) * C + kq;
-  const int lm_rows = S1 - s_tile - sub, am_rows = T - t_tile - sub;  // rows left from this lane's first
-  const int step = kRowsPerLoad * C;
+  const __amdgpu_buffer_rsrc_t lm_rs =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(lmb), 0, S1 * C * 4, 0x00020000);
+  const __amdgpu_buffer_rsrc_t am_rs =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(amb), 0, T * C * 4, 0x00020000);
+  const int lm_off = ((s_tile + sub) * C + kq) * 4, am_off = ((t_tile + sub) * C + kq) * 4;  // bytes
+  const int step = kRowsPerLoad * C * 4;
+  typedef int intx4 __attribute__((ext_vector_type(4)));
   auto fetch = [&](floatx4 (&into)[kLoads], int k0) {
-    const int width = min(4, max(C - k0 - kq, 0));
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
-      if (j < kLmLoads)
-        into[j] = load4_guarded<kVec>(lmb, lm_off + j * step + k0,
-                                      kRowsPerLoad * j < lm_rows ? width : 0, ninf);
-      else
-        into[j] = load4_guarded<kVec>(amb, am_off + (j - kLmLoads) * step + k0,
-                                      kRowsPerLoad * (j - kLmLoads) < am_rows ? width : 0, ninf);
+      const intx4 raw = j < kLmLoads
+                            ? __builtin_amdgcn_raw_buffer_load_b128(lm_rs, lm_off + (j * step + k0 * 4), 0, 0)
+                            : __builtin_amdgcn_raw_buffer_load_b128(
+                                  am_rs, am_off + ((j - kLmLoads) * step + k0 * 4), 0, 0);
+      into[j] = floatx4{__int_as_float(raw[0]), __int_as_float(raw[1]), __int_as_float(raw[2]),
+                        __int_as_float(raw[3])};
+    }
+    if (k0 + kPanK > C) {  // (wave-uniform) the slab that holds column C - 1
+#pragma unroll
+      for (int j = 0; j < kLoads; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (k0 + kq + i >= C) into[j][i] = ninf;
     }
   };
   const int chunks = (C + kPanK - 1) / kPanK;
-  // a wave takes the slabs in pairs (2 p, 2 p + 1), p = wave, wave + 8, ..: the two
-  // slabs of a pair are requested back to back and share their cache lines at k = 16
-  const int pairs = (chunks + 1) / 2;
 
   // ---- one pass over k.  The reference subtracts the row maxima before exp
   // (rnnt_loss.py:174-178); a maximum is known only after the whole row has been seen, so
@@ -504,14 +514,11 @@ __global__ void __launch_bounds__(kPanThreads)
   // per product.  The running maxima are kept beside the shifts, and when the waves
   // meet their partial sums are brought to the true maxima, exp(shift - max) <= 1.
   constexpr float kMargin = 30.f;
-  floatx4 slab0[kLoads], slab1[kLoads];
-  if (wave < pairs) {
-    fetch(slab0, 2 * wave * kPanK);
-    fetch(slab1, (2 * wave + 1) * kPanK);
-  }
+  floatx4 slab[kLoads];
+  if (wave < chunks) fetch(slab, wave * kPanK);
 
-  // ---- epilogue inputs, requested behind the first slabs (the symbols they depend on
-  // were requested before those) so that their latency hides under the loop:
+  // ---- epilogue inputs, requested behind the first slab (the symbols they depend on
+  // were requested before it) so that their latency hides under the loop:
   // am[b, t, sym[b, s]] for this thread's outputs ...
   float am_sym[kPanItems][4];
 #pragma unroll
@@ -580,9 +587,9 @@ __global__ void __launch_bounds__(kPanThreads)
     bool above = false;
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
-      const float top = fmaxf(fmaxf(slab[j][0], slab[j][1]), fmaxf(slab[j][2], slab[j][3]));
-      seen[j] = fmaxf(seen[j], top);
-      above |= __builtin_fmaf(top, kLog2e, shift2[j]) > kMargin * kLog2e;
+      // two three-input maxima; a row is above its margin exactly when its maximum is
+      seen[j] = fmaxf(fmaxf(fmaxf(slab[j][0], slab[j][1]), slab[j][2]), fmaxf(slab[j][3], seen[j]));
+      above |= __builtin_fmaf(seen[j], kLog2e, shift2[j]) > kMargin * kLog2e;
     }
     if (__any(above)) raise_shifts();
 #pragma unroll
@@ -604,10 +611,7 @@ __global__ void __launch_bounds__(kPanThreads)
                                                         0, 0, 0);
     }
   };
-  for (int pair = wave; pair < pairs; pair += kPanWaves) {
-    consume(slab0, 2 * (pair + kPanWaves));
-    if (2 * pair + 1 < chunks) consume(slab1, 2 * (pair + kPanWaves) + 1);
-  }
+  for (int chunk = wave; chunk < chunks; chunk += kPanWaves) consume(slab, chunk + kPanWaves);
 
   // ---- the waves meet: maxima first ...
 #pragma unroll
@@ -761,7 +765,6 @@ __global__ void __launch_bounds__(kLmThreads, 2)
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int half = lane >> 5, r32 = lane & 31;
-  const float ninf = -__builtin_huge_valf();
 
   // what this lane fetches of every slab: D rows sub_a + kRowsA j at k-offset kq_a; am
   // rows (frames) sub + 8 j at vocabulary offset kq
@@ -771,19 +774,39 @@ __global__ void __launch_bounds__(kLmThreads, 2)
   const int sub_a = lane / Shape::kRowLanes, kq_a = 4 * (lane % Shape::kRowLanes);
   floatx4 sa[kLoadsA], sb[kLoadsB];
   float shift2[kLoadsB];  // -(the frame's maximum) * log2(e)
+  // The loads go through buffer resources that cover D[b] and am[b]: one instruction
+  // each, no branch; a row past the last one lies past the resource and reads as 0.
+  // Frames at and past T (the last slab) must give products of 0: there D is replaced
+  // by 0 (the pad of a D row is not defined; am reads as 0 or holds the next utterance's
+  // frames, exp of which is finite).  Vocabulary columns at and past C belong to the next
+  // row: they only feed output columns that are never written.
+  typedef int intx4 __attribute__((ext_vector_type(4)));
+  const __amdgpu_buffer_rsrc_t d_rs =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(db), 0, S1 * ldd * 4, 0x00020000);
+  const __amdgpu_buffer_rsrc_t am_rs =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(amb), 0, T * C * 4, 0x00020000);
+  const int d_off = ((s_tile + sub_a) * ldd + kq_a) * 4, am_off = (sub * C + c_tile + kq) * 4;  // bytes
+  auto as_floats = [](intx4 raw) {
+    return floatx4{__int_as_float(raw[0]), __int_as_float(raw[1]), __int_as_float(raw[2]),
+                   __int_as_float(raw[3])};
+  };
   auto fetch = [&](int k0) {
 #pragma unroll
-    for (int j = 0; j < kLoadsA; ++j) {
-      const int sr = s_tile + sub_a + kRowsA * j;
-      // columns at and beyond T must read as 0: the pad of a D row is not defined
-      const int valid = sr < S1 ? min(4, max(T - k0 - kq_a, 0)) : 0;
-      sa[j] = load4_guarded<true>(db, sr * ldd + k0 + kq_a, valid);
+    for (int j = 0; j < kLoadsA; ++j)
+      sa[j] = as_floats(__builtin_amdgcn_raw_buffer_load_b128(
+          d_rs, d_off + (kRowsA * j * ldd + k0) * 4, 0, 0));
+    if (k0 + kLmK > T) {  // (wave-uniform) the slab that holds frame T - 1
+#pragma unroll
+      for (int j = 0; j < kLoadsA; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (k0 + kq_a + i >= T) sa[j][i] = 0.f;
     }
 #pragma unroll
     for (int j = 0; j < kLoadsB; ++j) {
-      const int tr = k0 + sub + 8 * j, c = c_tile + kq;
-      const int valid = tr < T ? min(4, max(C - c, 0)) : 0;
-      sb[j] = load4_guarded<true>(amb, tr * C + c, valid, ninf);
+      const int tr = k0 + sub + 8 * j;
+      sb[j] = as_floats(__builtin_amdgcn_raw_buffer_load_b128(
+          am_rs, am_off + (k0 + 8 * j) * C * 4, 0, 0));
       shift2[j] = tr < T ? -amx[tr] * kLog2e : 0.f;
     }
   };
@@ -1098,8 +1121,7 @@ void launch_fwd_panel(const float *lm, const float *am, const int64_t *symbols,
   using Shape = PanelShape<kS, kK>;
   const int t_tiles = T > 0 ? (T + kPanT - 1) / kPanT : 1;
   const int s_tiles = (S + 1 + kS - 1) / kS;
-  const bool vec = (C % 4 == 0) && aligned16(lm) && aligned16(am);
-  auto kernel = vec ? simple_fwd_panel_kernel<true, kS, kK> : simple_fwd_panel_kernel<false, kS, kK>;
+  auto kernel = simple_fwd_panel_kernel<kS, kK>;
   (void)allow_lds(reinterpret_cast<const void *>(kernel), Shape::kLdsBytes);
   hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(t_tiles * s_tiles, B)), dim3(kPanThreads),
                      Shape::kLdsBytes, stream, lm, am, symbols, boundary, lm_max, am_max, px, py,
@@ -1196,6 +1218,10 @@ int fwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
   if (B == 0) return FRNNT_OK;
   if (!lm || !am || (!symbols && S > 0) || !px || !py || !lm_max || !am_max)
     return fail(FRNNT_EINVAL, "simple_logprobs_fwd: null pointer");
+  // (the float32 kernel addresses an utterance's lm / am rows by 32-bit byte offsets)
+  if (std::is_same<R, float>::value &&
+      ((long)(S + 1) * C * 4 >= (1L << 31) || (long)T * C * 4 >= (1L << 31)))
+    return fail(FRNNT_ELIMIT, "simple_logprobs_fwd: one utterance's lm or am exceeds 2 GiB");
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   const long n_lm = (long)B * (S + 1), n_am = (long)B * T;
   const long rows = n_lm + n_am;
@@ -1229,6 +1255,11 @@ int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
   if (!lm || !am || (!symbols && S > 0) || !lm_max || !am_max || !norm_raw || !px_grad ||
       !py_grad || !dmat || !row_x || !row_y || !col_y)
     return fail(FRNNT_EINVAL, "simple_logprobs_bwd: null pointer");
+  // (the float32 kernels address an utterance's lm / am / D rows by 32-bit byte offsets)
+  if (std::is_same<R, float>::value &&
+      ((long)(S + 1) * C * 4 >= (1L << 31) || (long)T * C * 4 >= (1L << 31) ||
+       (long)(S + 1) * (T + 3) * 4 >= (1L << 31)))
+    return fail(FRNNT_ELIMIT, "simple_logprobs_bwd: one utterance's lm, am or lattice exceeds 2 GiB");
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   if (score_grad) {
     if (score_grad_stride != 0 && score_grad_stride != 1)

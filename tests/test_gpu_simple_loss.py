@@ -201,8 +201,12 @@ def test_baseline_configs(gpu_device, name):
                                    return_grad=True)
     wx0, wy0 = wx.clone(), wy.clone()
     want.backward()
-    _, (tx, ty) = O.loss_simple(w.lm.double(), w.am.double(), w.symbols, 0, boundary=w.boundary,
-                                reduction="sum", return_grad=True)
+    ta = w.am.double().requires_grad_(True)
+    tl = w.lm.double().requires_grad_(True)
+    truth, (tx, ty) = O.loss_simple(tl, ta, w.symbols, 0, boundary=w.boundary, reduction="sum",
+                                    return_grad=True)
+    tx, ty = tx.clone(), ty.clone()
+    truth.backward()
     da = w.am.to(dev).requires_grad_(True)
     dl = w.lm.to(dev).requires_grad_(True)
     got, (gx, gy) = fast_rnnt_amd.rnnt_loss_simple(
@@ -224,4 +228,15 @@ def test_baseline_configs(gpu_device, name):
     bound = _GRAD_BOUND[name]
     assert _close(gx0, wx0, bound) and _close(gy0, wy0, bound)
     assert gpu_off <= 1.5 * cpu_off + 2e-5
-    assert _close(da.grad, a.grad, bound, 1e-4) and _close(dl.grad, l.grad, bound, 1e-4)
+    # am.grad / lm.grad are sums of those over the lattice rows / frames: the same bound
+    # (+ 1e-4 relative) where 1e-4 holds per cell; at the large-vocabulary workload, where a
+    # row of lm.grad adds 400 cells that each may be off by an ulp of p, the float64
+    # oracle is the judge again
+    gpu_in = max((da.grad.cpu().double() - ta.grad).abs().max().item(),
+                 (dl.grad.cpu().double() - tl.grad).abs().max().item())
+    cpu_in = max((a.grad.double() - ta.grad).abs().max().item(),
+                 (l.grad.double() - tl.grad).abs().max().item())
+    _say(f"  am/lm.grad against float64: gpu {gpu_in:.2e}, cpu float32 {cpu_in:.2e}")
+    assert gpu_in <= 1.5 * cpu_in + 1e-4
+    if bound <= 1e-4:
+        assert _close(da.grad, a.grad, bound, 1e-4) and _close(dl.grad, l.grad, bound, 1e-4)
