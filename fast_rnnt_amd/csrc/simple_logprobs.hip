@@ -988,12 +988,26 @@ __global__ void __launch_bounds__(256, 2)
     shift_s[tid] = t < T ? am_max[(long)b * T + t] : 0.f;
     extra_s[tid] = t < T ? col_y[(long)b * T + t] : 0.f;
   }
+  // The panel and tile loads go through buffer resources that cover D[b], lm[b] and
+  // am[b]: one instruction each, no branch, any alignment.  A row past the last one lies
+  // past the resource and reads as 0; a column past the end of a row belongs to the next
+  // row, and only feeds frames >= T or vocabulary entries >= C, which are never written.
+  typedef int intx4 __attribute__((ext_vector_type(4)));
+  const __amdgpu_buffer_rsrc_t d_rs =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(db), 0, S1 * ldd * 4, 0x00020000);
+  const __amdgpu_buffer_rsrc_t lm_rs =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(lmb), 0, S1 * C * 4, 0x00020000);
+  const __amdgpu_buffer_rsrc_t am_rs =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(amb), 0, T * C * 4, 0x00020000);
+  auto get4 = [](__amdgpu_buffer_rsrc_t rs, int byte_offset) {
+    const intx4 raw = __builtin_amdgcn_raw_buffer_load_b128(rs, byte_offset, 0, 0);
+    return floatx4{__int_as_float(raw[0]), __int_as_float(raw[1]), __int_as_float(raw[2]),
+                   __int_as_float(raw[3])};
+  };
   floatx4 am_in[kAmT / 16];
 #pragma unroll
-  for (int j = 0; j < kAmT / 16; ++j) {
-    const int t = t_tile + q_row + 16 * j, c = c_tile + q_col;
-    am_in[j] = load4_guarded<kVec>(amb, t * C + c, t < T ? min(4, max(C - c, 0)) : 0);
-  }
+  for (int j = 0; j < kAmT / 16; ++j)
+    am_in[j] = get4(am_rs, ((t_tile + q_row + 16 * j) * C + c_tile + q_col) * 4);
 
   floatx16 acc, hot;
 #pragma unroll
@@ -1005,9 +1019,9 @@ __global__ void __launch_bounds__(256, 2)
     floatx4 ra[kSteps], rb[kSteps];
 #pragma unroll
     for (int j = 0; j < kSteps; ++j) {
-      const int k = q_row + 16 * j, t = t_tile + q_col, c = c_tile + q_col;
-      ra[j] = load4_guarded<kVec>(db, (k0 + k) * ldd + t, (k < rows && t < ldd) ? 4 : 0);
-      rb[j] = load4_guarded<kVec>(lmb, (k0 + k) * C + c, k < rows ? min(4, max(C - c, 0)) : 0);
+      const int k = k0 + q_row + 16 * j;
+      ra[j] = get4(d_rs, (k * ldd + t_tile + q_col) * 4);
+      rb[j] = get4(lm_rs, (k * C + c_tile + q_col) * 4);
     }
     if (k0 > 0) __syncthreads();  // the previous pass's readers are done with the panels
     for (int k = tid; k < 2 * pairs; k += 256) {
