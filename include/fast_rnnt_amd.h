@@ -32,6 +32,14 @@ extern "C" {
 #define FRNNT_EINVAL (-1)  /* bad argument (null pointer, negative size, ...) */
 #define FRNNT_ELAUNCH (-2) /* the HIP runtime refused the launch             */
 #define FRNNT_ELIMIT (-3)  /* a size exceeds what the kernels support        */
+/*
+ * Size limits (FRNNT_ELIMIT): the kernels address one utterance's arrays with 32-bit
+ * byte offsets -- the lattice (S+1) x (T+1) of the recursion must stay below 1 GiB per
+ * utterance, and for the float32 simple / smoothed loss an utterance's lm ((S+1) x C), am
+ * (T x C) and lattice below 2 GiB each; the recursion holds one row of T+1 scores per
+ * sweep wave in LDS (T up to a few ten thousand frames); get_rnnt_prune_ranges holds T
+ * window starts in LDS (T <= 38400).  The batch size has no limit of its own.
+ */
 
 /* Library version, major*100 + minor. */
 int frnnt_version(void);

@@ -35,6 +35,20 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.frnnt_mi_forward_f32(None, None, None, None, None, 0, 3, 4, 0, None) == 0
 
 
+def test_size_limits_are_reported_without_a_gpu():
+    # the float32 simple-loss kernels address an utterance's lm / am rows with 32-bit byte
+    # offsets; sizes beyond that are refused on the host, before any pointer is followed
+    lib = _lib.load()
+    dummy = ctypes.c_void_p(0x1000)
+    B, S, T, C = 1, 10, 70000, 8000          # T * C * 4 bytes >= 2 GiB
+    rc = lib.frnnt_simple_logprobs_fwd_f32(dummy, dummy, dummy, None, dummy, dummy, dummy, dummy,
+                                           None, B, S, T, C, 0, 0, None)
+    assert rc == -3 and b"2 GiB" in lib.frnnt_last_error()
+    B, S, T = 1, 20000, 20000                # (S+1) * (T+1) * 4 bytes >= 1 GiB
+    rc = lib.frnnt_mi_forward_f32(dummy, dummy, None, dummy, dummy, B, S, T, 0, None)
+    assert rc == -3 and b"1 GiB" in lib.frnnt_last_error()
+
+
 def test_cpu_tensors_are_refused():
     import torch
     from fast_rnnt_amd import _fast_rnnt
