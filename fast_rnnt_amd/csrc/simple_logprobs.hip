@@ -356,11 +356,10 @@ __global__ void __launch_bounds__(256)
 // four consecutive floats at any element-aligned address (global memory takes
 // unaligned 16-byte accesses); `valid` (0..4) leading elements are read, the rest is 0
 typedef float floatx4u __attribute__((ext_vector_type(4), aligned(4)));
-template <bool kVec>
 __device__ __forceinline__ dgemm::floatx4 load4_guarded(const float *base, int off, int valid,
                                                         float fill = 0.f) {
   dgemm::floatx4 r = {fill, fill, fill, fill};
-  if (kVec && valid >= 4) {
+  if (valid >= 4) {
     const floatx4u t = *reinterpret_cast<const floatx4u *>(base + off);
     r[0] = t[0], r[1] = t[1], r[2] = t[2], r[3] = t[3];
   } else {
@@ -821,7 +820,7 @@ __global__ void __launch_bounds__(kLmThreads, 2)
   for (int j = 0; j < kLmItems; ++j) {
     const int item = tid + kLmThreads * j;
     const int sr = s_tile + item / 8, c = c_tile + 4 * (item % 8);
-    lm_in[j] = load4_guarded<true>(lmb, sr * C + c, sr < S1 ? min(4, max(C - c, 0)) : 0);
+    lm_in[j] = load4_guarded(lmb, sr * C + c, sr < S1 ? min(4, max(C - c, 0)) : 0);
   }
   // ... and its rows' maximum, symbol and row sums
   float row_mx[kLmItems], row_rx[kLmItems], row_ry[kLmItems];
@@ -941,7 +940,6 @@ size_t am_panel_lds_bytes(int rows_cap) {
   return std::max(panels, staging) + (size_t)(2 * rows_cap + 2 * kAmT) * sizeof(float);
 }
 
-template <bool kVec>
 __global__ void __launch_bounds__(256, 2)
     simple_bwd_am_panel_kernel(const float *__restrict__ lm, const float *__restrict__ am,
                                const int64_t *__restrict__ symbols,
@@ -1114,7 +1112,7 @@ __global__ void __launch_bounds__(256, 2)
       if (c + i == term) res[i] += extra;
     }
     float *dst = am_grad + ((long)b * T + t) * C + c;
-    if (kVec && c + 4 <= C) {
+    if (c + 4 <= C) {
       *reinterpret_cast<floatx4u *>(dst) = floatx4u{res[0], res[1], res[2], res[3]};
     } else {
 #pragma unroll
@@ -1125,7 +1123,6 @@ __global__ void __launch_bounds__(256, 2)
 }
 
 // launchers: float goes to the slab / panel kernels, double to the LDS-tiled ones
-inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 template <int kS, int kK>
 void launch_fwd_panel(const float *lm, const float *am, const int64_t *symbols,
@@ -1198,7 +1195,7 @@ void launch_bwd_am(const float *lm, const float *am, const int64_t *symbols,
   const int rows_cap = std::min(kAmRows, (S + 2) & ~1);
   const size_t lds = am_panel_lds_bytes(rows_cap);
   // (the 16-byte accesses need no alignment)
-  auto kernel = simple_bwd_am_panel_kernel<true>;
+  auto kernel = simple_bwd_am_panel_kernel;
   (void)allow_lds(reinterpret_cast<const void *>(kernel), lds);
   hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(tiles, B)), dim3(256), lds, stream, lm, am,
                      symbols, boundary, lm_max, am_max, dmat, gpx, col_y, am_grad, B, S, T, C, ldd,
