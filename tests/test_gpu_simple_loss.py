@@ -240,3 +240,56 @@ def test_baseline_configs(gpu_device, name):
     assert gpu_in <= 1.5 * cpu_in + 1e-4
     if bound <= 1e-4:
         assert _close(da.grad, a.grad, bound, 1e-4) and _close(dl.grad, l.grad, bound, 1e-4)
+
+
+def test_graph_replay_matches_eager(gpu_device):
+    """rnnt_loss_simple + backward captured once in a HIP graph and replayed on new input
+    values (copied into the captured tensors), with eager steps and synchronisations between
+    the replays: every replay must give the eager step's loss and gradients bit for bit."""
+    dev = gpu_device
+    B, S, T, C = 3, 20, 40, 30
+    g = torch.Generator().manual_seed(11)
+    sym = torch.randint(1, C, (B, S), generator=g).to(dev)
+    z = torch.zeros(B, dtype=torch.int64)
+    bnd = torch.stack([z, z, torch.tensor([20, 12, 17]), torch.tensor([40, 33, 25])], 1).to(dev)
+    am = torch.randn(B, T, C, generator=g).to(dev).requires_grad_(True)
+    lm = torch.randn(B, S + 1, C, generator=g).to(dev).requires_grad_(True)
+
+    def step(a, l):
+        a.grad = None
+        l.grad = None
+        loss, (gx, gy) = fast_rnnt_amd.rnnt_loss_simple(l, a, sym, 0, boundary=bnd,
+                                                        reduction="sum", return_grad=True)
+        loss.backward()
+        return loss, gx, gy
+
+    quiet = getattr(torch.autograd.graph, "set_warn_on_accumulate_grad_stream_mismatch", None)
+    if quiet is not None:
+        quiet(False)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step(am, lm)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        loss, gx, gy = step(am, lm)
+    g_am, g_lm = am.grad, lm.grad
+    for n in range(4):
+        new_am = torch.randn(B, T, C, generator=g).to(dev)
+        new_lm = torch.randn(B, S + 1, C, generator=g).to(dev)
+        with torch.no_grad():
+            am.copy_(new_am)
+            lm.copy_(new_lm)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in (loss, gx, gy, g_am, g_lm)]
+        ea = new_am.clone().requires_grad_(True)
+        el = new_lm.clone().requires_grad_(True)
+        want_loss, wx, wy = step(ea, el)   # eager work between the replays
+        torch.cuda.synchronize()
+        _say(f"  replay {n}: loss {got[0].item():.6f} eager {want_loss.item():.6f}")
+        for a, b in zip(got, (want_loss, wx, wy, ea.grad, el.grad)):
+            assert torch.equal(a, b)
