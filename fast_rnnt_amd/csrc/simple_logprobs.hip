@@ -382,17 +382,20 @@ __device__ __forceinline__ float exp_shifted(float x, float shift2) {
 // Normalizer GEMM, wave-private LDS transposition.  Both operands are k-contiguous
 // ([rows][C]), the matrix cores want one row per lane.  Letting every lane fetch its
 // own row costs one cache-line lookup per lane and instruction, which is what bounds
-// that form; here a wave fetches a 128-row x 32-k slab with 16 coalesced 16-byte loads
-// (8 lanes per row), applies exp(x - max) in registers, writes the slab to its OWN
-// LDS region (pitch 33, conflict-free for the row-per-lane reads that follow) and
-// feeds the matrix cores from there.  The eight waves of a workgroup split k; they
+// that form; here a wave fetches a slab of (kS lattice rows + 32 frames) x kK k with
+// coalesced 16-byte loads (kK / 4 lanes per row), applies exp(x - shift) in registers,
+// writes the slab to its OWN LDS region (pitch kK + 1, conflict-free for the row-per-lane
+// reads that follow) and feeds the matrix cores from there; the next slab is requested
+// between the LDS writes and the MFMAs.  The eight waves of a workgroup split k; they
 // never wait for each other in the loop (a wave's LDS writes and reads are served in
-// program order), only once at the end, when the partial sums meet.  Two waves share
-// a SIMD, so one wave's exp / LDS-write phase runs under the other's MFMA phase.
-// A workgroup covers kS lattice rows (32-row tiles) x 32 frames and takes k in slabs
-// of kK: 96 rows with k = 32, or 128 rows with k = 16 (the LDS holds eight slabs either
-// way).  The host picks the form that pads S+1 least, so that at S+1 <= 128 the lm
-// operand is fetched once per 32 frames and the am operand once.
+// program order), only once at the end, when the partial sums meet.
+// On this part fp32 MFMA and the VALU work of another wave of the same SIMD do not
+// overlap, so the loop's time is the sum of its MFMA cycles and of everything else it
+// issues: it is written for instruction count (one load instruction and one add per 16
+// bytes, no guards; two 3-input maxima, one fma and one compare per row for the shifts).
+// A workgroup covers kS lattice rows (32-row tiles) x 32 frames: 96 or 128 rows, k in
+// slabs of 16.  The host picks the form that pads S+1 least, so that at S+1 <= 128 the
+// lm operand is fetched once per 32 frames and the am operand once.
 constexpr int kPanT = 32;                 // frames per workgroup
 constexpr int kPanOutPitch = kPanT + 1;   // pitch of a wave's partial sums in LDS
 constexpr int kPanWaves = 8;
