@@ -29,9 +29,9 @@ FP32_MFMA_PEAK_TFLOPS = 157.3
 # profiles/ (FETCH_SIZE and WRITE_SIZE, scaled by what the same counters read for a
 # copy of known size); filled in for the workloads that were profiled
 MEASURED_TRAFFIC = {
-    ("c2", "simple_fwd_panel_kernel<96, 16>"): 29256781,
-    ("c2", "mi_forward_kernel<float, false, 2>"): 6867904,
-    ("c2", "mi_backward_kernel<float, false, 2>"): 9810100,
+    ("c2", "simple_fwd_panel_kernel<96, 16>"): 29257616,
+    ("c2", "mi_forward_kernel<float, false, 2>"): 6868061,
+    ("c2", "mi_backward_kernel<float, false, 2>"): 9809965,
 }
 
 
