@@ -43,6 +43,7 @@ constexpr int kSeamPad = kChunk;        // slack on either side of a seam row, s
                                        // chunk of seam values is written without bounds tests
 constexpr int kFwdStagers = 2;         // staging waves per sweep wave
 constexpr int kBwdStagers = 3;
+constexpr int kBwdStagersFew = 7;  // with at most two sweep waves: 16 waves, the largest workgroup
 constexpr int kSpinLimit = 1 << 22;
 
 struct Window {
@@ -85,6 +86,16 @@ __device__ __forceinline__ int peek(const int *counter) {
 }
 __device__ __forceinline__ void publish(int *counter, int value) {
   __hip_atomic_store(counter, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+// The same for a counter that only tells of LDS writes by this very wave: LDS carries
+// out one wave's instructions in the order they were issued, so the counter's write
+// lands after the data without the wave waiting for its writes to finish (a release
+// makes it wait, ~190 cycles every time).  The empty asm keeps the compiler from
+// moving the data's writes below the counter's.
+__device__ __forceinline__ void publish_lds_writes(int *counter, int value) {
+  asm volatile("" ::: "memory");
+  __hip_atomic_store(counter, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  asm volatile("" ::: "memory");
 }
 
 // log(exp(a) + exp(c)) on the serial chain: same operation order as log_add(),
@@ -165,10 +176,26 @@ __device__ __forceinline__ void pull_row(R (&dst)[kTileSteps], const R *src) {
   }
 }
 
+// kChunk values of one lane into its tile row, 16 bytes per LDS write.
+template <typename R>
+__device__ __forceinline__ void push_chunk(R *dst, const R (&src)[kChunk]) {
+  constexpr int kPer = 16 / (int)sizeof(R);
+  typedef R Piece __attribute__((ext_vector_type(kPer)));
+  Piece *d = reinterpret_cast<Piece *>(dst);
+#pragma unroll
+  for (int i = 0; i < kChunk / kPer; ++i) {
+    Piece v;
+#pragma unroll
+    for (int e = 0; e < kPer; ++e) v[e] = src[i * kPer + e];
+    d[i] = v;
+  }
+}
+
 struct Counters {
   int ready[kMaxSweep];                   // seam columns published by sweep wave w
   int consumed[kMaxSweep];                // tiles sweep wave w has finished
-  int loaded[kMaxSweep * kBwdStagers];    // tiles staged for sweep wave w by stager l (kBwdStagers >= kFwdStagers)
+  int written[kMaxSweep];                 // backward: tiles whose gradients sweep wave w has left in LDS
+  int loaded[16];                         // tiles staged for sweep wave w by its stager l (index w * stagers + l)
 };
 
 // Geometry of what sweep wave `w` does in band `band`; identical on the sweep
@@ -469,10 +496,14 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
 // down plus what its right neighbour hands left; it is then split into a d1
 // share for the cell below and a d2 share for the cell to the left.  The staging
 // waves evaluate d1 / d2 (mutual_information_cpu.cu:196-212 and the two edge
-// loops :219-235); the sweep wave keeps four steps of px / py gradients in
-// registers and writes them with one 16-byte store per array.
-template <typename R, bool kModified, int kSweepCap>
-__global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
+// loops :219-235).  A single wave issues one instruction every 4-5 cycles, and a sweep
+// wave that also computes addresses and stores its results spends ~140 cycles per
+// step where the dependent chain (shift, add, multiply) needs ~25; so the sweep wave
+// only leaves the px / py gradients of a tile in the LDS buffer it has just read that
+// tile's d1 / d2 from (a lane's 32 steps, 16 bytes per write), and the staging waves
+// carry them to memory, each for the rows it stages, before they refill the buffer.
+template <typename R, bool kModified, int kSweepCap, int kStagers, int kBuffers>
+__global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
     mi_backward_kernel(const R *__restrict__ px, const int64_t *__restrict__ boundary,
                        const R *__restrict__ p, R *ans_grad, R *__restrict__ px_grad,
                        R *__restrict__ py_grad, int S, int T, int overwrite_ans_grad,
@@ -481,7 +512,7 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
   __shared__ Counters cnt;
 
   const int b = blockIdx.x;
-  const int nsweep = blockDim.x / (kWave * (1 + kBwdStagers));
+  const int nsweep = blockDim.x / (kWave * (1 + kStagers));
   const int nwaves = blockDim.x / kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // in a scalar register
   const int lane = threadIdx.x % kWave;
@@ -496,8 +527,9 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
   const __amdgpu_buffer_rsrc_t gy_rsrc = buffer_of(gyb, (size_t)(S + 1) * T);
 
   // Exact zeros everywhere the sweep does not write, one wave per row.  The staging
-  // waves do this after their last tile, off the critical path (a barrier after these
-  // stores would have to wait until they have all reached memory).
+  // waves do this once they are two tiles ahead of their sweep wave, off the critical
+  // path (a barrier after these stores would have to wait until they have all reached
+  // memory).
   // elements [begin, end) of the row that starts at element `row` of the resource;
   // begin and end are wave-uniform
   auto zero_range = [&](__amdgpu_buffer_rsrc_t rs, int row, int begin, int end) {
@@ -550,27 +582,27 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
   const R *pb = p + (size_t)b * (S + 1) * TP;
   R *seam = reinterpret_cast<R *>(dyn_lds);
   const int seam_pitch = (TP + 2 * kSeamPad + 3) & ~3;  // keeps the tiles 16-byte aligned
-  R *tiles = seam + (size_t)nsweep * seam_pitch;  // per sweep wave: d1[2], d2[2] tiles
+  R *tiles = seam + (size_t)nsweep * seam_pitch;  // per sweep wave: kBuffers d1 tiles, then as many d2 tiles
   const int band_rows = kWave * nsweep;
 
   if (wave >= nsweep) {
     // ------------------------------ staging wave -------------------------------
-    const int w = (wave - nsweep) / kBwdStagers, l = (wave - nsweep) % kBwdStagers;
-    R *base = tiles + (size_t)w * 4 * kTileElems;
+    const int w = (wave - nsweep) / kStagers, l = (wave - nsweep) % kStagers;
+    R *base = tiles + (size_t)w * 2 * kBuffers * kTileElems;
     const int half = lane >> 5, q = lane & 31;
-    int *my_loaded = &cnt.loaded[w * kBwdStagers + l];
-    // rows of a tile this wave stages: r(u) = 2*l + half + 2*kBwdStagers*u
-    constexpr int kRows = (kWave + 2 * kBwdStagers - 1) / (2 * kBwdStagers);
+    int *my_loaded = &cnt.loaded[w * kStagers + l];
+    // rows of a tile this wave stages: r(u) = 2*l + half + 2*kStagers*u
+    constexpr int kRows = (kWave + 2 * kStagers - 1) / (2 * kStagers);
     struct Staged {
       R here[kRows], below[kRows], x[kRows];
     };
-    // Global fetches of tile m+1 are issued (into registers) before this wave waits
-    // for the LDS buffers of tile m, so their latency overlaps the sweep.  The loads
-    // are range-checked and otherwise unconditional; staging replaces what was read
-    // for cells outside the window.
+    // Global fetches of tile m+1 are issued (into registers) as soon as tile m is staged,
+    // before this wave waits for the next LDS buffer, so their latency overlaps the
+    // sweep.  The loads are range-checked and otherwise unconditional; staging replaces
+    // what was read for cells outside the window.
     const __amdgpu_buffer_rsrc_t p_rsrc = buffer_of(const_cast<R *>(pb), (size_t)(S + 1) * TP);
     const __amdgpu_buffer_rsrc_t px_rsrc = buffer_of(const_cast<R *>(pxb), (size_t)S * T1);
-    constexpr int kStep = 2 * kBwdStagers;
+    constexpr int kStep = 2 * kStagers;
     constexpr int kSize = (int)sizeof(R);
     const int r_first = 2 * l + half;
     auto fetch = [&](Staged &in, const Band &g, int m) {
@@ -588,22 +620,80 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
         in.here[u] = get1(p_rsrc, here0 - u * (kStep * (TP - 1) * kSize), R());
       }
     };
-    int tile_base = 0;
+    // Gradients of tile m of band g, left by the sweep wave in buffer `buf`: element
+    // (row r, step q) is the cell in reversed column c = 32 m + q - r, i.e. column
+    // j = NT - c of lattice row i = NS - (row0 + r); gx goes to px_grad[s-1][t0 + j - shift],
+    // gy to py_grad[s][t0 + j - 1], where those exist (mutual_information_cpu.cu:213-216).
+    // The straight-line form below (every row group handled alike, borders by select) is
+    // faster than variants that skip the rows past the window's top or branch to a
+    // mask-free copy for tiles inside the window: those were 1 to 5 us slower per launch.
+    auto drain = [&](int pg_row0, int pm, int buf) {
+      const R *gxs = base + buf * kTileElems + r_first * kTilePitch + q;
+      const R *gys = gxs + kBuffers * kTileElems;
+      constexpr int kMinX = kModified ? 1 : 0;
+      const int i0 = NS - pg_row0 - r_first;                // lattice row of u = 0
+      const int j0 = NT - (pm * kTileSteps + q - r_first);  // and its column
+      const int x0 = ((win.s0 + i0 - 1) * T1 + win.t0 - shift + j0) * kSize;
+      const int y0 = ((win.s0 + i0) * T + win.t0 - 1 + j0) * kSize;
+      R vx[kRows], vy[kRows];
+#pragma unroll
+      for (int u = 0; u < kRows; ++u) {
+        if (r_first + kStep * u >= kWave) continue;
+        vx[u] = gxs[u * kStep * kTilePitch];
+        vy[u] = gys[u * kStep * kTilePitch];
+      }
+#pragma unroll
+      for (int u = 0; u < kRows; ++u) {
+        if (r_first + kStep * u >= kWave) continue;
+        // one row group further: kStep rows up in memory and as many columns right
+        const int xo = x0 - u * (kStep * (T1 - 1) * kSize), yo = y0 - u * (kStep * (T - 1) * kSize);
+        const int i = i0 - kStep * u, j = j0 + kStep * u;
+        const bool okx = i > 0 && (unsigned)(j - kMinX) < (unsigned)(NT + 1 - kMinX);
+        const bool oky = i >= 0 && (unsigned)(j - 1) < (unsigned)NT;
+        put1(gx_rsrc, okx ? xo : kDropped, vx[u]);
+        put1(gy_rsrc, oky ? yo : kDropped, vy[u]);
+      }
+    };
+    // which tile each buffer holds: its band's first row and its number in the band
+    int held_row0[kBuffers], held_m[kBuffers];
+#pragma unroll
+    for (int k = 0; k < kBuffers; ++k) held_row0[k] = held_m[k] = 0;
+    auto drain_buffer = [&](int buf) {
+      int row0 = held_row0[0], pm = held_m[0];
+#pragma unroll
+      for (int k = 1; k < kBuffers; ++k) {
+        row0 = buf == k ? held_row0[k] : row0;
+        pm = buf == k ? held_m[k] : pm;
+      }
+      drain(row0, pm, buf);
+    };
+    int tile_base = 0, buf = 0;  // buf = tile number modulo kBuffers
+    bool zeroed = false;
     for (int band = 0; band * band_rows <= NS; ++band) {
       const Band g = band_of(band, w, nsweep, NS, NT);
       if (g.row0 > NS) break;
-      Staged cur, nxt;
+      Staged cur;
       fetch(cur, g, 0);
       for (int m = 0; m < g.ntiles; ++m) {
         const int gt = tile_base + m;
-        if (m + 1 < g.ntiles) fetch(nxt, g, m + 1);
-        if (gt >= 2 && !wait_for(&cnt.consumed[w], gt - 1)) return;
-        R *d1dst = base + (gt & 1) * kTileElems, *d2dst = base + (2 + (gt & 1)) * kTileElems;
+        if (gt >= kBuffers) {
+          // the buffer still holds the gradients of tile gt - kBuffers
+          if (!wait_for(&cnt.written[w], gt - kBuffers + 1)) return;
+          drain_buffer(buf);
+        }
+#pragma unroll
+        for (int k = 0; k < kBuffers; ++k) {
+          held_row0[k] = buf == k ? g.row0 : held_row0[k];
+          held_m[k] = buf == k ? m : held_m[k];
+        }
+        R *d1dst = base + buf * kTileElems + r_first * kTilePitch + q;
+        R *d2dst = d1dst + kBuffers * kTileElems;
         // Which of the window's borders cross this tile (wave-uniform): reversed column 0,
         // where rows start (local step = row); column 0, where they end; the top row.
         const bool starts = m * kTileSteps <= kWave - 1;
         const bool ends = m * kTileSteps + kTileSteps - 1 >= NT;
-        const bool has_top = g.row0 + kWave - 1 >= NS;
+        const int live = NS - g.row0;
+        const bool has_top = live <= kWave - 1;
 #pragma unroll
         for (int u = 0; u < kRows; ++u) {
           const int r = r_first + kStep * u;
@@ -628,22 +718,37 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
           }
           if (has_top) {
             // the top row hands everything left (mutual_information_cpu.cu:228-235)
-            const int i = NS - (g.row0 + r);
+            const int i = live - r;
             if (i <= 0) {
               d1 = 0;
               d2 = (i == 0 && c >= 0 && c < NT) ? (R)1 : (R)0;
             }
           }
-          d1dst[r * kTilePitch + q] = d1;
-          d2dst[r * kTilePitch + q] = d2;
+          d1dst[u * kStep * kTilePitch] = d1;
+          d2dst[u * kStep * kTilePitch] = d2;
         }
         // every lane's LDS writes precede the release by lane 0 of the same wave
         if (lane == 0) publish(my_loaded, gt + 1);
-        cur = nxt;
+        // the next tile's inputs, fetched while this wave waits for its buffer
+        if (m + 1 < g.ntiles) fetch(cur, g, m + 1);
+        buf = buf + 1 == kBuffers ? 0 : buf + 1;
+        if (gt == kBuffers - 1) {
+          // the sweep wave is that many tiles behind now: time for the zeros around the window
+          zero_outside(wave - nsweep, nwaves - nsweep);
+          zeroed = true;
+        }
       }
       tile_base += g.ntiles;
     }
-    zero_outside(wave - nsweep, nwaves - nsweep);
+    // the tiles still in the buffers
+    const int first_left = max(tile_base - kBuffers, 0);
+    buf = first_left % kBuffers;
+    for (int gt = first_left; gt < tile_base; ++gt) {
+      if (!wait_for(&cnt.written[w], gt + 1)) return;
+      drain_buffer(buf);
+      buf = buf + 1 == kBuffers ? 0 : buf + 1;
+    }
+    if (!zeroed) zero_outside(wave - nsweep, nwaves - nsweep);
     // the loss, if asked for: the scores are the forward kernel's, complete before this
     // kernel started, and this wave has nothing left to do
     if (loss && b == 0 && wave == nsweep) reduce_scores(scores, loss, B, reduction, lane);
@@ -655,27 +760,16 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
   const int prev = (w + nsweep - 1) % nsweep;
   R *my_seam = seam + (size_t)w * seam_pitch + kSeamPad;
   const R *up_seam = seam + (size_t)prev * seam_pitch + kSeamPad;
-  const R *base = tiles + (size_t)w * 4 * kTileElems;
+  R *base = tiles + (size_t)w * 2 * kBuffers * kTileElems;
   const R seed = ans_grad ? ans_grad[b] : (R)1;
-  constexpr int kSize = (int)sizeof(R);
-  int tile_base = 0;
+  int tile_base = 0, buf = 0;  // buf = tile number modulo kBuffers
   for (int band = 0; band * band_rows <= NS; ++band) {
     const Band g = band_of(band, w, nsweep, NS, NT);
     if (g.row0 > NS) break;
     const int r = g.row0 + lane;
-    const int i = NS - r;
-    const bool row_ok = r <= NS;
     const bool has_up = g.row0 > 0;
     const int up_base = (w > 0 ? band : band - 1) * cols;
     const int my_base = band * cols;
-    // gx of cell (i, j) goes to px_grad[s-1][t0 + j - shift], gy to py_grad[s][t0 + j - 1].
-    // Byte offsets of (this lane's row, column NT + lane): step e of the sweep is column
-    // NT + lane - e, so a store subtracts its step; lanes without a row (or, for gx, in
-    // the top row) get an offset that every store drops.
-    const int gx_lane = (row_ok && i > 0)
-                            ? ((win.s0 + i - 1) * T1 + win.t0 - shift + NT + lane) * kSize
-                            : kNoRow;
-    const int gy_lane = row_ok ? ((win.s0 + i) * T + win.t0 - 1 + NT + lane) * kSize : kNoRow;
     // the gradient of the origin cell: lane NS - row0 at step NT + NS - row0
     const int fin_lane = NS - g.row0;
     const int fin_step = (fin_lane < kWave) ? NT + fin_lane : -1;
@@ -686,29 +780,27 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
     const bool has_down = g.nrows == kWave;
     int seen_ready = 0;
     R seen_seam = 0;
-    int seen_loaded[kBwdStagers];
+    int seen_loaded[kStagers];
 #pragma unroll
-    for (int l = 0; l < kBwdStagers; ++l) seen_loaded[l] = 0;
+    for (int l = 0; l < kStagers; ++l) seen_loaded[l] = 0;
     for (int m = 0; m < g.ntiles; ++m) {
       const int gt = tile_base + m;
 #pragma unroll
-      for (int l = 0; l < kBwdStagers; ++l)
+      for (int l = 0; l < kStagers; ++l)
         if (__builtin_amdgcn_readfirstlane(seen_loaded[l]) < gt + 1 &&
-            !wait_for(&cnt.loaded[w * kBwdStagers + l], gt + 1))
+            !wait_for(&cnt.loaded[w * kStagers + l], gt + 1))
           return;
       R d1q[kTileSteps], d2q[kTileSteps];
-      {
-        pull_row(d1q, base + (gt & 1) * kTileElems + lane * kTilePitch);
-        pull_row(d2q, base + (2 + (gt & 1)) * kTileElems + lane * kTilePitch);
-      }
-      if (lane == 0) publish(&cnt.consumed[w], gt + 1);
+      R *gx_row = base + buf * kTileElems + lane * kTilePitch;               // d1 in, gx out
+      R *gy_row = base + (kBuffers + buf) * kTileElems + lane * kTilePitch;  // d2 in, gy out
+      buf = buf + 1 == kBuffers ? 0 : buf + 1;
+      pull_row(d1q, gx_row);
+      pull_row(d2q, gy_row);
 
       bool alive = true;
-      auto chunk = [&](auto up_c, auto down_c, auto edge_c, int c4, int e0)
-                       __attribute__((always_inline)) {
+      auto chunk = [&](auto up_c, auto down_c, int c4, int e0) __attribute__((always_inline)) {
         constexpr bool kUp = decltype(up_c)::value;
         constexpr bool kDown = decltype(down_c)::value;
-        constexpr bool kEdge = decltype(edge_c)::value;
         R handed = 0;
         if (kUp) {
           const int need = min(e0 + kChunk - shift, cols);
@@ -730,7 +822,7 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
         }
         if (c4 == kTileSteps / kChunk - 1) {
 #pragma unroll
-          for (int l = 0; l < kBwdStagers; ++l) seen_loaded[l] = peek(&cnt.loaded[w * kBwdStagers + l]);
+          for (int l = 0; l < kStagers; ++l) seen_loaded[l] = peek(&cnt.loaded[w * kStagers + l]);
         }
         R down[kChunk], left[kChunk], cell[kChunk];
 #pragma unroll
@@ -765,45 +857,19 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
 #pragma unroll
             for (int k = 0; k < kChunk; ++k) sp[k] = down[k];
             const int done = max(0, min(e0 + kChunk - (kWave - 1), cols));
-            publish(&cnt.ready[w], my_base + done);
+            publish_lds_writes(&cnt.ready[w], my_base + done);
           }
         }
-        // write-out: a group of four steps is the columns j-3 .. j of its first step
-        const int gx_first = gx_lane - e0 * kSize, gy_first = gy_lane - e0 * kSize;
-        if (!kEdge) {
-#pragma unroll
-          for (int q4 = 0; q4 < kChunk; q4 += 4) {
-            put4(gx_rsrc, gx_first - (q4 + 3) * kSize, down[q4 + 3], down[q4 + 2], down[q4 + 1],
-                 down[q4]);
-            put4(gy_rsrc, gy_first - (q4 + 3) * kSize, left[q4 + 3], left[q4 + 2], left[q4 + 1],
-                 left[q4]);
-          }
-        } else {
-          const int j0 = NT - e0 + lane;  // column of the chunk's first step
-          constexpr int kMinX = kModified ? 1 : 0;
-#pragma unroll
-          for (int k = 0; k < kChunk; ++k) {
-            // inside the window: column <= NT (the lane has started) and >= its first
-            const bool okx = (unsigned)(j0 - k - kMinX) < (unsigned)(NT + 1 - kMinX);
-            const bool oky = (unsigned)(j0 - k - 1) < (unsigned)NT;
-            put1(gx_rsrc, (okx ? gx_first : kDropped) - k * kSize, down[k]);
-            put1(gy_rsrc, (oky ? gy_first : kDropped) - k * kSize, left[k]);
-          }
-        }
+        // the chunk's gradients take the place of its d1 / d2 in the tile
+        push_chunk(gx_row + c4 * kChunk, down);
+        push_chunk(gy_row + c4 * kChunk, left);
       };
       auto tile = [&](auto up_c, auto down_c) __attribute__((always_inline)) {
 #pragma unroll
         for (int c4 = 0; c4 < kTileSteps / kChunk; ++c4) {
           const int e0 = m * kTileSteps + c4 * kChunk;
-          if (e0 < g.nsteps && alive) {
-            // interior: every lane that has a row has started and stays right of
-            // column 0 for all of the chunk's steps
-            const bool interior = e0 >= g.nrows - 1 && e0 + kChunk <= NT;
-            if (interior)
-              chunk(up_c, down_c, std::false_type{}, c4, e0);
-            else
-              chunk(up_c, down_c, std::true_type{}, c4, e0);
-          }
+          // the window's edges need no care here: d1 = d2 = 0 outside it
+          if (e0 < g.nsteps && (!decltype(up_c)::value || alive)) chunk(up_c, down_c, c4, e0);
         }
       };
       if (has_up) {
@@ -818,6 +884,7 @@ __global__ void __launch_bounds__((1 + kBwdStagers) * kSweepCap *kWave)
           tile(std::false_type{}, std::false_type{});
       }
       if (!alive) return;
+      if (lane == 0) publish_lds_writes(&cnt.written[w], gt + 1);
     }
     if (lane == fin_lane && overwrite_ans_grad && ans_grad) ans_grad[b] = g_origin;
     tile_base += g.ntiles;
@@ -874,15 +941,29 @@ int backward_impl(const R *px, const R *py, const int64_t *boundary, const R *p,
   if ((size_t)(S + 1) * (T + 1) * sizeof(R) >= ((size_t)1 << 30))
     return fail(FRNNT_ELIMIT, "mi_backward: one utterance's lattice exceeds 1 GiB");
   const int n = pick_sweep_waves(S, T, sizeof(R), 2);
-  const size_t lds = (size_t)n * ((size_t)((T + 1 + 2 * kSeamPad + 3) & ~3) + 4 * kTileElems) * sizeof(R);
-  if (lds > kLdsBudget)
-    return fail(FRNNT_ELIMIT, "mi_backward: T=%d needs %zu bytes of LDS", T, lds);
-  auto kernel = n <= 2 ? (modified ? mi_backward_kernel<R, true, 2> : mi_backward_kernel<R, false, 2>)
-                       : (modified ? mi_backward_kernel<R, true, kMaxSweep>
-                                   : mi_backward_kernel<R, false, kMaxSweep>);
+  auto lds_bytes = [&](int buffers) {
+    return (size_t)n * ((size_t)((T + 1 + 2 * kSeamPad + 3) & ~3) + 2 * buffers * kTileElems) * sizeof(R);
+  };
+  if (lds_bytes(2) > kLdsBudget)
+    return fail(FRNNT_ELIMIT, "mi_backward: T=%d needs %zu bytes of LDS", T, lds_bytes(2));
+  // With at most two sweep waves there is room for more staging waves per sweep wave and,
+  // for floats, for a third tile buffer, which gives a staging wave two tiles' time instead
+  // of one to empty and refill a buffer.  (A workgroup of 16 waves leaves each 128
+  // registers, too few for a sweep wave's two tile rows of doubles.)
+  constexpr bool kFloat = sizeof(R) == 4;
+  constexpr int kFew = kFloat ? kBwdStagersFew : kBwdStagers;
+  constexpr int kFewBuffers = kFloat ? 3 : 2;
+  static_assert(2 * kFew <= 16 && kMaxSweep * kBwdStagers <= 16, "Counters::loaded is too short");
+  const bool few = n <= 2 && lds_bytes(kFewBuffers) <= kLdsBudget;
+  const int stagers = few ? kFew : kBwdStagers;
+  const size_t lds = lds_bytes(few ? kFewBuffers : 2);
+  auto kernel = few ? (modified ? mi_backward_kernel<R, true, 2, kFew, kFewBuffers>
+                                : mi_backward_kernel<R, false, 2, kFew, kFewBuffers>)
+                    : (modified ? mi_backward_kernel<R, true, kMaxSweep, kBwdStagers, 2>
+                                : mi_backward_kernel<R, false, kMaxSweep, kBwdStagers, 2>);
   if (!allow_lds(reinterpret_cast<const void *>(kernel), lds))
     return check_launch("mi_backward: hipFuncSetAttribute");
-  hipLaunchKernelGGL(kernel, dim3(B), dim3(n * (1 + kBwdStagers) * kWave), lds,
+  hipLaunchKernelGGL(kernel, dim3(B), dim3(n * (1 + stagers) * kWave), lds,
                      static_cast<hipStream_t>(stream), px, boundary, p, ans_grad, px_grad,
                      py_grad, S, T, overwrite_ans_grad, scores, loss, B, reduction);
   return check_launch("mi_backward");
