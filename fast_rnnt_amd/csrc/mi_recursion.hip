@@ -43,7 +43,9 @@ constexpr int kSeamPad = kChunk;        // slack on either side of a seam row, s
                                        // chunk of seam values is written without bounds tests
 constexpr int kFwdStagers = 2;         // staging waves per sweep wave
 constexpr int kBwdStagers = 3;
-constexpr int kBwdStagersFew = 7;  // with at most two sweep waves: 16 waves, the largest workgroup
+// with at most two sweep waves (16 waves are the largest workgroup)
+constexpr int kFwdStagersFew = 7;
+constexpr int kBwdStagersFew = 7;
 constexpr int kSpinLimit = 1 << 22;
 
 struct Window {
@@ -118,9 +120,6 @@ __device__ __forceinline__ double chain_log_add(double a, double c) { return log
 // turns "this lane has nothing to write here" into one select on the offset, with
 // no branch and no change of the execution mask.
 constexpr int kDropped = (int)0x80000000;
-// Byte offset standing for "this lane has no row": adding any in-row displacement
-// (less than 2^30 in magnitude) to it still lies outside every resource.
-constexpr int kNoRow = (int)0xC0000000;
 typedef int intx2 __attribute__((ext_vector_type(2)));
 typedef int intx4 __attribute__((ext_vector_type(4)));
 
@@ -193,8 +192,7 @@ __device__ __forceinline__ void push_chunk(R *dst, const R (&src)[kChunk]) {
 
 struct Counters {
   int ready[kMaxSweep];                   // seam columns published by sweep wave w
-  int consumed[kMaxSweep];                // tiles sweep wave w has finished
-  int written[kMaxSweep];                 // backward: tiles whose gradients sweep wave w has left in LDS
+  int written[kMaxSweep];                 // tiles whose results sweep wave w has left in LDS
   int loaded[16];                         // tiles staged for sweep wave w by its stager l (index w * stagers + l)
 };
 
@@ -216,9 +214,12 @@ __device__ __forceinline__ Band band_of(int band, int w, int nsweep, int NS, int
 // Staged per step and row: x = px feeding the cell from the row below,
 // y = py feeding it from the left; -inf where that edge does not exist, and
 // y = 0 at the origin cell so that the chain produces p = 0 there.
+// A sweep wave only runs the chain: it takes a tile's x / y from an LDS buffer and
+// leaves the tile's p in the place of x (16 bytes per LDS write); the staging waves
+// carry p to memory, each for the rows it stages, before they refill the buffer.
 // kSweepCap: most sweep waves the launch may use; it only sets the register budget.
-template <typename R, bool kModified, int kSweepCap>
-__global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
+template <typename R, bool kModified, int kSweepCap, int kStagers, int kBuffers>
+__global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
     mi_forward_kernel(const R *__restrict__ px, const R *__restrict__ py,
                       const int64_t *__restrict__ boundary, R *__restrict__ p,
                       R *__restrict__ ans, int S, int T) {
@@ -226,7 +227,7 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
   __shared__ Counters cnt;
 
   const int b = blockIdx.x;
-  const int nsweep = blockDim.x / (kWave * (1 + kFwdStagers));
+  const int nsweep = blockDim.x / (kWave * (1 + kStagers));
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // in a scalar register
   const int lane = threadIdx.x % kWave;
   const int T1 = kModified ? T : T + 1;
@@ -247,33 +248,32 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
   const R *pxb = px + (size_t)b * S * T1;
   const R *pyb = py + (size_t)b * (S + 1) * T;
   R *pb = p + (size_t)b * (S + 1) * TP;
-  const __amdgpu_buffer_rsrc_t p_rsrc = buffer_of(pb, (size_t)(S + 1) * TP);
   R *seam = reinterpret_cast<R *>(dyn_lds);
   const int seam_pitch = (TP + 2 * kSeamPad + 3) & ~3;  // keeps the tiles 16-byte aligned
-  R *tiles = seam + (size_t)nsweep * seam_pitch;  // [nsweep][2 arrays][2 buffers][kTileElems]
+  R *tiles = seam + (size_t)nsweep * seam_pitch;  // per sweep wave: kBuffers x tiles, then as many y tiles
   const int band_rows = kWave * nsweep;
 
   if (wave >= nsweep) {
     // ------------------------------ staging wave -------------------------------
-    const int w = (wave - nsweep) / kFwdStagers, l = (wave - nsweep) % kFwdStagers;
-    R *xt = tiles + (size_t)w * 4 * kTileElems;
-    R *yt = xt + 2 * kTileElems;
+    const int w = (wave - nsweep) / kStagers, l = (wave - nsweep) % kStagers;
+    R *base = tiles + (size_t)w * 2 * kBuffers * kTileElems;
     const int half = lane >> 5, q = lane & 31;
-    // rows of a tile this wave stages: r(u) = 2*l + half + 2*kFwdStagers*u
-    constexpr int kRows = (kWave + 2 * kFwdStagers - 1) / (2 * kFwdStagers);
+    int *my_loaded = &cnt.loaded[w * kStagers + l];
+    // rows of a tile this wave stages: r(u) = 2*l + half + 2*kStagers*u
+    constexpr int kRows = (kWave + 2 * kStagers - 1) / (2 * kStagers);
     struct Staged {
       R x[kRows], y[kRows];
     };
-    // Global fetches of a tile go to registers and do not need the LDS buffer, so
-    // the fetch of tile m+1 is issued before this wave waits for the buffer of tile
-    // m to be released: the memory latency overlaps the sweep.  The loads are
-    // range-checked and otherwise unconditional: what a lane reads for cells outside
-    // the window is either replaced at staging time (row 0, column 0: the -inf that
-    // closes the lattice) or never reaches a cell of the window (columns before a
-    // row's start or beyond its end only feed cells at least as far out).
+    // Global fetches of tile m+1 are issued (into registers) as soon as tile m is staged,
+    // before this wave waits for the next LDS buffer, so their latency overlaps the
+    // sweep.  The loads are range-checked and otherwise unconditional: what a lane reads
+    // for cells outside the window is either replaced at staging time (row 0, column 0:
+    // the -inf that closes the lattice) or never reaches a cell of the window (columns
+    // before a row's start or beyond its end only feed cells at least as far out).
     const __amdgpu_buffer_rsrc_t px_rsrc = buffer_of(const_cast<R *>(pxb), (size_t)S * T1);
     const __amdgpu_buffer_rsrc_t py_rsrc = buffer_of(const_cast<R *>(pyb), (size_t)(S + 1) * T);
-    constexpr int kStep = 2 * kFwdStagers;
+    const __amdgpu_buffer_rsrc_t p_rsrc = buffer_of(pb, (size_t)(S + 1) * TP);
+    constexpr int kStep = 2 * kStagers;
     constexpr int kSize = (int)sizeof(R);
     const int r_first = 2 * l + half;
     auto fetch = [&](Staged &in, const Band &g, int m) {
@@ -288,17 +288,60 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
         in.y[u] = get1(py_rsrc, y0 + u * (kStep * (T - 1) * kSize), R());
       }
     };
-    int tile_base = 0;
+    // p of tile pm of the band that starts at row0, left by the sweep wave in buffer `buf`:
+    // element (row r, step q) is the cell (row0 + r, 32 pm + q - r) of the window.
+    auto drain = [&](int row0, int pm, int buf) {
+      const R *ps = base + buf * kTileElems + r_first * kTilePitch + q;
+      const int i0 = row0 + r_first;
+      const int j0 = pm * kTileSteps + q - r_first;
+      const int o0 = ((win.s0 + i0) * TP + win.t0 + j0) * kSize;
+      R v[kRows];
+#pragma unroll
+      for (int u = 0; u < kRows; ++u) {
+        if (r_first + kStep * u >= kWave) continue;
+        v[u] = ps[u * kStep * kTilePitch];
+      }
+#pragma unroll
+      for (int u = 0; u < kRows; ++u) {
+        if (r_first + kStep * u >= kWave) continue;
+        const int i = i0 + kStep * u, j = j0 - kStep * u;
+        const bool ok = i <= NS && (unsigned)j <= (unsigned)NT;
+        put1(p_rsrc, ok ? o0 + u * (kStep * (TP - 1) * kSize) : kDropped, v[u]);
+      }
+    };
+    // which tile each buffer holds: its band's first row and its number in the band
+    int held_row0[kBuffers], held_m[kBuffers];
+#pragma unroll
+    for (int k = 0; k < kBuffers; ++k) held_row0[k] = held_m[k] = 0;
+    auto drain_buffer = [&](int buf) {
+      int row0 = held_row0[0], pm = held_m[0];
+#pragma unroll
+      for (int k = 1; k < kBuffers; ++k) {
+        row0 = buf == k ? held_row0[k] : row0;
+        pm = buf == k ? held_m[k] : pm;
+      }
+      drain(row0, pm, buf);
+    };
+    int tile_base = 0, buf = 0;  // buf = tile number modulo kBuffers
     for (int band = 0; band * band_rows <= NS; ++band) {
       const Band g = band_of(band, w, nsweep, NS, NT);
       if (g.row0 > NS) break;
-      Staged cur, nxt;
+      Staged cur;
       fetch(cur, g, 0);
       for (int m = 0; m < g.ntiles; ++m) {
         const int gt = tile_base + m;
-        if (m + 1 < g.ntiles) fetch(nxt, g, m + 1);
-        if (gt >= 2 && !wait_for(&cnt.consumed[w], gt - 1)) return;
-        R *xdst = xt + (gt & 1) * kTileElems, *ydst = yt + (gt & 1) * kTileElems;
+        if (gt >= kBuffers) {
+          // the buffer still holds p of tile gt - kBuffers
+          if (!wait_for(&cnt.written[w], gt - kBuffers + 1)) return;
+          drain_buffer(buf);
+        }
+#pragma unroll
+        for (int k = 0; k < kBuffers; ++k) {
+          held_row0[k] = buf == k ? g.row0 : held_row0[k];
+          held_m[k] = buf == k ? m : held_m[k];
+        }
+        R *xdst = base + buf * kTileElems + r_first * kTilePitch + q;
+        R *ydst = xdst + kBuffers * kTileElems;
         // only the first tiles hold a column 0 (local step = row), and only the first
         // band holds row 0
         const bool starts = m * kTileSteps <= kWave - 1 + shift;
@@ -314,13 +357,24 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
             if (j < shift) x = ninf;
           }
           if (u == 0 && i == 0) x = ninf;
-          xdst[r * kTilePitch + q] = x;
-          ydst[r * kTilePitch + q] = y;
+          xdst[u * kStep * kTilePitch] = x;
+          ydst[u * kStep * kTilePitch] = y;
         }
-        if (lane == 0) publish(&cnt.loaded[w * kFwdStagers + l], gt + 1);
-        cur = nxt;
+        // every lane's LDS writes precede the release by lane 0 of the same wave
+        if (lane == 0) publish(my_loaded, gt + 1);
+        // the next tile's inputs, fetched while this wave waits for its buffer
+        if (m + 1 < g.ntiles) fetch(cur, g, m + 1);
+        buf = buf + 1 == kBuffers ? 0 : buf + 1;
       }
       tile_base += g.ntiles;
+    }
+    // the tiles still in the buffers
+    const int first_left = max(tile_base - kBuffers, 0);
+    buf = first_left % kBuffers;
+    for (int gt = first_left; gt < tile_base; ++gt) {
+      if (!wait_for(&cnt.written[w], gt + 1)) return;
+      drain_buffer(buf);
+      buf = buf + 1 == kBuffers ? 0 : buf + 1;
     }
     return;
   }
@@ -330,20 +384,15 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
   const int prev = (w + nsweep - 1) % nsweep;
   R *my_seam = seam + (size_t)w * seam_pitch + kSeamPad;
   const R *up_seam = seam + (size_t)prev * seam_pitch + kSeamPad;
-  const R *xt = tiles + (size_t)w * 4 * kTileElems;
-  const R *yt = xt + 2 * kTileElems;
-  int tile_base = 0;
+  R *base = tiles + (size_t)w * 2 * kBuffers * kTileElems;
+  int tile_base = 0, buf = 0;  // buf = tile number modulo kBuffers
   for (int band = 0; band * band_rows <= NS; ++band) {
     const Band g = band_of(band, w, nsweep, NS, NT);
     if (g.row0 > NS) break;
     const int i = g.row0 + lane;
-    const bool row_ok = i <= NS;
     const bool has_up = g.row0 > 0;
     const int up_base = (w > 0 ? band : band - 1) * cols;
     const int my_base = band * cols;
-    // byte offset in p[b] of (this lane's row, column -lane): a chunk adds its first
-    // step; lanes without a row get an offset that every store drops
-    const int p_lane = row_ok ? ((win.s0 + i) * TP + win.t0 - lane) * (int)sizeof(R) : kNoRow;
     // the answer is the cell (NS, NT): lane NS - row0 at step NT + NS - row0
     const int fin_lane = NS - g.row0;
     const int fin_step = (fin_lane < kWave) ? NT + fin_lane : -1;
@@ -355,34 +404,29 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
     // that the LDS round trip is off the chain; a stale value only costs a re-read
     int seen_ready = 0;
     R seen_seam = ninf;
-    int seen_loaded[kFwdStagers];
+    int seen_loaded[kStagers];
 #pragma unroll
-    for (int l = 0; l < kFwdStagers; ++l) seen_loaded[l] = 0;
+    for (int l = 0; l < kStagers; ++l) seen_loaded[l] = 0;
     for (int m = 0; m < g.ntiles; ++m) {
       const int gt = tile_base + m;
 #pragma unroll
-      for (int l = 0; l < kFwdStagers; ++l)
+      for (int l = 0; l < kStagers; ++l)
         if (__builtin_amdgcn_readfirstlane(seen_loaded[l]) < gt + 1 &&
-            !wait_for(&cnt.loaded[w * kFwdStagers + l], gt + 1))
+            !wait_for(&cnt.loaded[w * kStagers + l], gt + 1))
           return;
-      // this lane's 32 steps of inputs go to registers in one burst, after which
-      // the staging waves may refill the buffer
+      // this lane's 32 steps of inputs go to registers in one burst
       R xq[kTileSteps], yq[kTileSteps];
-      {
-        pull_row(xq, xt + (gt & 1) * kTileElems + lane * kTilePitch);
-        pull_row(yq, yt + (gt & 1) * kTileElems + lane * kTilePitch);
-      }
-      if (lane == 0) publish(&cnt.consumed[w], gt + 1);
+      R *x_row = base + buf * kTileElems + lane * kTilePitch;  // x in, p out
+      pull_row(xq, x_row);
+      pull_row(yq, x_row + kBuffers * kTileElems);
+      buf = buf + 1 == kBuffers ? 0 : buf + 1;
 
       // One chunk of kChunk steps, specialised at compile time on whether the wave
-      // receives a seam (kUp), feeds one (kDown), and whether some lane's column
-      // leaves the window during the chunk (kEdge).
+      // receives a seam (kUp) and feeds one (kDown).
       bool alive = true;
-      auto chunk = [&](auto up_c, auto down_c, auto edge_c, int c4, int e0)
-                       __attribute__((always_inline)) {
+      auto chunk = [&](auto up_c, auto down_c, int c4, int e0) __attribute__((always_inline)) {
         constexpr bool kUp = decltype(up_c)::value;
         constexpr bool kDown = decltype(down_c)::value;
-        constexpr bool kEdge = decltype(edge_c)::value;
         R handed = ninf;  // lane k: the seam value lane 0 needs at step e0 + k
         if (kUp) {
           const int need = min(e0 + kChunk - shift, cols);
@@ -404,7 +448,7 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
         }
         if (c4 == kTileSteps / kChunk - 1) {
 #pragma unroll
-          for (int l = 0; l < kFwdStagers; ++l) seen_loaded[l] = peek(&cnt.loaded[w * kFwdStagers + l]);
+          for (int l = 0; l < kStagers; ++l) seen_loaded[l] = peek(&cnt.loaded[w * kStagers + l]);
         }
         R vals[kChunk];
 #pragma unroll
@@ -438,37 +482,17 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
 #pragma unroll
             for (int k = 0; k < kChunk; ++k) sp[k] = vals[k];
             const int done = max(0, min(e0 + kChunk - (kWave - 1), cols));
-            publish(&cnt.ready[w], my_base + done);
+            publish_lds_writes(&cnt.ready[w], my_base + done);
           }
         }
-        // p: whole groups of four columns inside the window, single columns at its ends
-        const int first = p_lane + e0 * (int)sizeof(R);
-        if (!kEdge) {
-#pragma unroll
-          for (int q4 = 0; q4 < kChunk; q4 += 4)
-            put4(p_rsrc, first + q4 * (int)sizeof(R), vals[q4], vals[q4 + 1], vals[q4 + 2],
-                 vals[q4 + 3]);
-        } else {
-          const int j0 = e0 - lane;
-#pragma unroll
-          for (int k = 0; k < kChunk; ++k) {
-            const bool ok = (unsigned)(j0 + k) <= (unsigned)NT;
-            put1(p_rsrc, (ok ? first : kDropped) + k * (int)sizeof(R), vals[k]);
-          }
-        }
+        // the chunk's p takes the place of its x in the tile
+        push_chunk(x_row + c4 * kChunk, vals);
       };
       auto tile = [&](auto up_c, auto down_c) __attribute__((always_inline)) {
 #pragma unroll
         for (int c4 = 0; c4 < kTileSteps / kChunk; ++c4) {
           const int e0 = m * kTileSteps + c4 * kChunk;
-          if (e0 < g.nsteps && alive) {
-            // interior: the columns of all lanes that have a row stay inside the window
-            const bool interior = e0 >= g.nrows - 1 && e0 + kChunk <= NT + 1;
-            if (interior)
-              chunk(up_c, down_c, std::false_type{}, c4, e0);
-            else
-              chunk(up_c, down_c, std::true_type{}, c4, e0);
-          }
+          if (e0 < g.nsteps && (!decltype(up_c)::value || alive)) chunk(up_c, down_c, c4, e0);
         }
       };
       if (has_up) {
@@ -483,6 +507,7 @@ __global__ void __launch_bounds__((1 + kFwdStagers) * kSweepCap *kWave)
           tile(std::false_type{}, std::false_type{});
       }
       if (!alive) return;
+      if (lane == 0) publish_lds_writes(&cnt.written[w], gt + 1);
     }
     if (lane == fin_lane) ans[b] = fin;
     tile_base += g.ntiles;
@@ -904,6 +929,11 @@ int pick_sweep_waves(int S, int T, size_t elem, int arrays) {
   return n;
 }
 
+// Dynamic LDS of a launch: per sweep wave a seam row and 2 x buffers tiles.
+size_t lds_bytes(int nsweep, int T, int buffers, size_t elem) {
+  return (size_t)nsweep * ((size_t)((T + 1 + 2 * kSeamPad + 3) & ~3) + (size_t)2 * buffers * kTileElems) * elem;
+}
+
 template <typename R>
 int forward_impl(const R *px, const R *py, const int64_t *boundary, R *p, R *ans, int B, int S,
                  int T, int modified, void *stream) {
@@ -913,15 +943,26 @@ int forward_impl(const R *px, const R *py, const int64_t *boundary, R *p, R *ans
   if ((size_t)(S + 1) * (T + 1) * sizeof(R) >= ((size_t)1 << 30))
     return fail(FRNNT_ELIMIT, "mi_forward: one utterance's lattice exceeds 1 GiB");
   const int n = pick_sweep_waves(S, T, sizeof(R), 2);
-  const size_t lds = (size_t)n * ((size_t)((T + 1 + 2 * kSeamPad + 3) & ~3) + 4 * kTileElems) * sizeof(R);
-  if (lds > kLdsBudget)
-    return fail(FRNNT_ELIMIT, "mi_forward: T=%d needs %zu bytes of LDS", T, lds);
-  auto kernel = n <= 2 ? (modified ? mi_forward_kernel<R, true, 2> : mi_forward_kernel<R, false, 2>)
-                       : (modified ? mi_forward_kernel<R, true, kMaxSweep>
-                                   : mi_forward_kernel<R, false, kMaxSweep>);
+  if (lds_bytes(n, T, 2, sizeof(R)) > kLdsBudget)
+    return fail(FRNNT_ELIMIT, "mi_forward: T=%d needs %zu bytes of LDS", T, lds_bytes(n, T, 2, sizeof(R)));
+  // With at most two sweep waves there is room for more staging waves per sweep wave and,
+  // for floats, for a third tile buffer, which gives a staging wave two tiles' time instead
+  // of one to empty and refill a buffer.  (A workgroup of 16 waves leaves each 128
+  // registers, too few for a sweep wave's two tile rows of doubles.)
+  constexpr bool kFloat = sizeof(R) == 4;
+  constexpr int kFew = kFloat ? kFwdStagersFew : kFwdStagers;
+  constexpr int kFewBuffers = kFloat ? 3 : 2;
+  static_assert(2 * kFew <= 16 && kMaxSweep * kFwdStagers <= 16, "Counters::loaded is too short");
+  const bool few = n <= 2 && lds_bytes(n, T, kFewBuffers, sizeof(R)) <= kLdsBudget;
+  const int stagers = few ? kFew : kFwdStagers;
+  const size_t lds = lds_bytes(n, T, few ? kFewBuffers : 2, sizeof(R));
+  auto kernel = few ? (modified ? mi_forward_kernel<R, true, 2, kFew, kFewBuffers>
+                                : mi_forward_kernel<R, false, 2, kFew, kFewBuffers>)
+                    : (modified ? mi_forward_kernel<R, true, kMaxSweep, kFwdStagers, 2>
+                                : mi_forward_kernel<R, false, kMaxSweep, kFwdStagers, 2>);
   if (!allow_lds(reinterpret_cast<const void *>(kernel), lds))
     return check_launch("mi_forward: hipFuncSetAttribute");
-  hipLaunchKernelGGL(kernel, dim3(B), dim3(n * (1 + kFwdStagers) * kWave), lds,
+  hipLaunchKernelGGL(kernel, dim3(B), dim3(n * (1 + stagers) * kWave), lds,
                      static_cast<hipStream_t>(stream), px, py, boundary, p, ans, S, T);
   return check_launch("mi_forward");
 }
@@ -941,11 +982,8 @@ int backward_impl(const R *px, const R *py, const int64_t *boundary, const R *p,
   if ((size_t)(S + 1) * (T + 1) * sizeof(R) >= ((size_t)1 << 30))
     return fail(FRNNT_ELIMIT, "mi_backward: one utterance's lattice exceeds 1 GiB");
   const int n = pick_sweep_waves(S, T, sizeof(R), 2);
-  auto lds_bytes = [&](int buffers) {
-    return (size_t)n * ((size_t)((T + 1 + 2 * kSeamPad + 3) & ~3) + 2 * buffers * kTileElems) * sizeof(R);
-  };
-  if (lds_bytes(2) > kLdsBudget)
-    return fail(FRNNT_ELIMIT, "mi_backward: T=%d needs %zu bytes of LDS", T, lds_bytes(2));
+  if (lds_bytes(n, T, 2, sizeof(R)) > kLdsBudget)
+    return fail(FRNNT_ELIMIT, "mi_backward: T=%d needs %zu bytes of LDS", T, lds_bytes(n, T, 2, sizeof(R)));
   // With at most two sweep waves there is room for more staging waves per sweep wave and,
   // for floats, for a third tile buffer, which gives a staging wave two tiles' time instead
   // of one to empty and refill a buffer.  (A workgroup of 16 waves leaves each 128
@@ -954,9 +992,9 @@ int backward_impl(const R *px, const R *py, const int64_t *boundary, const R *p,
   constexpr int kFew = kFloat ? kBwdStagersFew : kBwdStagers;
   constexpr int kFewBuffers = kFloat ? 3 : 2;
   static_assert(2 * kFew <= 16 && kMaxSweep * kBwdStagers <= 16, "Counters::loaded is too short");
-  const bool few = n <= 2 && lds_bytes(kFewBuffers) <= kLdsBudget;
+  const bool few = n <= 2 && lds_bytes(n, T, kFewBuffers, sizeof(R)) <= kLdsBudget;
   const int stagers = few ? kFew : kBwdStagers;
-  const size_t lds = lds_bytes(few ? kFewBuffers : 2);
+  const size_t lds = lds_bytes(n, T, few ? kFewBuffers : 2, sizeof(R));
   auto kernel = few ? (modified ? mi_backward_kernel<R, true, 2, kFew, kFewBuffers>
                                 : mi_backward_kernel<R, false, 2, kFew, kFewBuffers>)
                     : (modified ? mi_backward_kernel<R, true, kMaxSweep, kBwdStagers, 2>
