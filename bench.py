@@ -30,8 +30,8 @@ FP32_MFMA_PEAK_TFLOPS = 157.3
 # copy of known size); filled in for the workloads that were profiled
 MEASURED_TRAFFIC = {
     ("c2", "simple_fwd_panel_kernel<96, 16>"): 29257616,
-    ("c2", "mi_forward_kernel<float, false, 2>"): 6868061,
-    ("c2", "mi_backward_kernel<float, false, 2>"): 9809965,
+    ("c2", "mi_forward_kernel<float, false, 2, 2, 3>"): 6868061,
+    ("c2", "mi_backward_kernel<float, false, 2, 7, 3>"): 9809965,
 }
 
 
@@ -321,9 +321,9 @@ def main():
     gemm_flops = 2.0 * B * (S + 1) * T * w.C
     gemm_tflops = gemm_flops / (t_logp * 1e-3) / 1e12
     lines = [
-        hbm_line("mi_forward_kernel<float, false, 2>",
+        hbm_line("mi_forward_kernel<float, false, 2, 2, 3>",
                  _recursion_bytes(w.boundary, S, T, B, backward=False), t_fwd),
-        hbm_line("mi_backward_kernel<float, false, 2>",
+        hbm_line("mi_backward_kernel<float, false, 2, 7, 3>",
                  _recursion_bytes(w.boundary, S, T, B, backward=True), t_bwd),
         {"kernel": gemm_name, "bound": "mfma", "achieved": round(gemm_tflops, 3),
          "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",

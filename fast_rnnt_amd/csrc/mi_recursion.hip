@@ -43,8 +43,10 @@ constexpr int kSeamPad = kChunk;        // slack on either side of a seam row, s
                                        // chunk of seam values is written without bounds tests
 constexpr int kFwdStagers = 2;         // staging waves per sweep wave
 constexpr int kBwdStagers = 3;
-// with at most two sweep waves (16 waves are the largest workgroup)
-constexpr int kFwdStagersFew = 7;
+// With at most two sweep waves the backward kernel runs 16 waves, the largest workgroup:
+// its staging waves evaluate d1 / d2 and are what the sweep waits for.  The forward
+// kernel's staging waves only copy, and more of them slow the sweep waves down (c2
+// shape: 21.4 us with 2, 22.2 with 5, 23.0 with 7 per sweep wave).
 constexpr int kBwdStagersFew = 7;
 constexpr int kSpinLimit = 1 << 22;
 
@@ -945,19 +947,15 @@ int forward_impl(const R *px, const R *py, const int64_t *boundary, R *p, R *ans
   const int n = pick_sweep_waves(S, T, sizeof(R), 2);
   if (lds_bytes(n, T, 2, sizeof(R)) > kLdsBudget)
     return fail(FRNNT_ELIMIT, "mi_forward: T=%d needs %zu bytes of LDS", T, lds_bytes(n, T, 2, sizeof(R)));
-  // With at most two sweep waves there is room for more staging waves per sweep wave and,
-  // for floats, for a third tile buffer, which gives a staging wave two tiles' time instead
-  // of one to empty and refill a buffer.  (A workgroup of 16 waves leaves each 128
-  // registers, too few for a sweep wave's two tile rows of doubles.)
-  constexpr bool kFloat = sizeof(R) == 4;
-  constexpr int kFew = kFloat ? kFwdStagersFew : kFwdStagers;
-  constexpr int kFewBuffers = kFloat ? 3 : 2;
-  static_assert(2 * kFew <= 16 && kMaxSweep * kFwdStagers <= 16, "Counters::loaded is too short");
+  // With at most two sweep waves there is room, for floats, for a third tile buffer, which
+  // gives a staging wave two tiles' time instead of one to empty and refill a buffer.
+  constexpr int kFewBuffers = sizeof(R) == 4 ? 3 : 2;
+  static_assert(kMaxSweep * kFwdStagers <= 16, "Counters::loaded is too short");
   const bool few = n <= 2 && lds_bytes(n, T, kFewBuffers, sizeof(R)) <= kLdsBudget;
-  const int stagers = few ? kFew : kFwdStagers;
+  const int stagers = kFwdStagers;
   const size_t lds = lds_bytes(n, T, few ? kFewBuffers : 2, sizeof(R));
-  auto kernel = few ? (modified ? mi_forward_kernel<R, true, 2, kFew, kFewBuffers>
-                                : mi_forward_kernel<R, false, 2, kFew, kFewBuffers>)
+  auto kernel = few ? (modified ? mi_forward_kernel<R, true, 2, kFwdStagers, kFewBuffers>
+                                : mi_forward_kernel<R, false, 2, kFwdStagers, kFewBuffers>)
                     : (modified ? mi_forward_kernel<R, true, kMaxSweep, kFwdStagers, 2>
                                 : mi_forward_kernel<R, false, kMaxSweep, kFwdStagers, 2>);
   if (!allow_lds(reinterpret_cast<const void *>(kernel), lds))
