@@ -4,8 +4,9 @@
 One step = one ``rnnt_loss_simple(..., reduction="sum", return_grad=True)`` call
 plus ``loss.backward()`` on the synthetic ASR-shaped batch c2
 (B=32, T=250, S=80, C=500, fp32; inputs already resident in HBM).  Prints ONE
-JSON line: whole-call throughput (the step replayed as a HIP graph, checked
-bit-equal against eager steps; the eager loop's figure beside it), the roofline
+JSON line: whole-call throughput (the faster of an eager loop and of the step
+replayed as a HIP graph, which is checked bit-equal against eager steps; both
+figures are in the line), the roofline
 figure of the dominant kernel (timed live with events on the launch stream) and
 the CPU baseline (the oracle restatement of the reference path, timed on this
 host's cores).
@@ -29,9 +30,9 @@ FP32_MFMA_PEAK_TFLOPS = 157.3
 # profiles/ (FETCH_SIZE and WRITE_SIZE, scaled by what the same counters read for a
 # copy of known size); filled in for the workloads that were profiled
 MEASURED_TRAFFIC = {
-    ("c2", "simple_fwd_panel_kernel<96, 16>"): 29257616,
-    ("c2", "mi_forward_kernel<float, false, 2, 2, 3>"): 6868061,
-    ("c2", "mi_backward_kernel<float, false, 2, 7, 3>"): 9809965,
+    ("c2", "simple_fwd_panel_kernel<96, 16>"): 29257692,
+    ("c2", "mi_forward_kernel<float, false, 2, 2, 3>"): 6736766,
+    ("c2", "mi_backward_kernel<float, false, 2, 7, 3>"): 9688133,
 }
 
 
@@ -374,14 +375,16 @@ def main():
             "loss_rel_diff_vs_gpu": abs(gpu_loss - cpu_loss.item()) / abs(cpu_loss.item()),
         }
 
-    # The step is nine kernels of 4-25 us: an eager loop of nothing but this call is bound
-    # by the host's launch work on slow hosts (in training that work hides behind the
-    # model's own kernels).  The headline is therefore the replayed graph of the same step
-    # -- same kernels, outputs checked bit-equal against eager steps -- and the eager loop
-    # is reported beside it; without a graph (capture refused, --no-graph) eager is the headline.
+    # The step is eight kernels of 4-25 us.  An eager loop of nothing but this call is bound by
+    # the host's launch work on slow hosts (in training that work hides behind the model's own
+    # kernels); the replayed graph of the same step -- same kernels, outputs checked bit-equal
+    # against eager steps -- does not depend on the host, but its nodes start a little further
+    # apart than kernels a fast host has queued ahead.  Both loops time exactly args.steps whole
+    # steps; the headline is the faster of the two and config.mode says which, and both are
+    # reported beside it.  Without a graph (capture refused, --no-graph) eager is the headline.
     eager = {"value": round(calls_per_sec, 2), "unit": "calls/sec",
              "ms_per_step": round(ms_per_step, 4), "steps": args.steps}
-    graphed = replay is not None and "value" in replay
+    graphed = replay is not None and "value" in replay and replay["value"] > calls_per_sec
     mode = ("HIP-graph replay of one captured rnnt_loss_simple + backward step" if graphed
             else "eager calls")
     if graphed:
