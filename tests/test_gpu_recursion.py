@@ -125,6 +125,18 @@ def test_taller_than_one_workgroup(gpu_device):
     _compare(px32, py32, None, torch.ones(B), gpu_device, "tall32")
 
 
+def test_long_utterance_two_tile_buffers(gpu_device):
+    # T beyond what three LDS tile buffers per sweep wave leave room for (about 6100 frames
+    # with two sweep waves): the float kernels fall back to two buffers and fewer staging
+    # waves.  Inputs centred at -log 2 keep |p| small, so the float32 bounds stay meaningful.
+    g = torch.Generator().manual_seed(9)
+    B, S, T = 2, 70, 6300
+    px = -math.log(2.0) + 0.05 * torch.randn(B, S, T + 1, generator=g)
+    py = -math.log(2.0) + 0.05 * torch.randn(B, S + 1, T, generator=g)
+    bnd = torch.tensor([[0, 0, S, T], [3, 40, 66, 6290]], dtype=torch.int64)
+    _compare(px, py, bnd, torch.ones(B), gpu_device, "long")
+
+
 def test_north_star_shape(gpu_device):
     g = torch.Generator().manual_seed(1002)
     B, S, T = 32, 80, 250
