@@ -101,15 +101,32 @@ __global__ void __launch_bounds__(256)
 }
 
 // The same with the row held in registers (fp32, C a multiple of 4, at most
-// 256 * kVecs entries): the logits are read once, 16 bytes per lane and load.
+// 256 * kVecs entries): the logits are read once, 16 bytes per lane and load.  The two
+// entries the row contributes to px / py are taken from the registers that hold them
+// (selects under wave-uniform conditions, then a read of the owning lane), not read
+// again from memory: a second, dependent load would keep every wave alive for another
+// memory round trip.  The row's symbol comes through the scalar cache while the logits
+// travel.
 typedef float floatx4u __attribute__((ext_vector_type(4), aligned(4)));
+template <int kVecs>
+__device__ __forceinline__ float row_entry(const floatx4u (&v)[kVecs], int c) {
+  // c is wave-uniform and inside the row
+  const int piece = c >> 2, e = c & 3, vec = piece / kWave, owner = piece % kWave;
+  float cand = v[0][0];
+#pragma unroll
+  for (int i = 0; i < kVecs; ++i)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) cand = (i == vec && k == e) ? v[i][k] : cand;
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(cand), owner));
+}
 template <int kVecs>
 __global__ void __launch_bounds__(256)
     row_norm_regs_kernel(const float *__restrict__ logits, const int64_t *__restrict__ symbols,
                          const int64_t *__restrict__ ranges, float *__restrict__ norm,
                          float *__restrict__ xr, float *__restrict__ yr, long rows, int T, int Rr,
                          int S, int C, int term) {
-  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // in a scalar register
+  const long row = (long)blockIdx.x * 4 + wave;
   const int lane = threadIdx.x & 63;
   if (row >= rows) return;
   const float *x = logits + row * C;
@@ -121,6 +138,9 @@ __global__ void __launch_bounds__(256)
     v[i] = floatx4u{ninf, ninf, ninf, ninf};
     if (c < C) v[i] = *reinterpret_cast<const floatx4u *>(x + c);
   }
+  const int j = (int)(row % Rr);
+  const int b = (int)(row / ((long)Rr * T));
+  const int64_t sym = row_symbol(symbols, ranges, row, b, j, S, term);
   float m = ninf;
 #pragma unroll
   for (int i = 0; i < kVecs; ++i)
@@ -135,13 +155,13 @@ __global__ void __launch_bounds__(256)
     for (int e = 0; e < 4; ++e) sum += __expf(v[i][e] - shift);  // padding is -inf: adds 0
   sum = wave_sum_all(sum);
   const float lse = logf(sum) + shift;
+  const float at_sym = (sym >= 0 && sym < C) ? row_entry<kVecs>(v, (int)sym) - lse
+                                             : std::numeric_limits<float>::quiet_NaN();
+  const float at_term = row_entry<kVecs>(v, term) - lse;
   if (lane == 0) {
-    const int j = (int)(row % Rr);
-    const int b = (int)(row / ((long)Rr * T));
-    const int64_t sym = row_symbol(symbols, ranges, row, b, j, S, term);
     norm[row] = lse;
-    xr[row] = (sym >= 0 && sym < C) ? x[sym] - lse : std::numeric_limits<float>::quiet_NaN();
-    yr[row] = x[term] - lse;
+    xr[row] = at_sym;
+    yr[row] = at_term;
   }
 }
 
