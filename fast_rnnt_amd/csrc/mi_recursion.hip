@@ -715,12 +715,15 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
         }
         R *d1dst = base + buf * kTileElems + r_first * kTilePitch + q;
         R *d2dst = d1dst + kBuffers * kTileElems;
-        // Which of the window's borders cross this tile (wave-uniform): reversed column 0,
-        // where rows start (local step = row); column 0, where they end; the top row.
-        const bool starts = m * kTileSteps <= kWave - 1;
-        const bool ends = m * kTileSteps + kTileSteps - 1 >= NT;
-        const int live = NS - g.row0;
-        const bool has_top = live <= kWave - 1;
+        // Only two borders of the window need care here.  Column 0 hands everything down
+        // (mutual_information_cpu.cu:219-226; nothing at all in the modified lattice) and
+        // the top row hands everything left (:228-235).  Everywhere else outside the
+        // window the sweep needs no zeros: cells a row passes before its first column keep
+        // a gradient of exactly 0 (nothing has reached them, and d1 / d2 are finite), and
+        // what is computed past column 0 or above the top row only feeds cells further
+        // out, none of which is stored or handed to another wave.
+        const int at_col0 = NT - m * kTileSteps;  // q - r of the cells in column 0
+        const int top_r = NS - g.row0;            // the top row, if it lies in this band
 #pragma unroll
         for (int u = 0; u < kRows; ++u) {
           const int r = r_first + kStep * u;
@@ -732,25 +735,8 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
           R d1 = Num<R>::exp_(term1 - total);
           R d2 = (R)1 - d1;
           if (d1 - d1 != 0) d1 = d2 = 0;
-          const int c = m * kTileSteps + q - r;
-          if (starts && c < 0) d1 = d2 = 0;
-          if (ends) {
-            // column 0 hands everything down (mutual_information_cpu.cu:219-226), or
-            // nothing at all in the modified lattice; beyond it nothing is defined
-            const int j = NT - c;
-            if (j <= 0) {
-              d1 = (j == 0 && !kModified) ? (R)1 : (R)0;
-              d2 = 0;
-            }
-          }
-          if (has_top) {
-            // the top row hands everything left (mutual_information_cpu.cu:228-235)
-            const int i = live - r;
-            if (i <= 0) {
-              d1 = 0;
-              d2 = (i == 0 && c >= 0 && c < NT) ? (R)1 : (R)0;
-            }
-          }
+          if (q - r == at_col0) d1 = kModified ? (R)0 : (R)1;
+          if (r == top_r) d2 = 1;
           d1dst[u * kStep * kTilePitch] = d1;
           d2dst[u * kStep * kTilePitch] = d2;
         }
