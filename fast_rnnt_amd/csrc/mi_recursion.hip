@@ -41,13 +41,20 @@ constexpr int kTilePitch = kTileSteps + 4;  // rows start 16-byte aligned and sp
 constexpr int kTileElems = kWave * kTilePitch;
 constexpr int kSeamPad = kChunk;        // slack on either side of a seam row, so that a whole
                                        // chunk of seam values is written without bounds tests
+// The slack on the left is a little longer: the last lane's chunk that starts at step e0
+// (a multiple of kChunk) goes to seam columns e0 - 63 ..., and with 11 elements of slack
+// their address is a multiple of 16 bytes, so that a chunk is two 16-byte LDS writes.
+constexpr int kSeamPadLeft = kSeamPad + 3;
+static_assert((kSeamPadLeft - (kWave - 1)) % 4 == 0, "seam chunks are not 16-byte aligned");
+constexpr int kSeamSlack = kSeamPadLeft + kSeamPad;
 constexpr int kFwdStagers = 2;         // staging waves per sweep wave
 constexpr int kBwdStagers = 3;
-// With at most two sweep waves the backward kernel runs 16 waves, the largest workgroup:
-// its staging waves evaluate d1 / d2 and are what the sweep waits for.  The forward
-// kernel's staging waves only copy, and more of them slow the sweep waves down (c2
-// shape: 21.4 us with 2, 22.2 with 5, 23.0 with 7 per sweep wave).
-constexpr int kBwdStagersFew = 7;
+// With at most two sweep waves the backward kernel runs more staging waves per sweep wave:
+// they evaluate d1 / d2 and are what the sweep would otherwise wait for (c2 shape: 22.9 us
+// with 3, 20.6 with 4, 19.3 - 19.6 with 5 to 7).  The forward kernel's staging waves only
+// copy, and more of them slow the sweep waves down (21.4 us with 2, 22.2 with 5, 23.0 with
+// 7 per sweep wave).
+constexpr int kBwdStagersFew = 6;
 constexpr int kSpinLimit = 1 << 22;
 
 struct Window {
@@ -251,7 +258,7 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
   const R *pyb = py + (size_t)b * (S + 1) * T;
   R *pb = p + (size_t)b * (S + 1) * TP;
   R *seam = reinterpret_cast<R *>(dyn_lds);
-  const int seam_pitch = (TP + 2 * kSeamPad + 3) & ~3;  // keeps the tiles 16-byte aligned
+  const int seam_pitch = (TP + kSeamSlack + 3) & ~3;  // keeps the tiles 16-byte aligned
   R *tiles = seam + (size_t)nsweep * seam_pitch;  // per sweep wave: kBuffers x tiles, then as many y tiles
   const int band_rows = kWave * nsweep;
 
@@ -384,8 +391,8 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
   // -------------------------------- sweep wave ---------------------------------
   const int w = wave;
   const int prev = (w + nsweep - 1) % nsweep;
-  R *my_seam = seam + (size_t)w * seam_pitch + kSeamPad;
-  const R *up_seam = seam + (size_t)prev * seam_pitch + kSeamPad;
+  R *my_seam = seam + (size_t)w * seam_pitch + kSeamPadLeft;
+  const R *up_seam = seam + (size_t)prev * seam_pitch + kSeamPadLeft;
   R *base = tiles + (size_t)w * 2 * kBuffers * kTileElems;
   int tile_base = 0, buf = 0;  // buf = tile number modulo kBuffers
   for (int band = 0; band * band_rows <= NS; ++band) {
@@ -480,9 +487,7 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
         // seam: the last lane's columns e0 - 63 ... (the pads take what falls outside)
         if (kDown && e0 + kChunk > kWave - 1) {
           if (lane == kWave - 1) {
-            R *sp = my_seam + (e0 - (kWave - 1));
-#pragma unroll
-            for (int k = 0; k < kChunk; ++k) sp[k] = vals[k];
+            push_chunk(my_seam + (e0 - (kWave - 1)), vals);
             const int done = max(0, min(e0 + kChunk - (kWave - 1), cols));
             publish_lds_writes(&cnt.ready[w], my_base + done);
           }
@@ -608,7 +613,7 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
   const R *pxb = px + (size_t)b * S * T1;
   const R *pb = p + (size_t)b * (S + 1) * TP;
   R *seam = reinterpret_cast<R *>(dyn_lds);
-  const int seam_pitch = (TP + 2 * kSeamPad + 3) & ~3;  // keeps the tiles 16-byte aligned
+  const int seam_pitch = (TP + kSeamSlack + 3) & ~3;  // keeps the tiles 16-byte aligned
   R *tiles = seam + (size_t)nsweep * seam_pitch;  // per sweep wave: kBuffers d1 tiles, then as many d2 tiles
   const int band_rows = kWave * nsweep;
 
@@ -771,8 +776,8 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
   // -------------------------------- sweep wave ---------------------------------
   const int w = wave;
   const int prev = (w + nsweep - 1) % nsweep;
-  R *my_seam = seam + (size_t)w * seam_pitch + kSeamPad;
-  const R *up_seam = seam + (size_t)prev * seam_pitch + kSeamPad;
+  R *my_seam = seam + (size_t)w * seam_pitch + kSeamPadLeft;
+  const R *up_seam = seam + (size_t)prev * seam_pitch + kSeamPadLeft;
   R *base = tiles + (size_t)w * 2 * kBuffers * kTileElems;
   const R seed = ans_grad ? ans_grad[b] : (R)1;
   int tile_base = 0, buf = 0;  // buf = tile number modulo kBuffers
@@ -866,9 +871,7 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
         // outside)
         if (kDown && e0 + kChunk > kWave - 1) {
           if (lane == kWave - 1) {
-            R *sp = my_seam + (e0 - (kWave - 1));
-#pragma unroll
-            for (int k = 0; k < kChunk; ++k) sp[k] = down[k];
+            push_chunk(my_seam + (e0 - (kWave - 1)), down);
             const int done = max(0, min(e0 + kChunk - (kWave - 1), cols));
             publish_lds_writes(&cnt.ready[w], my_base + done);
           }
@@ -911,7 +914,7 @@ int pick_sweep_waves(int S, int T, size_t elem, int arrays) {
   int n = (S + 1 + kWave - 1) / kWave;
   n = n < 1 ? 1 : (n > kMaxSweep ? kMaxSweep : n);
   auto bytes = [&](int k) {
-    return (size_t)k * ((size_t)((T + 1 + 2 * kSeamPad + 3) & ~3) + (size_t)arrays * 2 * kTileElems) * elem;
+    return (size_t)k * ((size_t)((T + 1 + kSeamSlack + 3) & ~3) + (size_t)arrays * 2 * kTileElems) * elem;
   };
   while (n > 1 && bytes(n) > kLdsBudget) --n;
   return n;
@@ -919,7 +922,7 @@ int pick_sweep_waves(int S, int T, size_t elem, int arrays) {
 
 // Dynamic LDS of a launch: per sweep wave a seam row and 2 x buffers tiles.
 size_t lds_bytes(int nsweep, int T, int buffers, size_t elem) {
-  return (size_t)nsweep * ((size_t)((T + 1 + 2 * kSeamPad + 3) & ~3) + (size_t)2 * buffers * kTileElems) * elem;
+  return (size_t)nsweep * ((size_t)((T + 1 + kSeamSlack + 3) & ~3) + (size_t)2 * buffers * kTileElems) * elem;
 }
 
 template <typename R>
@@ -970,7 +973,7 @@ int backward_impl(const R *px, const R *py, const int64_t *boundary, const R *p,
     return fail(FRNNT_ELIMIT, "mi_backward: T=%d needs %zu bytes of LDS", T, lds_bytes(n, T, 2, sizeof(R)));
   // With at most two sweep waves there is room for more staging waves per sweep wave and,
   // for floats, for a third tile buffer, which gives a staging wave two tiles' time instead
-  // of one to empty and refill a buffer.  (A workgroup of 16 waves leaves each 128
+  // of one to empty and refill a buffer.  (A workgroup of 14 waves leaves each 128
   // registers, too few for a sweep wave's two tile rows of doubles.)
   constexpr bool kFloat = sizeof(R) == 4;
   constexpr int kFew = kFloat ? kBwdStagersFew : kBwdStagers;
