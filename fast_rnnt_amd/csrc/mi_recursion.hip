@@ -13,12 +13,14 @@
 // px/py (forward) or p/px (backward) with coalesced, range-checked row loads, turn
 // them into diagonal ("sheared") 64-row x 32-step tiles in LDS and -- for the
 // backward sweep -- also evaluate the exp() of the gradient split; the sweep wave
-// pulls a tile into registers with 16-byte LDS reads.  Results leave the sweep wave
-// as 16-byte row segments through range-checked buffer stores (an out-of-window
-// lane's store is dropped by the hardware instead of being branched around).
-// Tiles are double buffered; sweep and staging waves meet only through monotone
-// LDS counters (acquire/release, bounded spinning), never at a barrier, and the
-// sweep wave looks at a counter one chunk (one tile) before it needs it.
+// pulls a tile into registers with 16-byte LDS reads and leaves the tile's results
+// in the same LDS buffer with 16-byte writes.  The staging waves carry the results
+// to memory as coalesced row segments through range-checked buffer stores (a cell
+// outside the window gets an offset that the hardware drops instead of a branch)
+// before they refill the buffer.  There are two or three buffers per sweep wave;
+// sweep and staging waves meet only through monotone LDS counters (bounded
+// spinning), never at a barrier, and the sweep wave looks at a counter one chunk
+// (one tile) before it needs it.
 //
 // Rows beyond 64 go to further sweep waves; wave w+1 consumes the last row of
 // wave w through an LDS seam row guarded by a progress counter and simply runs a
@@ -123,7 +125,7 @@ __device__ __forceinline__ float chain_log_add(float a, float c) {
 }
 __device__ __forceinline__ double chain_log_add(double a, double c) { return log_add(a, c); }
 
-// Results leave the sweep waves through raw buffer stores: the resource covers one
+// Results go to memory through raw buffer stores: the resource covers one
 // utterance's array, a lane passes a byte offset, and an offset of kDropped lies
 // outside every resource, so the hardware's range check discards the store.  That
 // turns "this lane has nothing to write here" into one select on the offset, with
