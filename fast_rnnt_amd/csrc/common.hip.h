@@ -86,6 +86,17 @@ __device__ __forceinline__ double from_lane_below_or(double v, double first) {
   return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
 }
 
+// The value one lane holds, for all lanes (the lane index is wave-uniform).
+__device__ __forceinline__ float read_lane(float v, int lane) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+__device__ __forceinline__ double read_lane(double v, int lane) {
+  const long long vi = __double_as_longlong(v);
+  const int lo = __builtin_amdgcn_readlane((int)(vi & 0xffffffffLL), lane);
+  const int hi = __builtin_amdgcn_readlane((int)(vi >> 32), lane);
+  return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+
 // Value held by lane+1 (whole-wave shift left by one, DPP wave_shl:1); lane 63 receives 0.
 __device__ __forceinline__ float from_lane_above(float v) {
   return __int_as_float(

@@ -185,7 +185,8 @@ __global__ void __launch_bounds__(256)
 // adjoint: one block per lm row (b, s).  The block first lists, in order, the entries
 // of ranges[b] that point at s (an ordered compaction through LDS; only a few dozen of
 // the T * R entries match), then sums those rows of the incoming gradient -- in that
-// order, so the result is deterministic -- with coalesced loads.  For the listing a
+// order (shared out over the block's waves in a fixed way), so the result is
+// deterministic -- with coalesced loads.  For the listing a
 // thread takes kScanPerThread consecutive entries (all requested at once), and one
 // prefix sum over the threads' counts places everybody's matches.
 constexpr int kHitCapacity = 4096;   // matches listed per round
@@ -198,6 +199,7 @@ __global__ void __launch_bounds__(256)
                          R *__restrict__ lm_grad, int TR, int S1, int C) {
   __shared__ int hits[kHitCapacity];
   __shared__ int wave_count[4];
+  __shared__ __align__(16) float meet[4 * 512];  // the four waves' sums of 512 columns
   const int b = blockIdx.x / S1, s = blockIdx.x % S1;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t *rb = ranges + (long)b * TR;
@@ -244,28 +246,66 @@ __global__ void __launch_bounds__(256)
     k_next = k0;
     __syncthreads();
     const int n = listed;
-    for (int c0 = 0; c0 < C; c0 += 256) {
-      const int c = c0 + tid;
-      if (c >= C) continue;
-      R acc = first_round ? (R)0 : dst[c];
-      int i = 0;
-      for (; i + 8 <= n; i += 8) {
-        R g[8];
+    if (sizeof(R) == 4 && C % 4 == 0) {
+      // The four waves share the listed rows (wave w takes rows w, w + 4, ...), a lane
+      // reads 16 bytes of a row at a time, two stretches of 256 columns and four rows
+      // per request round; the waves' sums meet in LDS in a fixed order.
+      typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
+      const float *gf = reinterpret_cast<const float *>(gb);
+      float *df = reinterpret_cast<float *>(dst);
+      f4 *meet4 = reinterpret_cast<f4 *>(meet);
+      for (int c0 = 0; c0 < C; c0 += 512) {
+        const int ca = c0 + 4 * lane, cb = ca + 256;
+        f4 a = {0, 0, 0, 0}, b2 = {0, 0, 0, 0};
+        for (int i = wave; i < n; i += 16) {
+          f4 va[4], vb[4];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) g[u] = gb[(long)hits[i + u] * C + c];
+          for (int u = 0; u < 4; ++u) {
+            const int at = i + 4 * u;
+            const float *row = gf + (long)hits[at < n ? at : i] * C;
+            va[u] = (at < n && ca < C) ? *reinterpret_cast<const f4 *>(row + ca) : f4{0, 0, 0, 0};
+            vb[u] = (at < n && cb < C) ? *reinterpret_cast<const f4 *>(row + cb) : f4{0, 0, 0, 0};
+          }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) acc += g[u];
+          for (int u = 0; u < 4; ++u) a += va[u], b2 += vb[u];
+        }
+        meet4[wave * 128 + lane] = a;
+        meet4[wave * 128 + 64 + lane] = b2;
+        __syncthreads();
+        if (tid < 128) {
+          const int c = c0 + 4 * tid;
+          if (c < C) {
+            f4 sum = (meet4[tid] + meet4[128 + tid]) + (meet4[256 + tid] + meet4[384 + tid]);
+            if (!first_round) sum += *reinterpret_cast<const f4 *>(df + c);
+            *reinterpret_cast<f4 *>(df + c) = sum;
+          }
+        }
+        __syncthreads();
       }
-      if (i + 4 <= n) {
-        R g[4];
+    } else {
+      for (int c0 = 0; c0 < C; c0 += 256) {
+        const int c = c0 + tid;
+        if (c >= C) continue;
+        R acc = first_round ? (R)0 : dst[c];
+        int i = 0;
+        for (; i + 8 <= n; i += 8) {
+          R g[8];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) g[u] = gb[(long)hits[i + u] * C + c];
+          for (int u = 0; u < 8; ++u) g[u] = gb[(long)hits[i + u] * C + c];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) acc += g[u];
-        i += 4;
+          for (int u = 0; u < 8; ++u) acc += g[u];
+        }
+        if (i + 4 <= n) {
+          R g[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) g[u] = gb[(long)hits[i + u] * C + c];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) acc += g[u];
+          i += 4;
+        }
+        for (; i < n; ++i) acc += gb[(long)hits[i] * C + c];
+        dst[c] = acc;
       }
-      for (; i < n; ++i) acc += gb[(long)hits[i] * C + c];
-      dst[c] = acc;
     }
     first_round = false;
     __syncthreads();

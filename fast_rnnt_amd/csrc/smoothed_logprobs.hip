@@ -329,18 +329,26 @@ __global__ void __launch_bounds__(256)
     for (int i = first; i < last; ++i)
       if (pair_sym[i] == c) direct += pair_x[i];
   }
-  if (c == term) {
-    const int share = (n + kRowGroups - 1) / kRowGroups;
-    const int first = grp * share, last = min(first + share, n);
-    int row = first;
-    for (; row + 8 <= last; row += 8) {
+  // the termination symbol's column also takes the sum of row_y over all rows: the whole
+  // block adds it up (every thread a strided share, eight loads in flight, then a fixed
+  // tree), not the sixteen threads of that column alone
+  if (term / kColsPerBlock == (int)blockIdx.x) {  // (uniform)
+    R part = 0;
+    for (int row0 = threadIdx.x; row0 < n; row0 += 8 * 256) {
       R v[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = row_y[row + u];
+      for (int u = 0; u < 8; ++u) v[u] = row0 + u * 256 < n ? row_y[row0 + u * 256] : (R)0;
 #pragma unroll
-      for (int u = 0; u < 8; ++u) direct += v[u];
+      for (int u = 0; u < 8; ++u) part += v[u];
     }
-    for (; row < last; ++row) direct += row_y[row];
+    __syncthreads();  // pair_x is free now
+    pair_x[threadIdx.x] = part;
+    __syncthreads();
+    for (int off = 128; off > 0; off >>= 1) {
+      if ((int)threadIdx.x < off) pair_x[threadIdx.x] += pair_x[threadIdx.x + off];
+      __syncthreads();
+    }
+    if (c == term && grp == 0) direct += pair_x[0];
   }
   acc = sum_of_groups(acc, meet, col, grp);
   __syncthreads();
@@ -421,6 +429,79 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// The am row kernel with the per-symbol terms folded in:
+// am_grad[b,t,sym[b,s]] += a * gx[b,s,t] for every s.  A wave keeps a row of C sums in
+// LDS.  Lane l holds the symbols and the frame's gx of rows l, l + 64, ... (one strided
+// load per 64 rows).  An integer LDS minimum per symbol names the first row that carries
+// it; those rows write their gx side by side (one writer per column), and the few rows
+// whose symbol occurred before add theirs afterwards one at a time, in the order of s --
+// LDS carries out a wave's instructions in order, so the sum is always formed the same
+// way.  That replaces a second pass that had to read, modify and write one cache line of
+// am_grad per (b, s, t).
+constexpr int kSymRowsPerLane = 4;  // up to 256 symbols per utterance
+template <typename R>
+__global__ void __launch_bounds__(256)
+    smoothed_bwd_am_sym_kernel(const R *__restrict__ am, const R *__restrict__ am_max,
+                               const R *__restrict__ am_z, const R *__restrict__ unigram,
+                               const R *__restrict__ col_y, const R *__restrict__ col_g,
+                               const R *__restrict__ gpx, const int64_t *__restrict__ symbols,
+                               R *__restrict__ am_grad, long rows, int S, int T, int T1, int C,
+                               int term, R k_am) {
+  extern __shared__ __align__(16) unsigned char sym_lds[];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // in a scalar register
+  const long row = (long)blockIdx.x * 4 + wave;
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  R *extra = reinterpret_cast<R *>(sym_lds) + (size_t)wave * C;
+  int *first = reinterpret_cast<int *>(sym_lds + (size_t)4 * C * sizeof(R)) + (size_t)wave * C;
+  const int b = (int)(row / T), t = (int)(row % T);
+  int sym[kSymRowsPerLane];
+  R gx[kSymRowsPerLane];
+#pragma unroll
+  for (int q = 0; q < kSymRowsPerLane; ++q) {
+    const int s = q * kWave + lane;
+    const int64_t y = s < S ? symbols[(long)b * S + s] : -1;
+    sym[q] = (y >= 0 && y < C) ? (int)y : -1;
+    gx[q] = s < S ? gpx[((long)b * S + s) * T1 + t] : (R)0;
+  }
+  for (int c = lane; c < C; c += kWave) {
+    extra[c] = 0;
+    first[c] = 0x7fffffff;
+  }
+#pragma unroll
+  for (int q = 0; q < kSymRowsPerLane; ++q)
+    if (q * kWave < S && sym[q] >= 0) atomicMin(&first[sym[q]], q * kWave + lane);
+  bool later[kSymRowsPerLane];
+#pragma unroll
+  for (int q = 0; q < kSymRowsPerLane; ++q) {
+    later[q] = false;
+    if (q * kWave < S && sym[q] >= 0) {
+      later[q] = first[sym[q]] != q * kWave + lane;
+      if (!later[q]) extra[sym[q]] = gx[q];
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < kSymRowsPerLane; ++q) {
+    if (q * kWave >= S) break;
+    unsigned long long todo = __ballot(later[q]);
+    while (todo) {
+      const int i = __ffsll((long long)todo) - 1;
+      if (lane == i) extra[sym[q]] += gx[q];
+      todo &= todo - 1;
+    }
+  }
+  const R *x = am + row * C;
+  const R m = am_max[row];
+  const R w = -k_am * col_g[row] / am_z[row];
+  const R cy = k_am * col_y[row];
+  R *g = am_grad + row * C;
+  for (int c = lane; c < C; c += kWave) {
+    R v = w * Num<R>::exp_(x[c] - m) * unigram[c];
+    if (c == term) v += cy;
+    g[c] = v + k_am * extra[c];
+  }
+}
+
 template <typename R>
 int fwd_impl(const R *lm, const R *am, const int64_t *symbols, const R *pxj, const R *pyj, R *px,
              R *py, R *lm_max, R *lm_sum, R *am_max, R *am_z, R *unigram, R *partial, int B, int S,
@@ -490,11 +571,21 @@ int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const R *lm_max, 
                      stream, lm, symbols, lm_max, lm_sum, row_x, row_y, g_unigram, lm_grad, n_lm, S, C,
                      term, k_lm, (R)(1.0 / (double)n_lm));
   if (n_am > 0) {
-    hipLaunchKernelGGL(smoothed_bwd_am_kernel<R>, dim3((unsigned)((n_am + 3) / 4)), dim3(256), 0,
-                       stream, am, am_max, am_z, unigram, col_y, col_g, am_grad, n_am, C, term, k_am);
-    if (S > 0)
-      hipLaunchKernelGGL(smoothed_bwd_symbols_kernel<R>, dim3((unsigned)(B * S)), dim3(256), 0,
-                         stream, px_grad, symbols, am_grad, S, T, T1, C, k_am);
+    // one row of sums and one of row numbers per wave in LDS, when that fits
+    const size_t sym_lds = (size_t)4 * C * (sizeof(R) + sizeof(int));
+    if (S > 0 && S <= kSymRowsPerLane * kWave && sym_lds <= 64 * 1024 &&
+        allow_lds(reinterpret_cast<const void *>(smoothed_bwd_am_sym_kernel<R>), sym_lds)) {
+      hipLaunchKernelGGL(smoothed_bwd_am_sym_kernel<R>, dim3((unsigned)((n_am + 3) / 4)), dim3(256),
+                         sym_lds, stream, am, am_max, am_z, unigram, col_y, col_g, px_grad, symbols,
+                         am_grad, n_am, S, T, T1, C, term, k_am);
+    } else {
+      hipLaunchKernelGGL(smoothed_bwd_am_kernel<R>, dim3((unsigned)((n_am + 3) / 4)), dim3(256), 0,
+                         stream, am, am_max, am_z, unigram, col_y, col_g, am_grad, n_am, C, term,
+                         k_am);
+      if (S > 0)
+        hipLaunchKernelGGL(smoothed_bwd_symbols_kernel<R>, dim3((unsigned)(B * S)), dim3(256), 0,
+                           stream, px_grad, symbols, am_grad, S, T, T1, C, k_am);
+    }
   }
   return check_launch("smoothed_logprobs_bwd");
 }
