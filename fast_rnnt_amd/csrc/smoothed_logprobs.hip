@@ -113,11 +113,13 @@ __global__ void __launch_bounds__(256)
 }
 
 // The reductions over all rows of the batch end in a sum per vocabulary entry.  A block
-// of 256 threads takes 16 entries: 16 groups of 16 threads, every group walks its share
-// of the rows (64-byte reads), and the groups' sums meet in LDS in a fixed order, so the
-// result does not depend on timing.
+// of 1024 threads takes 16 entries: 64 groups of 16 threads, every group walks its share
+// of the rows (64-byte reads, eight in flight: with some hundred rows a single request
+// round), and the groups' sums meet in LDS in a fixed order, so the result does not
+// depend on timing.
 constexpr int kColsPerBlock = 16;
-constexpr int kRowGroups = 16;
+constexpr int kRowGroups = 64;
+constexpr int kUnigramThreads = kColsPerBlock * kRowGroups;
 
 template <typename R>
 __device__ __forceinline__ R sum_of_groups(R mine, R (*meet)[kColsPerBlock], int col, int grp) {
@@ -136,20 +138,20 @@ __device__ __forceinline__ R sum_partials(const R *__restrict__ partial, int blo
                                           int grp) {
   R acc = 0;
   int k = grp;
-  for (; k + 7 * kRowGroups < blocks; k += 8 * kRowGroups) {
+  for (; k < blocks; k += 8 * kRowGroups) {
     R v[8];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) v[u] = partial[(long)(k + u * kRowGroups) * C + c];
+    for (int u = 0; u < 8; ++u)
+      v[u] = k + u * kRowGroups < blocks ? partial[(long)(k + u * kRowGroups) * C + c] : (R)0;
 #pragma unroll
     for (int u = 0; u < 8; ++u) acc += v[u];
   }
-  for (; k < blocks; k += kRowGroups) acc += partial[(long)k * C + c];
   return acc;
 }
 
 // unigram[c] = (sum of the partials) / N + tiny
 template <typename R>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(kUnigramThreads)
     unigram_final_kernel(const R *__restrict__ partial, R *__restrict__ unigram, int blocks, long N,
                          int C) {
   __shared__ R meet[kRowGroups][kColsPerBlock];
@@ -302,7 +304,7 @@ __global__ void __launch_bounds__(256)
 constexpr int kPairChunk = 2048;
 
 template <typename R>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(kUnigramThreads)
     unigram_grad_kernel(const R *__restrict__ partial, const int64_t *__restrict__ symbols,
                         const R *__restrict__ row_x, const R *__restrict__ row_y,
                         const R *__restrict__ unigram, R *__restrict__ g_unigram, int blocks,
@@ -317,7 +319,7 @@ __global__ void __launch_bounds__(256)
   for (int row0 = 0; row0 < n; row0 += kPairChunk) {
     const int count = min(kPairChunk, n - row0);
     __syncthreads();
-    for (int i = threadIdx.x; i < count; i += 256) {
+    for (int i = threadIdx.x; i < count; i += kUnigramThreads) {
       const int row = row0 + i, b = row / S1, s = row - b * S1;
       const int64_t y = s < S ? symbols[(long)b * S + s] : -1;
       pair_sym[i] = (y >= 0 && y < C) ? (int)y : -1;
@@ -334,17 +336,18 @@ __global__ void __launch_bounds__(256)
   // tree), not the sixteen threads of that column alone
   if (term / kColsPerBlock == (int)blockIdx.x) {  // (uniform)
     R part = 0;
-    for (int row0 = threadIdx.x; row0 < n; row0 += 8 * 256) {
+    for (int row0 = threadIdx.x; row0 < n; row0 += 8 * kUnigramThreads) {
       R v[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = row0 + u * 256 < n ? row_y[row0 + u * 256] : (R)0;
+      for (int u = 0; u < 8; ++u)
+        v[u] = row0 + u * kUnigramThreads < n ? row_y[row0 + u * kUnigramThreads] : (R)0;
 #pragma unroll
       for (int u = 0; u < 8; ++u) part += v[u];
     }
     __syncthreads();  // pair_x is free now
     pair_x[threadIdx.x] = part;
     __syncthreads();
-    for (int off = 128; off > 0; off >>= 1) {
+    for (int off = kUnigramThreads / 2; off > 0; off >>= 1) {
       if ((int)threadIdx.x < off) pair_x[threadIdx.x] += pair_x[threadIdx.x + off];
       __syncthreads();
     }
@@ -521,7 +524,7 @@ int fwd_impl(const R *lm, const R *am, const int64_t *symbols, const R *pxj, con
                      lm, lm_max, lm_sum, n_lm, C);
   hipLaunchKernelGGL(weighted_column_partial_kernel<R>, dim3(blocks), dim3(256), 0, stream, lm,
                      lm_max, (const R *)nullptr, lm_sum, partial, n_lm, C);
-  hipLaunchKernelGGL(unigram_final_kernel<R>, dim3((C + kColsPerBlock - 1) / kColsPerBlock), dim3(256), 0, stream, partial,
+  hipLaunchKernelGGL(unigram_final_kernel<R>, dim3((C + kColsPerBlock - 1) / kColsPerBlock), dim3(kUnigramThreads), 0, stream, partial,
                      unigram, blocks, n_lm, C);
   if (n_am > 0)
     hipLaunchKernelGGL(am_row_stats_kernel<R>, dim3((unsigned)((n_am + 3) / 4)), dim3(256), 0,
@@ -564,7 +567,7 @@ int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const R *lm_max, 
   if (n_am > 0)
     hipLaunchKernelGGL(weighted_column_partial_kernel<R>, dim3(blocks), dim3(256), 0, stream, am,
                        am_max, col_g, am_z, partial, n_am, C);
-  hipLaunchKernelGGL(unigram_grad_kernel<R>, dim3((C + kColsPerBlock - 1) / kColsPerBlock), dim3(256), 0, stream, partial,
+  hipLaunchKernelGGL(unigram_grad_kernel<R>, dim3((C + kColsPerBlock - 1) / kColsPerBlock), dim3(kUnigramThreads), 0, stream, partial,
                      symbols, row_x, row_y, unigram, g_unigram, n_am > 0 ? blocks : 0, B, S, C, term,
                      k_am);
   hipLaunchKernelGGL(smoothed_bwd_lm_kernel<R>, dim3((unsigned)((n_lm + 3) / 4)), dim3(256), 0,
