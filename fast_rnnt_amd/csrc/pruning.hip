@@ -182,6 +182,38 @@ __global__ void __launch_bounds__(256)
   for (int c = lane; c < C; c += kWave) dst[c] = src[c];
 }
 
+// The same for rows of 4-byte elements whose length is a multiple of 4 (at most
+// 256 * kVecs): the whole row is requested at once, 16 bytes per lane and load, and
+// leaves as 16-byte stores.
+typedef int words4 __attribute__((ext_vector_type(4), aligned(4)));
+template <int kVecs>
+__global__ void __launch_bounds__(256)
+    prune_gather_vec_kernel(const int *__restrict__ lm, const int64_t *__restrict__ ranges,
+                            int *__restrict__ out, long rows, int TR, int S1, int C) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // in a scalar register
+  const long row = (long)blockIdx.x * 4 + wave;
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const long b = row / TR;
+  const int64_t s = ranges[row];
+  const bool valid = s >= 0 && s < S1;
+  const int *src = lm + (b * S1 + (valid ? s : 0)) * C;
+  const int nan_bits = 0x7fc00000;
+  words4 v[kVecs];
+#pragma unroll
+  for (int i = 0; i < kVecs; ++i) {
+    const int c = 4 * (lane + kWave * i);
+    v[i] = words4{nan_bits, nan_bits, nan_bits, nan_bits};
+    if (valid && c < C) v[i] = *reinterpret_cast<const words4 *>(src + c);
+  }
+  int *dst = out + row * C;
+#pragma unroll
+  for (int i = 0; i < kVecs; ++i) {
+    const int c = 4 * (lane + kWave * i);
+    if (c < C) *reinterpret_cast<words4 *>(dst + c) = v[i];
+  }
+}
+
 // adjoint: one block per lm row (b, s).  The block first lists, in order, the entries
 // of ranges[b] that point at s (an ordered compaction through LDS; only a few dozen of
 // the T * R entries match), then sums those rows of the incoming gradient -- in that
@@ -349,8 +381,28 @@ int gather_impl(const R *lm, const int64_t *ranges, R *out, int B, int S, int T,
   const long rows = (long)B * T * Rr;
   if (rows == 0 || C == 0) return FRNNT_OK;
   if (!lm || !ranges || !out) return fail(FRNNT_EINVAL, "prune_gather: null pointer");
-  hipLaunchKernelGGL(prune_gather_kernel<R>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), lm, ranges, out, rows, T * Rr, S + 1, C);
+  const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+  if (sizeof(R) == 4 && C % 4 == 0 && C <= 256 * 16) {
+    const int *src = reinterpret_cast<const int *>(lm);
+    int *dst = reinterpret_cast<int *>(out);
+#define FRNNT_GATHER(V)                                                                          \
+  hipLaunchKernelGGL(prune_gather_vec_kernel<V>, grid, block, 0, static_cast<hipStream_t>(stream), \
+                     src, ranges, dst, rows, T * Rr, S + 1, C)
+    if (C <= 256)
+      FRNNT_GATHER(1);
+    else if (C <= 512)
+      FRNNT_GATHER(2);
+    else if (C <= 1024)
+      FRNNT_GATHER(4);
+    else if (C <= 2048)
+      FRNNT_GATHER(8);
+    else
+      FRNNT_GATHER(16);
+#undef FRNNT_GATHER
+  } else {
+    hipLaunchKernelGGL(prune_gather_kernel<R>, grid, block, 0, static_cast<hipStream_t>(stream), lm,
+                       ranges, out, rows, T * Rr, S + 1, C);
+  }
   return check_launch("prune_gather");
 }
 
