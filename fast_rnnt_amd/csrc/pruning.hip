@@ -224,6 +224,8 @@ __global__ void __launch_bounds__(256)
 constexpr int kHitCapacity = 4096;   // matches listed per round
 constexpr int kScanPerThread = 8;
 constexpr int kScanChunk = 256 * kScanPerThread;
+// a round must be able to take a whole chunk of matches, or it would make no progress
+static_assert(kHitCapacity >= kScanChunk, "a chunk of matches must fit in the list");
 
 template <typename R>
 __global__ void __launch_bounds__(256)
@@ -278,12 +280,23 @@ __global__ void __launch_bounds__(256)
     k_next = k0;
     __syncthreads();
     const int n = listed;
-    if (sizeof(R) == 4 && C % 4 == 0) {
+    if (sizeof(R) == 4 && C % 4 == 0 && (long)TR * C * 4 < (1L << 31)) {
       // The four waves share the listed rows (wave w takes rows w, w + 4, ...), a lane
       // reads 16 bytes of a row at a time, two stretches of 256 columns and four rows
       // per request round; the waves' sums meet in LDS in a fixed order.
+      // Loads go through a buffer resource over the utterance's gradient rows: a lane
+      // with nothing to read passes an offset outside it and gets 0 -- no branch around
+      // the load, so that all loads of a round are in flight together.
       typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
-      const float *gf = reinterpret_cast<const float *>(gb);
+      typedef int intx4 __attribute__((ext_vector_type(4)));
+      const __amdgpu_buffer_rsrc_t g_rs = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<float *>(reinterpret_cast<const float *>(gb)), 0, TR * C * 4, 0x00020000);
+      constexpr int kNowhere = (int)0x80000000;
+      auto row_piece = [&](int byte_offset) {
+        const intx4 w = __builtin_amdgcn_raw_buffer_load_b128(g_rs, byte_offset, 0, 0);
+        return f4{__int_as_float(w[0]), __int_as_float(w[1]), __int_as_float(w[2]),
+                  __int_as_float(w[3])};
+      };
       float *df = reinterpret_cast<float *>(dst);
       f4 *meet4 = reinterpret_cast<f4 *>(meet);
       for (int c0 = 0; c0 < C; c0 += 512) {
@@ -294,9 +307,9 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
           for (int u = 0; u < 4; ++u) {
             const int at = i + 4 * u;
-            const float *row = gf + (long)hits[at < n ? at : i] * C;
-            va[u] = (at < n && ca < C) ? *reinterpret_cast<const f4 *>(row + ca) : f4{0, 0, 0, 0};
-            vb[u] = (at < n && cb < C) ? *reinterpret_cast<const f4 *>(row + cb) : f4{0, 0, 0, 0};
+            const int row = hits[at < n ? at : i] * C * 4;  // byte offset of the row
+            va[u] = row_piece((at < n && ca < C) ? row + ca * 4 : kNowhere);
+            vb[u] = row_piece((at < n && cb < C) ? row + cb * 4 : kNowhere);
           }
 #pragma unroll
           for (int u = 0; u < 4; ++u) a += va[u], b2 += vb[u];
