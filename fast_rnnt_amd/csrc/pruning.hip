@@ -108,10 +108,27 @@ __global__ void __launch_bounds__(256)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int b = blockIdx.y, t = blockIdx.x * kWave + lane;
   const bool ok = t < T;
-  const R *gx = px_grad + (long)b * S * T1 + t;
-  const R *gy = py_grad + (long)b * (S + 1) * T + t;
-  for (int s = wave; s <= S; s += 4) ty[s * kWave + lane] = ok ? gy[(long)s * T] : (R)0;
-  for (int s = wave; s < S; s += 4) tx[s * kWave + lane] = ok ? gx[(long)s * T1] : (R)0;
+  // (a frame past the end reads the last frame's column: no branch around the loads, so
+  // that eight rows are requested before the first is stored)
+  const int t_read = ok ? t : T - 1;
+  const R *gx = px_grad + (long)b * S * T1 + t_read;
+  const R *gy = py_grad + (long)b * (S + 1) * T + t_read;
+  for (int s0 = wave; s0 <= S; s0 += 32) {
+    R v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = gy[(long)min(s0 + 4 * u, S) * T];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (s0 + 4 * u <= S) ty[(s0 + 4 * u) * kWave + lane] = ok ? v[u] : (R)0;
+  }
+  for (int s0 = wave; s0 < S; s0 += 32) {
+    R v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = gx[(long)min(s0 + 4 * u, S - 1) * T1];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (s0 + 4 * u < S) tx[(s0 + 4 * u) * kWave + lane] = ok ? v[u] : (R)0;
+  }
   __syncthreads();
   const int n = S + 2 - Rr;  // candidate window starts
   const int per = (n + 3) / 4, lo = wave * per, hi = min(n, lo + per);
