@@ -286,6 +286,25 @@ def test_smoothed_gradients(gpu_device, kind):
     assert _close(da.grad, a.grad, 1e-6, 1e-6) and _close(dl.grad, l.grad, 1e-6, 1e-6)
 
 
+@pytest.mark.parametrize("S", [70, 130, 300])
+def test_smoothed_gradients_long_targets(gpu_device, S):
+    # more lattice rows than one wave holds (and, at 300, more than the fused am-gradient
+    # kernel takes), few symbols, so that most of them occur many times
+    dev = gpu_device
+    am, lm, sym, bnd = _case(210 + S, 2, S, S + 20, 13, torch.float64, "regular")
+    a = am.clone().requires_grad_(True)
+    l = lm.clone().requires_grad_(True)
+    want = O.loss_smoothed(l, a, sym, 3, 0.1, 0.3, boundary=bnd, rnnt_type="regular", reduction="sum")
+    want.backward()
+    da = am.to(dev).requires_grad_(True)
+    dl = lm.to(dev).requires_grad_(True)
+    got = fast_rnnt_amd.rnnt_loss_smoothed(dl, da, sym.to(dev), 3, 0.1, 0.3, boundary=bnd.to(dev),
+                                           rnnt_type="regular", reduction="sum")
+    got.backward()
+    assert _close(got, want, 0.0, 1e-9)
+    assert _close(da.grad, a.grad, 1e-8, 1e-8) and _close(dl.grad, l.grad, 1e-8, 1e-8)
+
+
 def test_small_s_range_never_gives_inf(gpu_device):
     # fast_rnnt/python/tests/rnnt_loss_test.py:615-705: T = 1, s_range raised to its minimum
     dev = gpu_device
