@@ -30,9 +30,9 @@ FP32_MFMA_PEAK_TFLOPS = 157.3
 # profiles/ (FETCH_SIZE and WRITE_SIZE, scaled by what the same counters read for a
 # copy of known size); filled in for the workloads that were profiled
 MEASURED_TRAFFIC = {
-    ("c2", "simple_fwd_panel_kernel<96, 16>"): 29257200,
-    ("c2", "mi_forward_kernel<float, false, 2, 2, 3>"): 6732627,
-    ("c2", "mi_backward_kernel<float, false, 2, 6, 3>"): 9667864,
+    ("c2", "simple_fwd_panel_kernel<96, 16>"): 29256606,
+    ("c2", "mi_forward_kernel<float, false, 2, 2, 3>"): 6732770,
+    ("c2", "mi_backward_kernel<float, false, 2, 6, 3>"): 9667752,
 }
 
 
@@ -375,7 +375,7 @@ def main():
             "loss_rel_diff_vs_gpu": abs(gpu_loss - cpu_loss.item()) / abs(cpu_loss.item()),
         }
 
-    # The step is eight kernels of 4-25 us.  An eager loop of nothing but this call is bound by
+    # The step is seven kernels of 4-36 us.  An eager loop of nothing but this call is bound by
     # the host's launch work on slow hosts (in training that work hides behind the model's own
     # kernels); the replayed graph of the same step -- same kernels, outputs checked bit-equal
     # against eager steps -- does not depend on the host, but its nodes start a little further

@@ -16,12 +16,14 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 // All tiles of batch element b run on XCD b % 8, so one XCD's L2 holds the operands
 // of only B/8 utterances.  The grid must have kXcds * ceil(B / kXcds) * tiles
 // workgroups; returns false for the padding ones.
-__device__ __forceinline__ bool decode_block(int tiles, int B, int &b, int &tile) {
-  const int id = blockIdx.x;
+__device__ __forceinline__ bool decode_block(int id, int tiles, int B, int &b, int &tile) {
   const int xcd = id % kXcds, slot = id / kXcds;
   b = xcd + kXcds * (slot / tiles);
   tile = slot % tiles;
   return b < B;
+}
+__device__ __forceinline__ bool decode_block(int tiles, int B, int &b, int &tile) {
+  return decode_block((int)blockIdx.x, tiles, B, b, tile);
 }
 inline unsigned xcd_grid(int tiles, int B) {
   return (unsigned)(kXcds * ((B + kXcds - 1) / kXcds) * tiles);
