@@ -33,6 +33,7 @@ MEASURED_TRAFFIC = {
     ("c2", "simple_fwd_panel_kernel<96, 16>"): 29256606,
     ("c2", "mi_forward_kernel<float, false, 2, 2, 3>"): 6732770,
     ("c2", "mi_backward_kernel<float, false, 2, 6, 3>"): 9667752,
+    ("c2", "simple_bwd_am_lm_kernel<96, 32>"): 59671565,
 }
 
 
@@ -305,7 +306,42 @@ def main():
         t_logp = _event_time_ms(
             lambda: fast_rnnt_amd.get_rnnt_logprobs(lm, am, sym, 0, boundary=bnd),
             args.kernel_reps)
-    stages = {"mi_forward_ms": t_fwd, "mi_backward_ms": t_bwd, "logprobs_fwd_ms": t_logp}
+        # The two gradient products (lm.grad, am.grad) through the backward entry point of
+        # the logprobs: it also launches the small prep kernel, which the same call without
+        # outputs runs alone; the difference of the two event timings is the product kernel(s).
+        C = w.C
+        f32 = dict(dtype=torch.float32, device=dev)
+        lm_c, am_c = lm.detach().contiguous(), am.detach().contiguous()
+        lm_max, am_max = torch.empty(B, S + 1, **f32), torch.empty(B, T, **f32)
+        norm_raw = torch.empty(B, S + 1, T, **f32)
+        stream = torch.cuda.current_stream().cuda_stream
+        _lib.call("frnnt_simple_logprobs_fwd_f32", lm_c.data_ptr(), am_c.data_ptr(), sym.data_ptr(),
+                  bnd.data_ptr(), px.data_ptr(), py.data_ptr(), lm_max.data_ptr(), am_max.data_ptr(),
+                  norm_raw.data_ptr(), B, S, T, C, 0, 0, stream)
+        gpx, gpy = torch.rand_like(px), torch.rand_like(py)
+        dmat = torch.empty(B, S + 1, (T + 3) // 4 * 4, **f32)
+        row_x, row_y = torch.empty(B, S + 1, **f32), torch.empty(B, S + 1, **f32)
+        col_y = torch.empty(B, T, **f32)
+        lm_grad, am_grad = torch.empty_like(lm_c), torch.empty_like(am_c)
+
+        def grads(want_lm, want_am):
+            _lib.call("frnnt_simple_logprobs_bwd_f32", lm_c.data_ptr(), am_c.data_ptr(),
+                      sym.data_ptr(), bnd.data_ptr(), lm_max.data_ptr(), am_max.data_ptr(),
+                      norm_raw.data_ptr(), None, 0, 1.0, gpx.data_ptr(), gpy.data_ptr(),
+                      dmat.data_ptr(), row_x.data_ptr(), row_y.data_ptr(), col_y.data_ptr(),
+                      lm_grad.data_ptr() if want_lm else None,
+                      am_grad.data_ptr() if want_am else None, B, S, T, C, 0, 0, stream)
+
+        t_prep = _event_time_ms(lambda: grads(False, False), args.kernel_reps)
+        one_launch = float(B) * (S + 1) * T * C < 1e9  # the library's rule for a single launch
+        if one_launch:
+            t_grads = {"both": _event_time_ms(lambda: grads(True, True), args.kernel_reps) - t_prep}
+        else:
+            t_grads = {"lm": _event_time_ms(lambda: grads(True, False), args.kernel_reps) - t_prep,
+                       "am": _event_time_ms(lambda: grads(False, True), args.kernel_reps) - t_prep}
+    stages = {"mi_forward_ms": t_fwd, "mi_backward_ms": t_bwd, "logprobs_fwd_ms": t_logp,
+              "bwd_prep_ms": t_prep}
+    stages.update({"bwd_grad_%s_ms" % k: v for k, v in t_grads.items()})
 
     def hbm_line(kernel, nbytes, t_ms):
         achieved = nbytes / (t_ms * 1e-3) / 1e9
@@ -321,7 +357,27 @@ def main():
         else "simple_fwd_panel_kernel<128, 16>"
     gemm_flops = 2.0 * B * (S + 1) * T * w.C
     gemm_tflops = gemm_flops / (t_logp * 1e-3) / 1e12
-    lines = [
+    rows96 = (S + 1 + 95) // 96 * 96 < (S + 1 + 127) // 128 * 128
+    lm_shape = "96, 32" if rows96 else "128, 16"
+
+    def mfma_line(kernel, flops, t_ms):
+        tflops = flops / (t_ms * 1e-3) / 1e12
+        return {"kernel": kernel, "bound": "mfma", "achieved": round(tflops, 3),
+                "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(tflops / FP32_MFMA_PEAK_TFLOPS, 5),
+                "traffic": MEASURED_TRAFFIC.get((w.name, kernel)), "algorithmic_flops": flops,
+                "avg_launch_us": round(1e3 * t_ms, 2)}
+
+    # each gradient product is one GEMM of the forward's size (the one-hot product that
+    # scatters px_grad into am.grad is not counted)
+    if "both" in t_grads:
+        grad_lines = [mfma_line("simple_bwd_am_lm_kernel<%s>" % lm_shape, 2 * gemm_flops,
+                                t_grads["both"])]
+    else:
+        grad_lines = [mfma_line("simple_bwd_am_panel_kernel", gemm_flops, t_grads["am"]),
+                      mfma_line("simple_bwd_lm_slab_kernel<%s>" % lm_shape, gemm_flops,
+                                t_grads["lm"])]
+    lines = grad_lines + [
         hbm_line("mi_forward_kernel<float, false, 2, 2, 3>",
                  _recursion_bytes(w.boundary, S, T, B, backward=False), t_fwd),
         hbm_line("mi_backward_kernel<float, false, 2, 6, 3>",
