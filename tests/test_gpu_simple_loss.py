@@ -242,6 +242,54 @@ def test_baseline_configs(gpu_device, name):
         assert _close(da.grad, a.grad, bound, 1e-4) and _close(dl.grad, l.grad, bound, 1e-4)
 
 
+@pytest.mark.parametrize("shape", [(3, 80, 250, 500), (2, 100, 130, 96), (2, 7, 9, 5)])
+def test_gradient_products_together_and_apart(gpu_device, shape):
+    # frnnt_simple_logprobs_bwd forms lm.grad and am.grad in one launch while the products
+    # are short, and in two launches when only one of them is asked for: the same tiles,
+    # so am.grad must come out bit for bit the same, and lm.grad (whose tiles take the
+    # frames in shorter slabs inside the common launch) to rounding.
+    from fast_rnnt_amd import _lib
+    dev = gpu_device
+    B, S, T, C = shape
+    g = torch.Generator().manual_seed(77)
+    f32 = dict(dtype=torch.float32, device=dev)
+    lm = torch.randn(B, S + 1, C, generator=g).to(dev)
+    am = torch.randn(B, T, C, generator=g).to(dev)
+    sym = torch.randint(0, C, (B, S), generator=g).to(dev)
+    bnd = torch.tensor([[0, 0, S, T]] * B, dtype=torch.int64).to(dev)
+    px, py = torch.empty(B, S, T + 1, **f32), torch.empty(B, S + 1, T, **f32)
+    lm_max, am_max = torch.empty(B, S + 1, **f32), torch.empty(B, T, **f32)
+    norm_raw = torch.empty(B, S + 1, T, **f32)
+    stream = torch.cuda.current_stream().cuda_stream
+    _say(f"gradient products B={B} S={S} T={T} C={C}")
+    _lib.call("frnnt_simple_logprobs_fwd_f32", lm.data_ptr(), am.data_ptr(), sym.data_ptr(),
+              bnd.data_ptr(), px.data_ptr(), py.data_ptr(), lm_max.data_ptr(), am_max.data_ptr(),
+              norm_raw.data_ptr(), B, S, T, C, 0, 0, stream)
+    gpx = torch.rand(B, S, T + 1, generator=g).to(dev)
+    gpy = torch.rand(B, S + 1, T, generator=g).to(dev)
+    dmat = torch.empty(B, S + 1, (T + 3) // 4 * 4, **f32)
+    row_x, row_y = torch.empty(B, S + 1, **f32), torch.empty(B, S + 1, **f32)
+    col_y = torch.empty(B, T, **f32)
+
+    def grads(want_lm, want_am):
+        lm_grad = torch.full_like(lm, float("nan")) if want_lm else None
+        am_grad = torch.full_like(am, float("nan")) if want_am else None
+        _lib.call("frnnt_simple_logprobs_bwd_f32", lm.data_ptr(), am.data_ptr(), sym.data_ptr(),
+                  bnd.data_ptr(), lm_max.data_ptr(), am_max.data_ptr(), norm_raw.data_ptr(), None,
+                  0, 1.0, gpx.data_ptr(), gpy.data_ptr(), dmat.data_ptr(), row_x.data_ptr(),
+                  row_y.data_ptr(), col_y.data_ptr(), _lib.ptr(lm_grad), _lib.ptr(am_grad), B, S,
+                  T, C, 0, 0, stream)
+        torch.cuda.synchronize()
+        return lm_grad, am_grad
+
+    lm_both, am_both = grads(True, True)
+    lm_only, _ = grads(True, False)
+    _, am_only = grads(False, True)
+    assert torch.equal(am_both, am_only)
+    assert not torch.isnan(lm_both).any()
+    assert (lm_both - lm_only).abs().max().item() <= 1e-5 * max(1.0, lm_only.abs().max().item())
+
+
 def test_graph_replay_matches_eager(gpu_device):
     """rnnt_loss_simple + backward captured once in a HIP graph and replayed on new input
     values (copied into the captured tensors), with eager steps and synchronisations between
