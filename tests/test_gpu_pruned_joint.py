@@ -218,6 +218,50 @@ def test_pruning_gather_and_its_gradient(gpu_device):
     assert _close(dl.grad, l.grad, 1e-5, 1e-5) and _close(da.grad, a.grad, 1e-5, 1e-5)
 
 
+@pytest.mark.parametrize("C", [516, 1000, 1001, 2048, 4100])
+def test_pruning_gather_wide_rows(gpu_device, C):
+    # rows of several 16-byte pieces per lane, rows longer than the vector kernels take,
+    # and a row length that is no multiple of 4 (the element-wise kernels)
+    dev = gpu_device
+    g = torch.Generator().manual_seed(400 + C)
+    B, S, T, R = 2, 9, 14, 4
+    lm = torch.randn(B, S + 1, C, generator=g)
+    am = torch.randn(B, T, C, generator=g)
+    ranges = torch.randint(0, S + 2 - R, (B, T), generator=g).unsqueeze(-1) + torch.arange(R)
+    dl = lm.to(dev).requires_grad_(True)
+    _say(f"pruning gather and adjoint, C={C}")
+    _, lm_p = fast_rnnt_amd.do_rnnt_pruning(am.to(dev), dl, ranges.to(dev))
+    want = torch.gather(lm.unsqueeze(1).expand(B, T, S + 1, C), 2,
+                        ranges.unsqueeze(-1).expand(B, T, R, C))
+    assert torch.equal(lm_p.detach().cpu(), want)
+    w = torch.randn(B, T, R, C, generator=g)
+    (lm_p * w.to(dev)).sum().backward()
+    ref = torch.zeros(B, S + 1, C, dtype=torch.float64)
+    ref.scatter_add_(1, ranges.reshape(B, T * R, 1).expand(B, T * R, C),
+                     w.double().reshape(B, T * R, C))
+    assert (dl.grad.cpu().double() - ref).abs().max().item() <= 1e-5
+
+
+@pytest.mark.parametrize("C", [1500, 4096, 4100])
+def test_joint_loss_wide_rows(gpu_device, C):
+    # logits rows held in registers with 8 and 16 pieces per lane, and rows too long for that
+    dev = gpu_device
+    g = torch.Generator().manual_seed(500 + C)
+    B, S, T = 2, 5, 7
+    logits = torch.randn(B, T, S + 1, C, generator=g) * 2
+    sym = torch.randint(1, C, (B, S), generator=g)
+    bnd = torch.tensor([[0, 0, S, T], [0, 0, S - 1, T - 1]], dtype=torch.int64)
+    a = logits.clone().requires_grad_(True)
+    want = O.loss_joint(a, sym, 0, boundary=bnd, reduction="sum")
+    want.backward()
+    d = logits.to(dev).requires_grad_(True)
+    _say(f"joint loss, C={C}")
+    got = fast_rnnt_amd.rnnt_loss(d, sym.to(dev), 0, boundary=bnd.to(dev), reduction="sum")
+    got.backward()
+    assert abs(got.item() - want.item()) <= 1e-5 * abs(want.item())
+    assert (d.grad.cpu() - a.grad).abs().max().item() <= 1e-5
+
+
 def test_pruning_gradient_when_most_frames_share_a_row(gpu_device):
     """do_rnnt_pruning's lm gradient (the adjoint of the gather, rnnt_loss.py:797-802)
     when thousands of (frame, j) entries point at the same lm row: more than the adjoint
