@@ -30,10 +30,10 @@ FP32_MFMA_PEAK_TFLOPS = 157.3
 # profiles/ (FETCH_SIZE and WRITE_SIZE, scaled by what the same counters read for a
 # copy of known size); filled in for the workloads that were profiled
 MEASURED_TRAFFIC = {
-    ("c2", "simple_fwd_panel_kernel<96, 16>"): 29256514,
-    ("c2", "mi_forward_kernel<float, false, 2, 2, 3>"): 6732706,
-    ("c2", "mi_backward_kernel<float, false, 2, 6, 3>"): 9667988,
-    ("c2", "simple_bwd_am_lm_kernel<96, 16>"): 57652961,
+    ("c2", "simple_fwd_panel_kernel<96, 16>"): 29256563,
+    ("c2", "mi_forward_kernel<float, false, 2, 2, 3>"): 6732768,
+    ("c2", "mi_backward_kernel<float, false, 2, 6, 3>"): 9667956,
+    ("c2", "simple_bwd_am_lm_kernel<96, 16>"): 50092198,
 }
 
 
