@@ -2,6 +2,10 @@
 
 The export list is the reference's (fast_rnnt/python/fast_rnnt/__init__.py:1-15).
 """
+# The reference's version (CMakeLists.txt:50, written into the package by setup.py:100-103)
+# with a local label for this build.
+__version__ = "1.2+mi355x"
+
 from ._fast_rnnt import with_cuda
 
 from .mutual_information import mutual_information_recursion

@@ -60,6 +60,29 @@ def _require_gpu(*tensors: Tensor) -> None:
             raise RuntimeError("fast_rnnt_amd runs on GPU tensors only (no CPU path)")
 
 
+def _check_tensors(floats, indices) -> None:
+    """What must hold before raw pointers go to the library: every tensor on one GPU,
+    the floating-point ones of one dtype, the index tensors int64.  The kernels read
+    index tensors as 64-bit words and all floating-point buffers as one element type, so
+    anything else would be read past its end; the reference fails in the same places
+    with a RuntimeError from torch.gather / scatter_ / matmul."""
+    floats = [(n, t) for n, t in floats if t is not None]
+    indices = [(n, t) for n, t in indices if t is not None]
+    name0, first = floats[0]
+    for name, t in floats + indices:
+        if t.device != first.device:
+            raise RuntimeError(f"{name} is on {t.device}, {name0} on {first.device}: "
+                               "all tensors must be on the same device")
+    for name, t in floats:
+        if t.dtype != first.dtype:
+            raise RuntimeError(f"{name} is {t.dtype}, {name0} is {first.dtype}: "
+                               "floating-point tensors must share one dtype")
+    for name, t in indices:
+        if t.dtype != torch.int64:
+            raise RuntimeError(f"{name} must be an int64 tensor, got {t.dtype}")
+    _require_gpu(*(t for _, t in floats + indices))
+
+
 class _SimpleLogprobs(torch.autograd.Function):
     """(px, py) of the additive-joiner loss: frnnt_simple_logprobs_fwd/bwd."""
 
@@ -135,8 +158,7 @@ def get_rnnt_logprobs(
     assert symbols.shape == (B, S), symbols.shape
     validate_st_lengths(S, T, rnnt_type == "regular", boundary)
     assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
-    assert lm.dtype == am.dtype, (lm.dtype, am.dtype)
-    _require_gpu(lm, am, symbols, boundary)
+    _check_tensors([("am", am), ("lm", lm)], [("symbols", symbols), ("boundary", boundary)])
     return _SimpleLogprobs.apply(lm, am, symbols, boundary, termination_symbol, rnnt_type)
 
 
@@ -316,10 +338,8 @@ def rnnt_loss_simple(
     assert symbols.shape == (B, S), symbols.shape
     validate_st_lengths(S, T, rnnt_type == "regular", boundary)
     assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
-    assert lm.dtype == am.dtype, (lm.dtype, am.dtype)
-    _require_gpu(lm, am, symbols, boundary)
+    _check_tensors([("am", am), ("lm", lm)], [("symbols", symbols), ("boundary", boundary)])
     if boundary is not None:
-        assert boundary.dtype == torch.int64
         assert boundary.shape == (B, 4)
         for s_begin, t_begin, s_end, t_end in boundary_rows(boundary):
             assert 0 <= s_begin <= s_end <= S
@@ -392,7 +412,7 @@ def get_rnnt_logprobs_joint(
     assert symbols.shape == (B, S), symbols.shape
     validate_st_lengths(S, T, rnnt_type == "regular", boundary)
     assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
-    _require_gpu(logits, symbols, boundary)
+    _check_tensors([("logits", logits)], [("symbols", symbols), ("boundary", boundary)])
     return _LatticeLogprobs.apply(logits, symbols, None, boundary, termination_symbol, rnnt_type)
 
 
@@ -444,7 +464,7 @@ def get_rnnt_prune_ranges(px_grad: Tensor, py_grad: Tensor, boundary: Tensor,
     assert py_grad.shape == (B, S + 1, T), py_grad.shape
     assert boundary.shape == (B, 4), boundary.shape
     validate_st_lengths(S, T, is_regular, boundary)
-    _require_gpu(px_grad, py_grad, boundary)
+    _check_tensors([("px_grad", px_grad), ("py_grad", py_grad)], [("boundary", boundary)])
 
     if is_regular:
         Ss = boundary[:, 2]
@@ -516,7 +536,7 @@ def do_rnnt_pruning(am: Tensor, lm: Tensor, ranges: Tensor) -> Tuple[Tensor, Ten
     assert am.shape[1] == ranges.shape[1], (am.shape[1], ranges.shape[1])
     (B, T, s_range) = ranges.shape
     (B, S1, C) = lm.shape
-    _require_gpu(am, lm, ranges)
+    _check_tensors([("am", am), ("lm", lm)], [("ranges", ranges)])
     am_pruning = am.unsqueeze(2).expand((B, T, s_range, C))
     lm_pruning = _PruneGather.apply(lm, ranges)
     return am_pruning, lm_pruning
@@ -545,7 +565,8 @@ def get_rnnt_logprobs_pruned(
     (B, S) = symbols.shape
     validate_st_lengths(S, T, rnnt_type == "regular", boundary)
     assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
-    _require_gpu(logits, symbols, ranges, boundary)
+    _check_tensors([("logits", logits)],
+                   [("symbols", symbols), ("ranges", ranges), ("boundary", boundary)])
     return _LatticeLogprobs.apply(logits, symbols, ranges, boundary, termination_symbol,
                                   rnnt_type)
 
@@ -646,7 +667,7 @@ def get_rnnt_logprobs_smoothed(
     assert symbols.shape == (B, S), symbols.shape
     validate_st_lengths(S, T, rnnt_type == "regular", boundary)
     assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
-    _require_gpu(lm, am, symbols, boundary)
+    _check_tensors([("am", am), ("lm", lm)], [("symbols", symbols), ("boundary", boundary)])
 
     # joint part, without the boundary / constrained post-processing (applied last)
     base_type = "regular" if rnnt_type == "regular" else "modified"

@@ -4,7 +4,8 @@
 fast_rnnt/python/csrc/mutual_information.cu:27-67 on CPU tensors, and
 ``mutual_information_recursion`` follows
 fast_rnnt/python/fast_rnnt/mutual_information.py:24-298, including the eager
-backward inside forward and the in-place scaling of the saved gradients.
+backward inside forward and the in-place scaling of the saved gradients;
+``joint_mutual_information_recursion`` follows :314-425 of the same file.
 """
 import ctypes
 import os
@@ -144,3 +145,43 @@ def mutual_information_recursion(px, py, boundary=None, return_grad=False):
     sink = [None, None]
     scores = _Recursion.apply(px.contiguous(), py.contiguous(), sink, boundary, return_grad)
     return (scores, (sink[0], sink[1])) if return_grad else scores
+
+
+def joint_mutual_information_recursion(px, py, boundary=None):
+    """Mirrors fast_rnnt/python/fast_rnnt/mutual_information.py:314-425: the recursion
+    on the summed terms, with the total score split over the summands by occupation-
+    weighted sums (term n gets sum(px_grad * px[n]) + sum(py_grad * py[n])); what is
+    left over -- log-of-sum minus sum-of-log -- is credited to term 0 (:420-424).
+    -inf entries are raised to the most negative finite number first (:411-412), so a
+    blocked cell contributes 0 * finite = 0.  Returns a tensor of shape (len(px), B).
+    """
+    n_terms = len(px)
+    assert len(py) == n_terms and n_terms > 0
+    B, S, T1 = px[0].shape
+    T = py[0].shape[2]
+    assert T1 in (T, T + 1)
+    assert py[0].shape == (B, S + 1, T)
+    assert px[0].dtype == py[0].dtype
+    if boundary is not None:
+        assert boundary.dtype == torch.int64
+        assert boundary.shape == (B, 4)
+        for s0, t0, s1, t1 in boundary.tolist():
+            assert 0 <= s0 <= s1 <= S
+            assert 0 <= t0 <= t1 <= T
+    with torch.no_grad():
+        x_total = torch.stack(list(px), dim=0).sum(dim=0).contiguous()
+        y_total = torch.stack(list(py), dim=0).sum(dim=0).contiguous()
+        p = torch.empty(B, S + 1, T + 1, dtype=x_total.dtype)
+        total = mi_forward(x_total, y_total, boundary, p)
+        occ_x, occ_y = mi_backward(x_total, y_total, boundary, p,
+                                   torch.ones(B, dtype=x_total.dtype))
+    floor = torch.finfo(x_total.dtype).min
+    shares = []
+    for x, y in zip(px, py):
+        shares.append((occ_x * x.clamp(min=floor)).sum(dim=(1, 2))
+                      + (occ_y * y.clamp(min=floor)).sum(dim=(1, 2)))
+    shares = torch.stack(shares, dim=0)  # (N, B)
+    with torch.no_grad():
+        leftover = total - shares.sum(dim=0)
+    first = shares[0] + leftover
+    return torch.cat((first.unsqueeze(0), shares[1:]), dim=0)

@@ -14,6 +14,8 @@ import fast_rnnt_amd
 from fast_rnnt_amd import workloads
 from oracle import losses as O
 
+import ulp_sensitivity as U
+
 pytestmark = pytest.mark.gpu
 KINDS = ["regular", "modified", "constrained"]
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
@@ -368,6 +370,36 @@ def test_small_s_range_never_gives_inf(gpu_device):
         assert torch.isfinite(loss).all(), (S, loss)
 
 
+@pytest.mark.parametrize("kind", KINDS)
+def test_pruned_with_every_row_kept_equals_unpruned(gpu_device, kind):
+    # ranges that keep all S + 1 rows of every frame: rnnt_loss_pruned must give what
+    # rnnt_loss gives on the same logits, loss and gradient (the identity the reference's
+    # pruned tests print side by side, rnnt_loss_test.py:435-515), and both the oracle's
+    dev = gpu_device
+    for n, (B, S, T, C) in enumerate([(2, 5, 9, 8), (3, 20, 41, 30), (2, 66, 80, 17)]):
+        am, lm, sym, bnd = _case(300 + n, B, S, T, C, torch.float32, kind)
+        g = torch.Generator().manual_seed(300 + n)
+        logits = torch.randn(B, T, S + 1, C, generator=g)
+        ranges = torch.arange(S + 1).reshape(1, 1, S + 1).expand(B, T, S + 1).contiguous()
+        _say(f"pruned(S+1) == joint, {kind} shape{n}")
+        a = logits.clone().requires_grad_(True)
+        want = O.loss_joint(a, sym, 0, boundary=bnd, rnnt_type=kind, reduction="none")
+        want.sum().backward()
+        full = logits.to(dev).requires_grad_(True)
+        joint = fast_rnnt_amd.rnnt_loss(full, sym.to(dev), 0, boundary=bnd.to(dev),
+                                        rnnt_type=kind, reduction="none")
+        joint.sum().backward()
+        kept = logits.to(dev).requires_grad_(True)
+        pruned = fast_rnnt_amd.rnnt_loss_pruned(kept, sym.to(dev), ranges.to(dev), 0,
+                                                boundary=bnd.to(dev), rnnt_type=kind,
+                                                reduction="none")
+        pruned.sum().backward()
+        assert torch.equal(pruned, joint)
+        assert torch.equal(kept.grad, full.grad)
+        assert _close(joint, want, 0.0, 1e-5)
+        assert _close(full.grad, a.grad, 1e-4, 1e-4)
+
+
 def test_c5_unpruned_full_size(gpu_device):
     dev = gpu_device
     w = workloads.make("c5")
@@ -424,9 +456,18 @@ def test_c3_pruned_full_size(gpu_device):
          f"side uses its own gradients: {frames} of {wr.shape[0] * wr.shape[1]}")
     assert abs(gs.item() - ws.item()) <= 1e-5 * abs(ws.item())
     assert abs(gl.item() - wl.item()) <= 1e-5 * abs(wl.item())
-    # Scores reach |p| ~ 3000 here, where one float32 ulp of p is 2.4e-4: a single
-    # differently rounded cell of p moves the occupation of its neighbours by up to
-    # that much (relative), so 1e-4 absolute cannot be guaranteed once px / py differ
-    # in their last bit between the two pipelines (measured: 1.0e-4).  Bound: 2e-4.
-    assert _close(ggx, wgx, 2e-4) and _close(ggy, wgy, 2e-4)
-    assert _close(da.grad, a.grad, 2e-4, 1e-3) and _close(dl.grad, l.grad, 2e-4, 1e-3)
+    # Scores reach |p| ~ 3000 here, where one float32 ulp of p is 2.4e-4, and the two
+    # pipelines' px / py agree only to rounding (two GEMM summation orders).  The bound is
+    # what such rounding does to the float32 CPU reference ITSELF: 1.25 x the movement of
+    # its gradients under a one-ulp nudge of px / py (tests/ulp_sensitivity.py; 1.0e-4 at
+    # this workload, so 1.25e-4), not less than the acceptance criterion's 1e-4.  The
+    # recursion kernels alone, on identical px / py, stay below 1e-4
+    # (tests/test_gpu_recursion_fidelity.py).
+    opx, opy = O.lattice_logprobs_smoothed(w.lm, w.am, w.symbols, 0, 0.25, 0.0,
+                                           boundary=w.boundary)
+    bound = U.grad_bound(opx, opy, w.boundary)
+    _say(f"  px_grad / py_grad bound from the reference's one-ulp sensitivity: {bound:.2e}")
+    assert bound <= 2e-4
+    assert _close(ggx, wgx, bound) and _close(ggy, wgy, bound)
+    # am.grad / lm.grad add such cells up over lattice rows / frames
+    assert _close(da.grad, a.grad, 2 * bound, 1e-3) and _close(dl.grad, l.grad, 2 * bound, 1e-3)

@@ -70,7 +70,15 @@ def _compare(px, py, bnd, w, dev, tag):
     assert torch.equal(written, ~torch.isnan(p_gpu))
     pc, pg = p_cpu[written], p_gpu[written]
     same_inf = torch.isinf(pc) & (pc == pg)
-    assert bool((same_inf | ((pc - pg).abs() <= rtol * pc.abs().clamp(min=1.0))).all())
+    # A cell of p is a running sum along lattice paths: its absolute error is set by the
+    # largest magnitude met on the way, not by its own.  Scores that climb to hundreds and
+    # come back through zero keep errors of a few ulps of that maximum (the float32 CPU
+    # reference itself is then 6e-5 off the float64 one at cells with |p| < 1, see
+    # tests/test_oracle_conditioning.py), so the relative bound gets that much slack.
+    finite = torch.isfinite(pc)
+    top = pc[finite].abs().max().item() if bool(finite.any()) else 0.0
+    slack = 4 * torch.finfo(dtype).eps * top
+    assert bool((same_inf | ((pc - pg).abs() <= rtol * pc.abs().clamp(min=1.0) + slack)).all())
     assert (gx_cpu - gx_gpu.cpu()).abs().max().item() <= gtol if gx_cpu.numel() else True
     assert (gy_cpu - gy_gpu.cpu()).abs().max().item() <= gtol if gy_cpu.numel() else True
     # the gradient reaching the lattice origin is written back into ans_grad
@@ -195,3 +203,46 @@ def test_joint_recursion_splits_the_total(gpu_device):
     m2 = fast_rnnt_amd.joint_mutual_information_recursion((px * 0.5, px * 0.5), (py * 0.5, py * 0.5))
     assert torch.allclose(m, m1[0], atol=1e-9)
     assert torch.allclose(m, m2.sum(0), atol=1e-9)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("modified", [False, True])
+def test_joint_recursion_matches_oracle(gpu_device, dtype, modified):
+    # shares per term and their gradients against the CPU restatement of
+    # mutual_information.py:314-425, with windows and blocked cells
+    dev = gpu_device
+    g = torch.Generator().manual_seed(31 + int(modified))
+    for B, S, T, N in [(3, 6, 9, 1), (4, 70, 40, 3), (2, 33, 150, 2)]:
+        _say(f"joint recursion {dtype} modified={modified} B={B} S={S} T={T} N={N}")
+        xs = [torch.randn(B, S, T + (0 if modified else 1), generator=g, dtype=dtype) / N
+              for _ in range(N)]
+        ys = [torch.randn(B, S + 1, T, generator=g, dtype=dtype) / N for _ in range(N)]
+        xs[0][:, 1, 2] = -math.inf
+        if not modified:
+            xs[0][:, :, T] = -math.inf
+        for bnd in (None, _windows(g, B, S, T, modified)):
+            cx = [x.clone().requires_grad_(True) for x in xs]
+            cy = [y.clone().requires_grad_(True) for y in ys]
+            want = oracle.joint_mutual_information_recursion(cx, cy, bnd)
+            weights = torch.randn(N, B, generator=g, dtype=dtype)
+            live = torch.isfinite(want.detach().sum(0))  # utterances with a path
+            (want[:, live] * weights[:, live]).sum().backward()
+            dx = [x.to(dev).requires_grad_(True) for x in xs]
+            dy = [y.to(dev).requires_grad_(True) for y in ys]
+            got = fast_rnnt_amd.joint_mutual_information_recursion(
+                dx, dy, bnd.to(dev) if bnd is not None else None)
+            (got[:, live.to(dev)] * weights.to(dev)[:, live.to(dev)]).sum().backward()
+            assert got.shape == (N, B)
+            tol = 2e-5 if dtype == torch.float32 else 1e-10
+            w_, g_ = want.detach()[:, live], got.detach().cpu()[:, live]
+            assert torch.allclose(g_, w_, rtol=tol, atol=tol * max(1.0, float(w_.abs().max())))
+            # the total is the plain recursion's score
+            plain = fast_rnnt_amd.mutual_information_recursion(
+                sum(x.to(dev) for x in xs), sum(y.to(dev) for y in ys),
+                bnd.to(dev) if bnd is not None else None)
+            assert torch.allclose(got.detach().sum(0)[live.to(dev)], plain[live.to(dev)],
+                                  rtol=tol, atol=tol * 10)
+            gtol = 1e-4 if dtype == torch.float32 else 1e-9
+            for n in range(N):
+                assert (dx[n].grad.cpu() - cx[n].grad).abs().max().item() <= gtol * 3
+                assert (dy[n].grad.cpu() - cy[n].grad).abs().max().item() <= gtol * 3

@@ -1,7 +1,8 @@
 """rnnt_loss_simple / get_rnnt_logprobs on the GPU against the CPU oracle.
 
 Tolerances (float32): loss 1e-5 relative, px_grad / py_grad 1e-4 absolute
-(2.5e-4 at the large-vocabulary workload, see _GRAD_BOUND), am.grad / lm.grad the same
+(at the large-vocabulary workload: 1.25 x what one ulp of px / py does to the float32 CPU
+reference itself, 2.7e-4, see test_baseline_configs), am.grad / lm.grad the same
 absolute + 1e-4 relative; float64: 1e-9.
 """
 import sys
@@ -13,6 +14,8 @@ import fast_rnnt_amd
 from fast_rnnt_amd import rnnt_loss as R
 from fast_rnnt_amd import workloads
 from oracle import losses as O
+
+import ulp_sensitivity as U
 
 pytestmark = pytest.mark.gpu
 KINDS = ["regular", "modified", "constrained"]
@@ -134,9 +137,13 @@ def test_loss_and_all_gradients(gpu_device, dtype, kind):
     dev = gpu_device
     for n, (B, S, T, C) in enumerate([(3, 5, 9, 8), (4, 20, 75, 50), (2, 66, 140, 70),
                                       (2, 101, 120, 44)]):
-        for reduction in ("sum", "mean", "none"):
-            _say(f"loss {kind} {dtype} shape{n} reduction={reduction}")
-            am, lm, sym, bnd = _case(60 + n, B, S, T, C, dtype, kind)
+        # with a boundary, and without one: the fused node then runs the recursion kernels'
+        # whole-lattice path (nothing to zero around the window) and the loss reduction
+        # fused into the backward recursion on it
+        for reduction, with_boundary in [("sum", True), ("mean", True), ("none", True),
+                                         ("sum", False), ("mean", False), ("none", False)]:
+            _say(f"loss {kind} {dtype} shape{n} reduction={reduction} boundary={with_boundary}")
+            am, lm, sym, bnd = _case(60 + n, B, S, T, C, dtype, kind, with_boundary)
             a = am.clone().requires_grad_(True)
             l = lm.clone().requires_grad_(True)
             want, (wx, wy) = O.loss_simple(l, a, sym, 0, boundary=bnd, rnnt_type=kind,
@@ -147,8 +154,8 @@ def test_loss_and_all_gradients(gpu_device, dtype, kind):
             da = am.to(dev).requires_grad_(True)
             dl = lm.to(dev).requires_grad_(True)
             got, (gx, gy) = fast_rnnt_amd.rnnt_loss_simple(
-                dl, da, sym.to(dev), 0, boundary=bnd.to(dev), rnnt_type=kind,
-                reduction=reduction, return_grad=True)
+                dl, da, sym.to(dev), 0, boundary=bnd.to(dev) if bnd is not None else None,
+                rnnt_type=kind, reduction=reduction, return_grad=True)
             gx0, gy0 = gx.clone(), gy.clone()
             got.sum().backward()
             f32 = dtype == torch.float32
@@ -179,15 +186,15 @@ def test_delay_penalty_and_only_one_input_needs_grad(gpu_device):
         fast_rnnt_amd.rnnt_loss_simple(dl, am.to(dev), sym.to(dev), 0, reduction="bogus")
 
 
-# One float32 ulp of the lattice scores p is 2.4e-4 at |p| ~ 3000 (c2, c4 per utterance).
-# The occupation gradients are exp of differences of p, so once px / py differ in their
-# last bit between two pipelines (the normalizer's summation order differs between any two
-# GEMMs), a cell of p that rounds the other way moves the gradients around it by up to
-# one such ulp times the occupation there.  1e-4 holds at c1 and c2; at c4 the measured
-# difference is 2.1e-4 and the bound one ulp of p, 2.5e-4.  What keeps that honest is
-# the second check: against the float64 oracle the GPU's gradients must be as close as
-# the float32 CPU reference's own.
-_GRAD_BOUND = {"c1": 1e-4, "c2": 1e-4, "c4": 2.5e-4}
+# One float32 ulp of the lattice scores p is 2.4e-4 at |p| ~ 3000 (c2) and 4.9e-4 at
+# ~4500 (c4).  The occupation gradients are exp of differences of p, so once px / py differ
+# in their last bit between two pipelines (the normalizer's summation order differs between
+# any two GEMMs), the gradients move by what tests/ulp_sensitivity.py measures on the float32
+# CPU reference alone: below 1e-4 at c1 and c2, 2.1e-4 at c4.  The bound is the acceptance
+# criterion's 1e-4 or 1.25 x that movement, whichever is larger (the recursion kernels by
+# themselves, on identical px / py, meet 1e-4 at every workload:
+# tests/test_gpu_recursion_fidelity.py).  A second check keeps that honest: against the
+# float64 oracle the GPU's gradients must be as close as the float32 CPU reference's own.
 
 
 @pytest.mark.parametrize("name", ["c1", "c2", "c4"])
@@ -225,7 +232,10 @@ def test_baseline_configs(gpu_device, name):
          f"lm.grad maxdiff={(dl.grad.cpu() - l.grad).abs().max().item():.2e}; "
          f"px/py_grad against float64: gpu {gpu_off:.2e}, cpu float32 {cpu_off:.2e}")
     assert rel <= 1e-5
-    bound = _GRAD_BOUND[name]
+    opx, opy = O.lattice_logprobs_simple(w.lm, w.am, w.symbols, 0, boundary=w.boundary)
+    bound = U.grad_bound(opx, opy, w.boundary)
+    _say(f"  px_grad / py_grad bound from the reference's one-ulp sensitivity: {bound:.2e}")
+    assert bound <= (1e-4 if name != "c4" else 3e-4)
     assert _close(gx0, wx0, bound) and _close(gy0, wy0, bound)
     assert gpu_off <= 1.5 * cpu_off + 2e-5
     # am.grad / lm.grad are sums of those over the lattice rows / frames: the same bound

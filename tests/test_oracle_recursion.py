@@ -206,3 +206,76 @@ def test_bit_equal_to_reference_build(dtype, modified):
         g1 = recursion.mi_backward(px, py, bnd, p1, w)
         g2 = ref.mutual_information_backward(px, py, bnd, p2, w.clone())
         assert torch.equal(g1[0], g2[0]) and torch.equal(g1[1], g2[1])
+
+
+# ---- joint_mutual_information_recursion (mutual_information.py:314-425) ---------------
+
+@pytest.mark.parametrize("modified", [False, True])
+def test_joint_recursion_constant_terms_closed_form(modified):
+    # term n is a_n on every x-step and b_n on every y-step.  A path of the regular lattice
+    # takes S x-steps and T y-steps, so term n's share is S a_n + T b_n and what is left of
+    # the total, log C(S+T, S), goes to term 0; a path of the modified lattice takes S
+    # diagonal steps and T - S y-steps, and there are C(T, S) of them.
+    S, T = 4, 7
+    a, b = [0.3, -1.1, 0.25], [-0.7, 0.4, -0.05]
+    px = [torch.full((2, S, T if modified else T + 1), v, dtype=torch.float64) for v in a]
+    py = [torch.full((2, S + 1, T), v, dtype=torch.float64) for v in b]
+    got = recursion.joint_mutual_information_recursion(px, py)
+    assert got.shape == (3, 2)
+    ny = T - S if modified else T
+    paths = truth.log_binom(T, S) if modified else truth.log_binom(S + T, S)
+    for n in range(3):
+        want = S * a[n] + ny * b[n] + (paths if n == 0 else 0.0)
+        assert abs(got[n, 0].item() - want) < 1e-10 and abs(got[n, 1].item() - want) < 1e-10
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_joint_recursion_one_term_and_halves(dtype):
+    # mutual_information_test.py:138-154: one term gives the plain recursion, and the
+    # shares of two halves add up to it; with windows, and with blocked cells in px
+    g = torch.Generator().manual_seed(21)
+    B, S, T = 3, 6, 9
+    px = torch.randn(B, S, T + 1, generator=g, dtype=dtype)
+    py = torch.randn(B, S + 1, T, generator=g, dtype=dtype)
+    px[:, :, T] = -math.inf
+    px[1, 2, 3] = -math.inf
+    bnd = torch.tensor([[0, 0, S, T], [1, 2, 5, 8], [0, 0, 3, 9]])
+    for boundary in (None, bnd):
+        plain = recursion.mutual_information_recursion(px, py, boundary)
+        one = recursion.joint_mutual_information_recursion((px,), (py,), boundary)
+        two = recursion.joint_mutual_information_recursion((px * 0.5, px * 0.5),
+                                                           (py * 0.5, py * 0.5), boundary)
+        tol = 1e-5 if dtype == torch.float32 else 1e-12
+        assert one.shape == (1, B) and two.shape == (2, B)
+        assert torch.allclose(one[0], plain, rtol=tol, atol=tol)
+        assert torch.allclose(two.sum(0), plain, rtol=tol, atol=tol)
+        assert torch.isfinite(two).all()  # -inf * 0 was kept out
+
+
+def test_joint_recursion_gradients_are_the_occupations():
+    # d(sum of shares)/d px[n] is the occupation of the summed lattice for every n:
+    # compare with autograd through an independent logaddexp programme on the sums
+    g = torch.Generator().manual_seed(22)
+    B, S, T = 2, 4, 5
+    bnd = torch.tensor([[0, 0, 4, 5], [1, 0, 3, 4]])
+    xs = [torch.randn(B, S, T + 1, generator=g, dtype=torch.float64).requires_grad_(True)
+          for _ in range(2)]
+    ys = [torch.randn(B, S + 1, T, generator=g, dtype=torch.float64).requires_grad_(True)
+          for _ in range(2)]
+    shares = recursion.joint_mutual_information_recursion(xs, ys, bnd)
+    shares.sum().backward()
+    ax = (xs[0] + xs[1]).detach().requires_grad_(True)
+    ay = (ys[0] + ys[1]).detach().requires_grad_(True)
+    total = truth.dp_torch(ax, ay, bnd, modified=False)
+    total.sum().backward()
+    assert torch.allclose(shares.sum(0).detach(), total.detach(), atol=1e-10)
+    for n in range(2):
+        assert torch.allclose(xs[n].grad, ax.grad, atol=1e-10)
+        assert torch.allclose(ys[n].grad, ay.grad, atol=1e-10)
+    # and a single share: weights another term's occupation-weighted sum does not see
+    for t in xs + ys:
+        t.grad = None
+    shares = recursion.joint_mutual_information_recursion(xs, ys, bnd)
+    shares[1].sum().backward()
+    assert torch.allclose(xs[1].grad, ax.grad, atol=1e-10)
+    assert xs[0].grad is None or float(xs[0].grad.abs().max()) == 0.0
