@@ -46,5 +46,7 @@ def reference_sensitivity(px, py, boundary, trials: int = 4, seed: int = 5) -> f
 
 def grad_bound(px, py, boundary, floor: float = 1e-4, slack: float = 1.25) -> float:
     """The px_grad / py_grad bound a float32 parity test may use on these inputs: the
-    acceptance criterion's 1e-4, or `slack` times what one ulp does to the reference."""
-    return max(floor, slack * reference_sensitivity(px, py, boundary))
+    acceptance criterion's 1e-4 while one ulp moves the reference by no more than that,
+    `slack` times the movement otherwise."""
+    moved = reference_sensitivity(px, py, boundary)
+    return floor if moved <= floor else slack * moved
