@@ -20,6 +20,8 @@
 //                   + sum_s [c = sym[b,s]] gx[s,t] + [c = term] sum_s gy[s,t]
 // i.e. two more GEMMs with the same fused-exp loaders (what autograd derives for
 // rnnt_loss.py:174-220; the derivatives through the two max() cancel).
+#include <mutex>
+
 #include "xcd_grid.hip.h"
 #include "tile_gemm.hip.h"
 
@@ -1392,10 +1394,66 @@ int reduce_impl(const R *scores, R *loss, int B, int reduction, void *stream) {
   return check_launch("loss_reduce");
 }
 
+// ---- scratch that the library owns: for callers that cannot allocate --------------------
+// One array per GPU, part of the code object, held until the process ends.  In host code
+// the array's name is only a handle: its device address is looked up once per device
+// (with that device current) and kept; kernels and everything else get that address.
+constexpr size_t kOwnScratchFloats = (size_t)4 << 20;  // 16 MiB
+static __device__ __align__(256) float own_scratch[kOwnScratchFloats];
+constexpr int kMaxDevices = 64;
+
+float *own_scratch_address() {
+  static std::mutex guard;
+  static float *address[kMaxDevices] = {nullptr};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(guard);
+  if (!address[device]) {
+    void *found = nullptr;
+    if (hipGetSymbolAddress(&found, HIP_SYMBOL(own_scratch)) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    address[device] = static_cast<float *>(found);
+  }
+  return address[device];
+}
+
 }  // namespace
 }  // namespace frnnt
 
 extern "C" {
+
+int frnnt_simple_logprobs_bwd_noalloc_f32(const float *lm, const float *am, const int64_t *symbols,
+                                          const int64_t *boundary, const float *lm_max,
+                                          const float *am_max, const float *norm_raw,
+                                          const float *score_grad, int score_grad_stride,
+                                          double score_grad_scale, float *px_grad,
+                                          float *py_grad, float *lm_grad, float *am_grad, int B,
+                                          int S, int T, int C, int termination_symbol,
+                                          int rnnt_type, void *stream) {
+  using frnnt::fail;
+  if (B < 0 || S < 0 || T < 0) return fail(FRNNT_EINVAL, "simple_logprobs_bwd_noalloc: bad size");
+  // dmat | row_x | row_y | col_y, each starting 16-byte aligned
+  const size_t ldd = ((size_t)T + 3) & ~(size_t)3;
+  const size_t n_rows = ((size_t)B * (S + 1) + 3) & ~(size_t)3;
+  const size_t n_cols = ((size_t)B * T + 3) & ~(size_t)3;
+  const size_t n_dmat = (size_t)B * (S + 1) * ldd;
+  const size_t need = n_dmat + 2 * n_rows + n_cols;
+  if (need > frnnt::kOwnScratchFloats)
+    return fail(FRNNT_ELIMIT,
+                "simple_logprobs_bwd_noalloc: B=%d S=%d T=%d needs %zu bytes of scratch, the "
+                "library's own buffer holds %zu; use frnnt_simple_logprobs_bwd_f32 with a "
+                "caller-provided workspace",
+                B, S, T, need * sizeof(float), frnnt::kOwnScratchFloats * sizeof(float));
+  float *base = frnnt::own_scratch_address();
+  if (!base) return fail(FRNNT_ELAUNCH, "simple_logprobs_bwd_noalloc: hipGetSymbolAddress failed");
+  float *dmat = base, *row_x = dmat + n_dmat, *row_y = row_x + n_rows, *col_y = row_y + n_rows;
+  return frnnt::bwd_impl<float>(lm, am, symbols, boundary, lm_max, am_max, norm_raw, score_grad,
+                                score_grad_stride, score_grad_scale, px_grad, py_grad, dmat, row_x,
+                                row_y, col_y, lm_grad, am_grad, B, S, T, C, termination_symbol,
+                                rnnt_type, stream);
+}
 
 int frnnt_simple_logprobs_fwd_f32(const float *lm, const float *am, const int64_t *symbols,
                                   const int64_t *boundary, float *px, float *py, float *lm_max,

@@ -150,6 +150,26 @@ int frnnt_simple_logprobs_bwd_f64(const double *lm, const double *am, const int6
                                   double *lm_grad, double *am_grad, int B, int S, int T, int C,
                                   int termination_symbol, int rnnt_type, void *stream);
 /*
+ * frnnt_simple_logprobs_bwd_f32 for callers that cannot allocate device memory (code under
+ * HIP graph capture, serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments and results, without the four scratch
+ * buffers: dmat, row_x, row_y and col_y live in a 16 MiB array that is part of the
+ * library's code object, one copy per GPU, held until the process ends.  The call
+ * allocates nothing.  FRNNT_ELIMIT when 4 * (B (S+1) (T rounded up to 4) + 2 B (S+1) + B T)
+ * bytes (each part rounded up to 16) exceed 16 MiB.  All calls on one GPU share that
+ * array: calls that overlap there (two streams, two threads) race, so issue them one
+ * after the other on one stream.  The first call on a device looks the array's address
+ * up (hipGetSymbolAddress); make that call outside a stream capture.
+ */
+int frnnt_simple_logprobs_bwd_noalloc_f32(const float *lm, const float *am, const int64_t *symbols,
+                                          const int64_t *boundary, const float *lm_max,
+                                          const float *am_max, const float *norm_raw,
+                                          const float *score_grad, int score_grad_stride,
+                                          double score_grad_scale, float *px_grad,
+                                          float *py_grad, float *lm_grad, float *am_grad, int B,
+                                          int S, int T, int C, int termination_symbol,
+                                          int rnnt_type, void *stream);
+/*
  * The lm-only / am-only smoothing of get_rnnt_logprobs_smoothed (rnnt_loss.py:1135-1369)
  * applied to joint px / py (px_joint, py_joint: outputs of frnnt_simple_logprobs_fwd
  * without a boundary, regular or modified layout):
