@@ -203,12 +203,12 @@ def _bench_lattice(args, w, dev):
     def fwd():
         _lib.call("frnnt_lattice_logprobs_fwd_f32", lg.data_ptr(), sym.data_ptr(), rp,
                   bnd.data_ptr(), px.data_ptr(), py.data_ptr(), norm.data_ptr(), xr.data_ptr(),
-                  yr.data_ptr(), B, S, T, R, C, 0, 0, stream)
+                  yr.data_ptr(), B, S, T, R, C, 0, 0, 1, stream)
 
     def bwd():
         _lib.call("frnnt_lattice_logprobs_bwd_f32", lg.data_ptr(), sym.data_ptr(), rp,
                   bnd.data_ptr(), norm.data_ptr(), gpx.data_ptr(), gpy.data_ptr(), grad.data_ptr(),
-                  B, S, T, R, C, 0, 0, stream)
+                  B, S, T, R, C, 0, 0, 1, stream)
 
     t_f = _event_time_ms(fwd, args.kernel_reps)
     t_b = _event_time_ms(bwd, args.kernel_reps)

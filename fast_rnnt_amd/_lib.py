@@ -42,10 +42,10 @@ _SIGNATURES = {
     "frnnt_simple_loss_fwd_f64": ([_P] * 14 + [_I] * 7 + [_P], _I),
     "frnnt_loss_reduce_f32": ([_P, _P, _I, _I, _P], _I),
     "frnnt_loss_reduce_f64": ([_P, _P, _I, _I, _P], _I),
-    "frnnt_lattice_logprobs_fwd_f32": ([_P] * 9 + [_I] * 7 + [_P], _I),
-    "frnnt_lattice_logprobs_fwd_f64": ([_P] * 9 + [_I] * 7 + [_P], _I),
-    "frnnt_lattice_logprobs_bwd_f32": ([_P] * 8 + [_I] * 7 + [_P], _I),
-    "frnnt_lattice_logprobs_bwd_f64": ([_P] * 8 + [_I] * 7 + [_P], _I),
+    "frnnt_lattice_logprobs_fwd_f32": ([_P] * 9 + [_I] * 8 + [_P], _I),
+    "frnnt_lattice_logprobs_fwd_f64": ([_P] * 9 + [_I] * 8 + [_P], _I),
+    "frnnt_lattice_logprobs_bwd_f32": ([_P] * 8 + [_I] * 8 + [_P], _I),
+    "frnnt_lattice_logprobs_bwd_f64": ([_P] * 8 + [_I] * 8 + [_P], _I),
     "frnnt_prune_ranges_f32": ([_P] * 4 + [_I] * 5 + [_P], _I),
     "frnnt_prune_ranges_f64": ([_P] * 4 + [_I] * 5 + [_P], _I),
     "frnnt_prune_gather_f32": ([_P] * 3 + [_I] * 5 + [_P], _I),

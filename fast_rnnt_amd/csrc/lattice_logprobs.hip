@@ -69,15 +69,31 @@ __device__ __forceinline__ int64_t row_symbol(const int64_t *symbols, const int6
   return s == S ? (int64_t)term : symbols[(long)b * S + s];
 }
 
+// True when the logits row (b, t) x lattice row s lies outside utterance b's boundary
+// window [s_begin, s_end] x [t_begin, t_end): the recursion never looks at its px / py
+// and hands it a gradient of exact zeros.  Callers that go on to the recursion with the
+// same boundary (the loss functions) let the kernels skip such rows -- about a third of
+// a ragged batch.  `s` < 0 stands for "not known", only the frame is tested then.
+__device__ __forceinline__ bool outside_window(const int64_t *boundary, int b, int t, int64_t s) {
+  const int64_t s_begin = boundary[4 * b + 0], t_begin = boundary[4 * b + 1];
+  const int64_t s_end = boundary[4 * b + 2], t_end = boundary[4 * b + 3];
+  return t < t_begin || t >= t_end || (s >= 0 && (s < s_begin || s > s_end));
+}
+
 // 4 rows per 256-thread block.
 template <typename R>
 __global__ void __launch_bounds__(256)
     row_norm_kernel(const R *__restrict__ logits, const int64_t *__restrict__ symbols,
-                    const int64_t *__restrict__ ranges, R *__restrict__ norm, R *__restrict__ xr,
-                    R *__restrict__ yr, long rows, int T, int Rr, int S, int C, int term) {
+                    const int64_t *__restrict__ ranges, const int64_t *__restrict__ window,
+                    R *__restrict__ norm, R *__restrict__ xr, R *__restrict__ yr, long rows, int T,
+                    int Rr, int S, int C, int term) {
   const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (row >= rows) return;
+  if (window &&
+      outside_window(window, (int)(row / ((long)Rr * T)), (int)((row / Rr) % T),
+                     ranges ? ranges[row] : row % Rr))
+    return;
   const R *x = logits + row * C;
   R m = Num<R>::neg_inf();
   for (int c = lane; c < C; c += kWave) {
@@ -100,14 +116,20 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-// The same with the row held in registers (fp32, C a multiple of 4, at most
-// 256 * kVecs entries): the logits are read once, 16 bytes per lane and load.  The two
-// entries the row contributes to px / py are taken from the registers that hold them
-// (selects under wave-uniform conditions, then a read of the owning lane), not read
-// again from memory: a second, dependent load would keep every wave alive for another
-// memory round trip.  The row's symbol comes through the scalar cache while the logits
-// travel.
+// The same with the rows held in registers (fp32, C a multiple of 4, at most
+// 256 * kVecs entries).  A wave takes kRows consecutive rows (the launchers use 1: more
+// rows per wave were slower).  The rows are fetched through a raw buffer resource
+// that covers just the wave's rows -- 16 bytes per lane and load, every load of every row
+// in flight before the first is used; a row that needs no work (past the end, or outside
+// the boundary window when the caller asked for that) and a piece past the end of a row
+// get an offset outside the resource, which reads as 0 and moves no data: no branch
+// stands between the loads.  The two entries a row contributes to px / py are taken from
+// the registers that hold them (selects under wave-uniform conditions, then a read of
+// the owning lane), not read again from memory.  `kStream`: the logits exceed what the
+// last-level cache holds, so they are read with the non-temporal hint.
 typedef float floatx4u __attribute__((ext_vector_type(4), aligned(4)));
+typedef int intx4 __attribute__((ext_vector_type(4)));
+constexpr int kOutOfRange = (int)0x80000000;  // an offset outside every buffer resource
 template <int kVecs>
 __device__ __forceinline__ float row_entry(const floatx4u (&v)[kVecs], int c) {
   // c is wave-uniform and inside the row
@@ -119,76 +141,129 @@ __device__ __forceinline__ float row_entry(const floatx4u (&v)[kVecs], int c) {
     for (int k = 0; k < 4; ++k) cand = (i == vec && k == e) ? v[i][k] : cand;
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(cand), owner));
 }
-template <int kVecs>
+__device__ __forceinline__ floatx4u as_floats(intx4 raw) {
+  return floatx4u{__int_as_float(raw[0]), __int_as_float(raw[1]), __int_as_float(raw[2]),
+                  __int_as_float(raw[3])};
+}
+// which rows of the wave's group need work (bit r), wave-uniform
+template <int kRows>
+__device__ __forceinline__ unsigned live_rows(long first, long rows, const int64_t *ranges,
+                                              const int64_t *window, int T, int Rr) {
+  unsigned live = 0;
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) {
+    const long row = first + r;
+    if (row >= rows) break;
+    bool needed = true;
+    if (window)
+      needed = !outside_window(window, (int)(row / ((long)Rr * T)), (int)((row / Rr) % T),
+                               ranges ? ranges[row] : row % Rr);
+    live |= needed ? 1u << r : 0u;
+  }
+  return live;
+}
+template <int kVecs, int kRows, bool kStream>
 __global__ void __launch_bounds__(256)
     row_norm_regs_kernel(const float *__restrict__ logits, const int64_t *__restrict__ symbols,
-                         const int64_t *__restrict__ ranges, float *__restrict__ norm,
+                         const int64_t *__restrict__ ranges,
+                         const int64_t *__restrict__ window, float *__restrict__ norm,
                          float *__restrict__ xr, float *__restrict__ yr, long rows, int T, int Rr,
                          int S, int C, int term) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // in a scalar register
-  const long row = (long)blockIdx.x * 4 + wave;
+  const long first = ((long)blockIdx.x * 4 + wave) * kRows;
   const int lane = threadIdx.x & 63;
-  if (row >= rows) return;
-  const float *x = logits + row * C;
+  if (first >= rows) return;
+  const unsigned live = live_rows<kRows>(first, rows, ranges, window, T, Rr);
+  if (live == 0) return;
+  const long here = rows - first < kRows ? rows - first : kRows;
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float *>(logits + first * C), 0, (int)(here * C * 4), 0x00020000);
+  constexpr int kAux = kStream ? 2 : 0;
+  floatx4u v[kRows][kVecs];
+#pragma unroll
+  for (int r = 0; r < kRows; ++r)
+#pragma unroll
+    for (int i = 0; i < kVecs; ++i) {
+      const int c = 4 * (lane + kWave * i);
+      const bool wanted = ((live >> r) & 1) && c < C;
+      v[r][i] = as_floats(
+          __builtin_amdgcn_raw_buffer_load_b128(rs, wanted ? (r * C + c) * 4 : kOutOfRange, 0, kAux));
+    }
   const float ninf = -__builtin_huge_valf();
-  floatx4u v[kVecs];
 #pragma unroll
-  for (int i = 0; i < kVecs; ++i) {
-    const int c = 4 * (lane + kWave * i);
-    v[i] = floatx4u{ninf, ninf, ninf, ninf};
-    if (c < C) v[i] = *reinterpret_cast<const floatx4u *>(x + c);
-  }
-  const int j = (int)(row % Rr);
-  const int b = (int)(row / ((long)Rr * T));
-  const int64_t sym = row_symbol(symbols, ranges, row, b, j, S, term);
-  float m = ninf;
+  for (int r = 0; r < kRows; ++r) {
+    if (!((live >> r) & 1)) continue;  // wave-uniform
+    const long row = first + r;
+    // what lies past the end of the row takes no part
 #pragma unroll
-  for (int i = 0; i < kVecs; ++i)
+    for (int i = 0; i < kVecs; ++i)
+      if (4 * (lane + kWave * i) >= C) v[r][i] = floatx4u{ninf, ninf, ninf, ninf};
+    const int j = (int)(row % Rr);
+    const int b = (int)(row / ((long)Rr * T));
+    const int64_t sym = row_symbol(symbols, ranges, row, b, j, S, term);
+    float m = ninf;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) m = (v[i][e] > m || v[i][e] != v[i][e]) ? v[i][e] : m;
-  m = wave_max_all(m);
-  const float shift = (m - m == 0) ? m : 0.f;  // torch.logsumexp: infinite max -> shift by 0
-  float sum = 0;
+    for (int i = 0; i < kVecs; ++i)
 #pragma unroll
-  for (int i = 0; i < kVecs; ++i)
+      for (int e = 0; e < 4; ++e) m = (v[r][i][e] > m || v[r][i][e] != v[r][i][e]) ? v[r][i][e] : m;
+    m = wave_max_all(m);
+    const float shift = (m - m == 0) ? m : 0.f;  // torch.logsumexp: infinite max -> shift by 0
+    float sum = 0;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) sum += __expf(v[i][e] - shift);  // padding is -inf: adds 0
-  sum = wave_sum_all(sum);
-  const float lse = logf(sum) + shift;
-  const float at_sym = (sym >= 0 && sym < C) ? row_entry<kVecs>(v, (int)sym) - lse
-                                             : std::numeric_limits<float>::quiet_NaN();
-  const float at_term = row_entry<kVecs>(v, term) - lse;
-  if (lane == 0) {
-    norm[row] = lse;
-    xr[row] = at_sym;
-    yr[row] = at_term;
+    for (int i = 0; i < kVecs; ++i)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sum += __expf(v[r][i][e] - shift);  // padding is -inf: adds 0
+    sum = wave_sum_all(sum);
+    const float lse = logf(sum) + shift;
+    const float at_sym = (sym >= 0 && sym < C) ? row_entry<kVecs>(v[r], (int)sym) - lse
+                                               : std::numeric_limits<float>::quiet_NaN();
+    const float at_term = row_entry<kVecs>(v[r], term) - lse;
+    if (lane == 0) {
+      norm[row] = lse;
+      xr[row] = at_sym;
+      yr[row] = at_term;
+    }
   }
 }
 
+// Logits beyond this many bytes do not stay in the last-level cache between the forward
+// and the backward pass: they are streamed (non-temporal hint), which leaves the cache to
+// what is used again.  Below it the hint costs (a 80 MB gradient pass: 23.8 -> 26.6 us).
+constexpr long kStreamBytes = 192L << 20;
+
 template <typename R>
-bool launch_row_norm_regs(const R *, const int64_t *, const int64_t *, R *, R *, R *, long, int, int,
-                          int, int, int, hipStream_t) {
+bool launch_row_norm_regs(const R *, const int64_t *, const int64_t *, const int64_t *, R *, R *,
+                          R *, long, int, int, int, int, int, hipStream_t) {
   return false;
 }
 template <>
 bool launch_row_norm_regs<float>(const float *logits, const int64_t *symbols, const int64_t *ranges,
-                                 float *norm, float *xr, float *yr, long rows, int T, int Rr, int S,
-                                 int C, int term, hipStream_t stream) {
+                                 const int64_t *window, float *norm, float *xr, float *yr, long rows,
+                                 int T, int Rr, int S, int C, int term, hipStream_t stream) {
   if (C % 4 != 0 || C > 256 * 16) return false;
-  const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
-#define FRNNT_ROW_NORM(V)                                                                        \
-  hipLaunchKernelGGL(row_norm_regs_kernel<V>, grid, block, 0, stream, logits, symbols, ranges,   \
-                     norm, xr, yr, rows, T, Rr, S, C, term)
+  const bool big = rows * C * 4 > kStreamBytes;
+#define FRNNT_ROW_NORM(V, N)                                                                     \
+  do {                                                                                           \
+    const dim3 grid((unsigned)((rows + 4 * N - 1) / (4 * N))), block(256);                       \
+    if (big)                                                                                     \
+      hipLaunchKernelGGL((row_norm_regs_kernel<V, N, true>), grid, block, 0, stream, logits,     \
+                         symbols, ranges, window, norm, xr, yr, rows, T, Rr, S, C, term);        \
+    else                                                                                         \
+      hipLaunchKernelGGL((row_norm_regs_kernel<V, N, false>), grid, block, 0, stream, logits,    \
+                         symbols, ranges, window, norm, xr, yr, rows, T, Rr, S, C, term);        \
+  } while (0)
+  // (one row per wave: two or four rows per wave were measured 3 to 10 % slower on
+  // 390 MB and on 80 MB of logits)
   if (C <= 256)
-    FRNNT_ROW_NORM(1);
+    FRNNT_ROW_NORM(1, 1);
   else if (C <= 512)
-    FRNNT_ROW_NORM(2);
+    FRNNT_ROW_NORM(2, 1);
   else if (C <= 1024)
-    FRNNT_ROW_NORM(4);
+    FRNNT_ROW_NORM(4, 1);
   else if (C <= 2048)
-    FRNNT_ROW_NORM(8);
+    FRNNT_ROW_NORM(8, 1);
   else
-    FRNNT_ROW_NORM(16);
+    FRNNT_ROW_NORM(16, 1);
 #undef FRNNT_ROW_NORM
   return true;
 }
@@ -238,12 +313,18 @@ template <typename R>
 __global__ void __launch_bounds__(256)
     row_grad_kernel(const R *__restrict__ logits, const int64_t *__restrict__ symbols,
                     const int64_t *__restrict__ ranges, const int64_t *__restrict__ boundary,
-                    const R *__restrict__ norm, const R *__restrict__ gpx,
-                    const R *__restrict__ gpy, R *__restrict__ glogits, long rows, int S, int T,
-                    int Rr, int C, int term, int rnnt_type) {
+                    const int64_t *__restrict__ window, const R *__restrict__ norm,
+                    const R *__restrict__ gpx, const R *__restrict__ gpy, R *__restrict__ glogits,
+                    long rows, int S, int T, int Rr, int C, int term, int rnnt_type) {
   const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (row >= rows) return;
+  if (window &&
+      outside_window(window, (int)(row / ((long)Rr * T)), (int)((row / Rr) % T),
+                     ranges ? ranges[row] : row % Rr)) {
+    for (int c = lane; c < C; c += kWave) glogits[row * C + c] = 0;
+    return;
+  }
   const int S1 = S + 1;
   const int T1 = rnnt_type == kRegular ? T + 1 : T;
   const int j = (int)(row % Rr);
@@ -276,91 +357,123 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-// The same with the row held in registers (fp32, C a multiple of 4, at most
-// 256 * kVecs entries): the logits are requested first, 16 bytes per lane and load,
-// so that they travel while the row's scalars (range, gradients, normalizer) are
-// looked up; the gradient leaves as 16-byte stores.
-template <int kVecs>
+// The same with the rows held in registers (fp32, C a multiple of 4, at most
+// 256 * kVecs entries), kRows consecutive rows per wave as in row_norm_regs_kernel: every
+// load of every row is in flight (branch-free, through a buffer resource over the wave's
+// rows) while the rows' scalars (range, gradients, normalizer) are looked up; the gradient
+// leaves as 16-byte stores.  A row outside the window (when the caller says the gradients
+// vanish there) is not read: exact zeros are stored.
+template <int kVecs, int kRows, bool kStream>
 __global__ void __launch_bounds__(256)
     row_grad_regs_kernel(const float *__restrict__ logits, const int64_t *__restrict__ symbols,
                          const int64_t *__restrict__ ranges, const int64_t *__restrict__ boundary,
-                         const float *__restrict__ norm, const float *__restrict__ gpx,
-                         const float *__restrict__ gpy, float *__restrict__ glogits, long rows,
-                         int S, int T, int Rr, int C, int term, int rnnt_type) {
-  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+                         const int64_t *__restrict__ window, const float *__restrict__ norm,
+                         const float *__restrict__ gpx, const float *__restrict__ gpy,
+                         float *__restrict__ glogits, long rows, int S, int T, int Rr, int C,
+                         int term, int rnnt_type) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // in a scalar register
+  const long first = ((long)blockIdx.x * 4 + wave) * kRows;
   const int lane = threadIdx.x & 63;
-  if (row >= rows) return;
-  const float *x = logits + row * C;
-  floatx4u v[kVecs];
+  if (first >= rows) return;
+  const unsigned live = live_rows<kRows>(first, rows, ranges, window, T, Rr);
+  const long here = rows - first < kRows ? rows - first : kRows;
+  const __amdgpu_buffer_rsrc_t in_rs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float *>(logits + first * C), 0, (int)(here * C * 4), 0x00020000);
+  const __amdgpu_buffer_rsrc_t out_rs =
+      __builtin_amdgcn_make_buffer_rsrc(glogits + first * C, 0, (int)(here * C * 4), 0x00020000);
+  constexpr int kAux = kStream ? 2 : 0;
+  floatx4u v[kRows][kVecs];
 #pragma unroll
-  for (int i = 0; i < kVecs; ++i) {
-    const int c = 4 * (lane + kWave * i);
-    v[i] = floatx4u{0.f, 0.f, 0.f, 0.f};
-    if (c < C) v[i] = *reinterpret_cast<const floatx4u *>(x + c);
-  }
+  for (int r = 0; r < kRows; ++r)
+#pragma unroll
+    for (int i = 0; i < kVecs; ++i) {
+      const int c = 4 * (lane + kWave * i);
+      const bool wanted = ((live >> r) & 1) && c < C;
+      v[r][i] = as_floats(
+          __builtin_amdgcn_raw_buffer_load_b128(in_rs, wanted ? (r * C + c) * 4 : kOutOfRange, 0, kAux));
+    }
   const int S1 = S + 1;
   const int T1 = rnnt_type == kRegular ? T + 1 : T;
-  const int j = (int)(row % Rr);
-  const long frame = row / Rr;
-  const int t = (int)(frame % T), b = (int)(frame / T);
-  const int64_t r0 = ranges ? ranges[frame * Rr] : 0;
-  int64_t s64 = ((int64_t)j + r0) % S1;
-  if (s64 < 0) s64 += S1;
-  const int s = (int)s64;
-  const bool masked = rnnt_type == kRegular && boundary && boundary[4 * b + 3] == t;
-  auto gx_at = [&](int ss) -> float {
-    if (ss < 0 || ss >= S || masked) return 0.f;
-    return gpx[((long)b * S + ss) * T1 + t];
-  };
-  const float gx = gx_at(s);
-  float gy = gpy[((long)b * S1 + s) * T + t];
-  if (rnnt_type == kConstrained) gy += gx_at(s - 1);
-  const int sym = (int)row_symbol(symbols, ranges, row, b, j, S, term);
-  const float lse = norm[row];
-  const float w = -(gx + gy);
-  float *g = glogits + row * C;
 #pragma unroll
-  for (int i = 0; i < kVecs; ++i) {
-    const int c = 4 * (lane + kWave * i);
-    if (c >= C) continue;
-    floatx4u o;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float r = __expf(v[i][e] - lse) * w;
-      if (c + e == sym) r += gx;
-      if (c + e == term) r += gy;
-      o[e] = r;
+  for (int r = 0; r < kRows; ++r) {
+    const long row = first + r;
+    if (row >= rows) break;
+    float gx = 0.f, gy = 0.f, lse = 0.f;
+    int sym = -1;
+    if ((live >> r) & 1) {  // wave-uniform
+      const int j = (int)(row % Rr);
+      const long frame = row / Rr;
+      const int t = (int)(frame % T), b = (int)(frame / T);
+      const int64_t r0 = ranges ? ranges[frame * Rr] : 0;
+      int64_t s64 = ((int64_t)j + r0) % S1;
+      if (s64 < 0) s64 += S1;
+      const int s = (int)s64;
+      const bool masked = rnnt_type == kRegular && boundary && boundary[4 * b + 3] == t;
+      auto gx_at = [&](int ss) -> float {
+        if (ss < 0 || ss >= S || masked) return 0.f;
+        return gpx[((long)b * S + ss) * T1 + t];
+      };
+      gx = gx_at(s);
+      gy = gpy[((long)b * S1 + s) * T + t];
+      if (rnnt_type == kConstrained) gy += gx_at(s - 1);
+      sym = (int)row_symbol(symbols, ranges, row, b, j, S, term);
+      lse = norm[row];
     }
-    *reinterpret_cast<floatx4u *>(g + c) = o;
+    const float w = -(gx + gy);
+    const bool zero = !((live >> r) & 1);
+#pragma unroll
+    for (int i = 0; i < kVecs; ++i) {
+      const int c = 4 * (lane + kWave * i);
+      intx4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float g = __expf(v[r][i][e] - lse) * w;
+        if (c + e == sym) g += gx;
+        if (c + e == term) g += gy;
+        o[e] = zero ? 0 : __float_as_int(g);  // (term may equal an entry of a skipped row)
+      }
+      __builtin_amdgcn_raw_buffer_store_b128(o, out_rs, c < C ? (r * C + c) * 4 : kOutOfRange, 0,
+                                             kAux);
+    }
   }
 }
 
 template <typename R>
-bool launch_row_grad_regs(const R *, const int64_t *, const int64_t *, const int64_t *, const R *,
-                          const R *, const R *, R *, long, int, int, int, int, int, int,
-                          hipStream_t) {
+bool launch_row_grad_regs(const R *, const int64_t *, const int64_t *, const int64_t *,
+                          const int64_t *, const R *, const R *, const R *, R *, long, int, int, int,
+                          int, int, int, hipStream_t) {
   return false;
 }
 template <>
 bool launch_row_grad_regs<float>(const float *logits, const int64_t *symbols, const int64_t *ranges,
-                                 const int64_t *boundary, const float *norm, const float *gpx,
-                                 const float *gpy, float *glogits, long rows, int S, int T, int Rr,
-                                 int C, int term, int rnnt_type, hipStream_t stream) {
+                                 const int64_t *boundary, const int64_t *window, const float *norm,
+                                 const float *gpx, const float *gpy, float *glogits, long rows,
+                                 int S, int T, int Rr, int C, int term, int rnnt_type,
+                                 hipStream_t stream) {
   if (C % 4 != 0 || C > 256 * 16) return false;
-  const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
-#define FRNNT_ROW_GRAD(V)                                                                        \
-  hipLaunchKernelGGL(row_grad_regs_kernel<V>, grid, block, 0, stream, logits, symbols, ranges,   \
-                     boundary, norm, gpx, gpy, glogits, rows, S, T, Rr, C, term, rnnt_type)
+  const bool big = rows * C * 4 > kStreamBytes;
+#define FRNNT_ROW_GRAD(V, N)                                                                     \
+  do {                                                                                           \
+    const dim3 grid((unsigned)((rows + 4 * N - 1) / (4 * N))), block(256);                       \
+    if (big)                                                                                     \
+      hipLaunchKernelGGL((row_grad_regs_kernel<V, N, true>), grid, block, 0, stream, logits,     \
+                         symbols, ranges, boundary, window, norm, gpx, gpy, glogits, rows, S, T, \
+                         Rr, C, term, rnnt_type);                                                \
+    else                                                                                         \
+      hipLaunchKernelGGL((row_grad_regs_kernel<V, N, false>), grid, block, 0, stream, logits,    \
+                         symbols, ranges, boundary, window, norm, gpx, gpy, glogits, rows, S, T, \
+                         Rr, C, term, rnnt_type);                                                \
+  } while (0)
   if (C <= 256)
-    FRNNT_ROW_GRAD(1);
+    FRNNT_ROW_GRAD(1, 1);
   else if (C <= 512)
-    FRNNT_ROW_GRAD(2);
+    FRNNT_ROW_GRAD(2, 1);
   else if (C <= 1024)
-    FRNNT_ROW_GRAD(4);
+    FRNNT_ROW_GRAD(4, 1);
   else if (C <= 2048)
-    FRNNT_ROW_GRAD(8);
+    FRNNT_ROW_GRAD(8, 1);
   else
-    FRNNT_ROW_GRAD(16);
+    FRNNT_ROW_GRAD(16, 1);
 #undef FRNNT_ROW_GRAD
   return true;
 }
@@ -368,7 +481,7 @@ bool launch_row_grad_regs<float>(const float *logits, const int64_t *symbols, co
 template <typename R>
 int fwd_impl(const R *logits, const int64_t *symbols, const int64_t *ranges,
              const int64_t *boundary, R *px, R *py, R *norm, R *xr, R *yr, int B, int S, int T,
-             int Rr, int C, int term, int rnnt_type, void *stream_) {
+             int Rr, int C, int term, int rnnt_type, int window_only, void *stream_) {
   if (B < 0 || S < 0 || T < 0 || Rr < 1 || C < 1)
     return fail(FRNNT_EINVAL, "lattice_logprobs_fwd: bad size");
   if (Rr > S + 1) return fail(FRNNT_EINVAL, "lattice_logprobs_fwd: more range rows than S + 1");
@@ -381,11 +494,13 @@ int fwd_impl(const R *logits, const int64_t *symbols, const int64_t *ranges,
     return fail(FRNNT_EINVAL, "lattice_logprobs_fwd: null pointer");
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   const long rows = (long)B * T * Rr;
+  const int64_t *window = window_only ? boundary : nullptr;
   if (rows > 0)
-    if (!launch_row_norm_regs<R>(logits, symbols, ranges, norm, xr, yr, rows, T, Rr, S, C, term,
-                                 stream))
+    if (!launch_row_norm_regs<R>(logits, symbols, ranges, window, norm, xr, yr, rows, T, Rr, S, C,
+                                 term, stream))
       hipLaunchKernelGGL(row_norm_kernel<R>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
-                         stream, logits, symbols, ranges, norm, xr, yr, rows, T, Rr, S, C, term);
+                         stream, logits, symbols, ranges, window, norm, xr, yr, rows, T, Rr, S, C,
+                         term);
   const int T1 = rnnt_type == kRegular ? T + 1 : T;
   const long total = (long)B * S * T1 + (long)B * (S + 1) * T;
   if (total > 0)
@@ -398,7 +513,7 @@ template <typename R>
 int bwd_impl(const R *logits, const int64_t *symbols, const int64_t *ranges,
              const int64_t *boundary, const R *norm, const R *px_grad, const R *py_grad,
              R *logits_grad, int B, int S, int T, int Rr, int C, int term, int rnnt_type,
-             void *stream_) {
+             int window_only, void *stream_) {
   if (B < 0 || S < 0 || T < 0 || Rr < 1 || C < 1 || Rr > S + 1 || (!ranges && Rr != S + 1))
     return fail(FRNNT_EINVAL, "lattice_logprobs_bwd: bad size");
   if (rnnt_type < 0 || rnnt_type > 2 || term < 0 || term >= C)
@@ -407,12 +522,13 @@ int bwd_impl(const R *logits, const int64_t *symbols, const int64_t *ranges,
   if (!logits || (!symbols && S > 0) || !norm || !px_grad || !py_grad || !logits_grad)
     return fail(FRNNT_EINVAL, "lattice_logprobs_bwd: null pointer");
   const long rows = (long)B * T * Rr;
-  if (!launch_row_grad_regs<R>(logits, symbols, ranges, boundary, norm, px_grad, py_grad,
+  const int64_t *window = window_only ? boundary : nullptr;
+  if (!launch_row_grad_regs<R>(logits, symbols, ranges, boundary, window, norm, px_grad, py_grad,
                                logits_grad, rows, S, T, Rr, C, term, rnnt_type,
                                static_cast<hipStream_t>(stream_)))
     hipLaunchKernelGGL(row_grad_kernel<R>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
-                       static_cast<hipStream_t>(stream_), logits, symbols, ranges, boundary, norm,
-                       px_grad, py_grad, logits_grad, rows, S, T, Rr, C, term, rnnt_type);
+                       static_cast<hipStream_t>(stream_), logits, symbols, ranges, boundary, window,
+                       norm, px_grad, py_grad, logits_grad, rows, S, T, Rr, C, term, rnnt_type);
   return check_launch("lattice_logprobs_bwd");
 }
 
@@ -425,35 +541,37 @@ int frnnt_lattice_logprobs_fwd_f32(const float *logits, const int64_t *symbols,
                                    const int64_t *ranges, const int64_t *boundary, float *px,
                                    float *py, float *norm, float *xr, float *yr, int B, int S,
                                    int T, int R, int C, int termination_symbol, int rnnt_type,
-                                   void *stream) {
+                                   int window_only, void *stream) {
   return frnnt::fwd_impl<float>(logits, symbols, ranges, boundary, px, py, norm, xr, yr, B, S, T, R,
-                                C, termination_symbol, rnnt_type, stream);
+                                C, termination_symbol, rnnt_type, window_only, stream);
 }
 int frnnt_lattice_logprobs_fwd_f64(const double *logits, const int64_t *symbols,
                                    const int64_t *ranges, const int64_t *boundary, double *px,
                                    double *py, double *norm, double *xr, double *yr, int B, int S,
                                    int T, int R, int C, int termination_symbol, int rnnt_type,
-                                   void *stream) {
+                                   int window_only, void *stream) {
   return frnnt::fwd_impl<double>(logits, symbols, ranges, boundary, px, py, norm, xr, yr, B, S, T,
-                                 R, C, termination_symbol, rnnt_type, stream);
+                                 R, C, termination_symbol, rnnt_type, window_only, stream);
 }
 int frnnt_lattice_logprobs_bwd_f32(const float *logits, const int64_t *symbols,
                                    const int64_t *ranges, const int64_t *boundary,
                                    const float *norm, const float *px_grad, const float *py_grad,
                                    float *logits_grad, int B, int S, int T, int R, int C,
-                                   int termination_symbol, int rnnt_type, void *stream) {
+                                   int termination_symbol, int rnnt_type, int window_only,
+                                   void *stream) {
   return frnnt::bwd_impl<float>(logits, symbols, ranges, boundary, norm, px_grad, py_grad,
-                                logits_grad, B, S, T, R, C, termination_symbol, rnnt_type, stream);
+                                logits_grad, B, S, T, R, C, termination_symbol, rnnt_type,
+                                window_only, stream);
 }
 int frnnt_lattice_logprobs_bwd_f64(const double *logits, const int64_t *symbols,
                                    const int64_t *ranges, const int64_t *boundary,
                                    const double *norm, const double *px_grad,
                                    const double *py_grad, double *logits_grad, int B, int S, int T,
                                    int R, int C, int termination_symbol, int rnnt_type,
-                                   void *stream) {
+                                   int window_only, void *stream) {
   return frnnt::bwd_impl<double>(logits, symbols, ranges, boundary, norm, px_grad, py_grad,
                                  logits_grad, B, S, T, R, C, termination_symbol, rnnt_type,
-                                 stream);
+                                 window_only, stream);
 }
 
 }  // extern "C"

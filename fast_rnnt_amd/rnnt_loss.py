@@ -20,7 +20,8 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from .mutual_information import boundary_rows, mutual_information_recursion
+from .mutual_information import (_assert_boundary, boundary_rows,
+                                 mutual_information_recursion)
 
 _RNNT_TYPES = {"regular": 0, "modified": 1, "constrained": 2}
 
@@ -357,7 +358,10 @@ class _LatticeLogprobs(torch.autograd.Function):
     frnnt_lattice_logprobs_fwd/bwd."""
 
     @staticmethod
-    def forward(ctx, logits, symbols, ranges, boundary, termination_symbol, rnnt_type):
+    def forward(ctx, logits, symbols, ranges, boundary, termination_symbol, rnnt_type,
+                window_only=False):
+        # window_only: the caller feeds (px, py) to the recursion with this same boundary,
+        # so cells outside each utterance's window may stay undefined and carry no gradient
         B, T, R, C = logits.shape
         S = symbols.shape[1]
         kind = _RNNT_TYPES[rnnt_type]
@@ -368,6 +372,7 @@ class _LatticeLogprobs(torch.autograd.Function):
         bnd_c = boundary.contiguous() if boundary is not None else None
         opts = dict(dtype=logits.dtype, device=logits.device)
         T1 = T + 1 if kind == 0 else T
+        windowed = bool(window_only) and bnd_c is not None
         with torch.cuda.device(logits.device):
             px = torch.empty(B, S, T1, **opts)
             py = torch.empty(B, S + 1, T, **opts)
@@ -377,16 +382,16 @@ class _LatticeLogprobs(torch.autograd.Function):
             _lib.call("frnnt_lattice_logprobs_fwd_" + sfx, lg.data_ptr(), sym_c.data_ptr(),
                       _lib.ptr(rng_c), _lib.ptr(bnd_c), px.data_ptr(), py.data_ptr(),
                       norm.data_ptr(), xr.data_ptr(), yr.data_ptr(), B, S, T, R, C,
-                      int(termination_symbol), kind, _lib.stream_of(logits))
+                      int(termination_symbol), kind, int(windowed), _lib.stream_of(logits))
         if ctx.needs_input_grad[0]:
             ctx.save_for_backward(lg, sym_c, rng_c, bnd_c, norm)
-            ctx.meta = (B, S, T, R, C, int(termination_symbol), kind, sfx)
+            ctx.meta = (B, S, T, R, C, int(termination_symbol), kind, sfx, int(windowed))
         return px, py
 
     @staticmethod
     def backward(ctx, gpx, gpy):
         lg, sym, rng, bnd, norm = ctx.saved_tensors
-        B, S, T, R, C, term, kind, sfx = ctx.meta
+        B, S, T, R, C, term, kind, sfx, windowed = ctx.meta
         opts = dict(dtype=lg.dtype, device=lg.device)
         T1 = T + 1 if kind == 0 else T
         with torch.cuda.device(lg.device):
@@ -395,9 +400,23 @@ class _LatticeLogprobs(torch.autograd.Function):
             grad = torch.empty_like(lg)
             _lib.call("frnnt_lattice_logprobs_bwd_" + sfx, lg.data_ptr(), sym.data_ptr(),
                       _lib.ptr(rng), _lib.ptr(bnd), norm.data_ptr(), gpx.data_ptr(),
-                      gpy.data_ptr(), grad.data_ptr(), B, S, T, R, C, term, kind,
+                      gpy.data_ptr(), grad.data_ptr(), B, S, T, R, C, term, kind, windowed,
                       _lib.stream_of(lg))
-        return grad, None, None, None, None, None
+        return grad, None, None, None, None, None, None
+
+
+def _joint_logprobs(logits, symbols, termination_symbol, boundary, rnnt_type, window_only):
+    assert logits.ndim == 4, logits.ndim
+    (B, T, S1, C) = logits.shape
+    S = S1 - 1
+    assert symbols.shape == (B, S), symbols.shape
+    validate_st_lengths(S, T, rnnt_type == "regular", boundary)
+    assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
+    _check_tensors([("logits", logits)], [("symbols", symbols), ("boundary", boundary)])
+    if window_only and boundary is not None:
+        _assert_boundary(boundary, B, S, T)
+    return _LatticeLogprobs.apply(logits, symbols, None, boundary, termination_symbol, rnnt_type,
+                                  window_only)
 
 
 def get_rnnt_logprobs_joint(
@@ -406,14 +425,7 @@ def get_rnnt_logprobs_joint(
 ) -> Tuple[Tensor, Tensor]:
     """(px, py) from the full joiner output ``logits`` of shape ``(B, T, S+1, C)``
     (fast_rnnt/python/fast_rnnt/rnnt_loss.py:343-449)."""
-    assert logits.ndim == 4, logits.ndim
-    (B, T, S1, C) = logits.shape
-    S = S1 - 1
-    assert symbols.shape == (B, S), symbols.shape
-    validate_st_lengths(S, T, rnnt_type == "regular", boundary)
-    assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
-    _check_tensors([("logits", logits)], [("symbols", symbols), ("boundary", boundary)])
-    return _LatticeLogprobs.apply(logits, symbols, None, boundary, termination_symbol, rnnt_type)
+    return _joint_logprobs(logits, symbols, termination_symbol, boundary, rnnt_type, False)
 
 
 def rnnt_loss(
@@ -421,10 +433,10 @@ def rnnt_loss(
     boundary: Optional[Tensor] = None, rnnt_type: str = "regular",
     delay_penalty: float = 0.0, reduction: Optional[str] = "mean", return_grad: bool = False,
 ) -> Tensor:
-    """The unpruned RNN-T loss on joiner logits ``(B, T, S+1, C)`` (rnnt_loss.py:452-547)."""
-    px, py = get_rnnt_logprobs_joint(logits=logits, symbols=symbols,
-                                     termination_symbol=termination_symbol,
-                                     boundary=boundary, rnnt_type=rnnt_type)
+    """The unpruned RNN-T loss on joiner logits ``(B, T, S+1, C)`` (rnnt_loss.py:452-547).
+    The logits of cells outside an utterance's boundary window are not read: the
+    recursion never visits them and their gradient is exactly zero."""
+    px, py = _joint_logprobs(logits, symbols, termination_symbol, boundary, rnnt_type, True)
     return _recursion_and_reduce(px, py, boundary, rnnt_type, delay_penalty, reduction,
                                  return_grad)
 
@@ -552,13 +564,8 @@ def _roll_by_shifts(src: Tensor, shifts: torch.LongTensor):
     return torch.gather(src, 2, index)
 
 
-def get_rnnt_logprobs_pruned(
-    logits: Tensor, symbols: Tensor, ranges: Tensor, termination_symbol: int,
-    boundary: Optional[Tensor] = None, rnnt_type: str = "regular",
-) -> Tuple[Tensor, Tensor]:
-    """(px, py) from pruned joiner logits ``(B, T, s_range, C)`` and the
-    ``ranges`` they were computed for (rnnt_loss.py:856-1024); lattice cells
-    outside the kept range of their frame are -inf."""
+def _pruned_logprobs(logits, symbols, ranges, termination_symbol, boundary, rnnt_type,
+                     window_only):
     assert logits.ndim == 4, logits.ndim
     (B, T, s_range, C) = logits.shape
     assert ranges.shape == (B, T, s_range), f"{ranges.shape} == ({B}, {T}, {s_range})"
@@ -567,8 +574,21 @@ def get_rnnt_logprobs_pruned(
     assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
     _check_tensors([("logits", logits)],
                    [("symbols", symbols), ("ranges", ranges), ("boundary", boundary)])
+    if window_only and boundary is not None:
+        _assert_boundary(boundary, B, S, T)
     return _LatticeLogprobs.apply(logits, symbols, ranges, boundary, termination_symbol,
-                                  rnnt_type)
+                                  rnnt_type, window_only)
+
+
+def get_rnnt_logprobs_pruned(
+    logits: Tensor, symbols: Tensor, ranges: Tensor, termination_symbol: int,
+    boundary: Optional[Tensor] = None, rnnt_type: str = "regular",
+) -> Tuple[Tensor, Tensor]:
+    """(px, py) from pruned joiner logits ``(B, T, s_range, C)`` and the
+    ``ranges`` they were computed for (rnnt_loss.py:856-1024); lattice cells
+    outside the kept range of their frame are -inf."""
+    return _pruned_logprobs(logits, symbols, ranges, termination_symbol, boundary, rnnt_type,
+                            False)
 
 
 def rnnt_loss_pruned(
@@ -576,10 +596,10 @@ def rnnt_loss_pruned(
     boundary: Optional[Tensor] = None, rnnt_type: str = "regular",
     delay_penalty: float = 0.0, reduction: Optional[str] = "mean", return_grad: bool = False,
 ) -> Tensor:
-    """The pruned RNN-T loss on joiner logits ``(B, T, s_range, C)`` (rnnt_loss.py:1027-1132)."""
-    px, py = get_rnnt_logprobs_pruned(logits=logits, symbols=symbols, ranges=ranges,
-                                      termination_symbol=termination_symbol,
-                                      boundary=boundary, rnnt_type=rnnt_type)
+    """The pruned RNN-T loss on joiner logits ``(B, T, s_range, C)`` (rnnt_loss.py:1027-1132).
+    As in :func:`rnnt_loss`, logits outside an utterance's boundary window are not read."""
+    px, py = _pruned_logprobs(logits, symbols, ranges, termination_symbol, boundary, rnnt_type,
+                              True)
     return _recursion_and_reduce(px, py, boundary, rnnt_type, delay_penalty, reduction,
                                  return_grad)
 

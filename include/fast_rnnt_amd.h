@@ -260,17 +260,25 @@ int frnnt_loss_reduce_f64(const double *scores, double *loss, int B, int reducti
  *   px [B][S][T+1] (rnnt_type 0) or [B][S][T]; py [B][S+1][T]                   out
  *   norm, xr, yr [B][T][R]: out; norm (the logsumexp) is needed by the backward
  *   entry point, xr / yr are staging buffers
+ *   window_only: 0 = every cell of px / py is computed.  1 (needs a boundary) = the caller
+ *   goes on to the lattice recursion with the same boundary, which never looks outside
+ *   utterance b's window [s_begin, s_end] x [t_begin, t_end): logits rows outside it are
+ *   not read and their entries of norm, xr, yr, px, py are left undefined.  The backward
+ *   entry point takes the same flag: such rows then get a gradient of exact zeros without
+ *   being read (the recursion's px_grad / py_grad vanish there).  This is what rnnt_loss
+ *   and rnnt_loss_pruned (rnnt_loss.py:452-547, :1027-1132) use; about a third of the rows
+ *   of a ragged batch lie outside.
  */
 int frnnt_lattice_logprobs_fwd_f32(const float *logits, const int64_t *symbols,
                                    const int64_t *ranges, const int64_t *boundary, float *px,
                                    float *py, float *norm, float *xr, float *yr, int B, int S,
                                    int T, int R, int C, int termination_symbol, int rnnt_type,
-                                   void *stream);
+                                   int window_only, void *stream);
 int frnnt_lattice_logprobs_fwd_f64(const double *logits, const int64_t *symbols,
                                    const int64_t *ranges, const int64_t *boundary, double *px,
                                    double *py, double *norm, double *xr, double *yr, int B, int S,
                                    int T, int R, int C, int termination_symbol, int rnnt_type,
-                                   void *stream);
+                                   int window_only, void *stream);
 
 /*
  * Backward of the above (what autograd derives for rnnt_loss.py:418-447 /
@@ -281,13 +289,14 @@ int frnnt_lattice_logprobs_bwd_f32(const float *logits, const int64_t *symbols,
                                    const int64_t *ranges, const int64_t *boundary,
                                    const float *norm, const float *px_grad, const float *py_grad,
                                    float *logits_grad, int B, int S, int T, int R, int C,
-                                   int termination_symbol, int rnnt_type, void *stream);
+                                   int termination_symbol, int rnnt_type, int window_only,
+                                   void *stream);
 int frnnt_lattice_logprobs_bwd_f64(const double *logits, const int64_t *symbols,
                                    const int64_t *ranges, const int64_t *boundary,
                                    const double *norm, const double *px_grad,
                                    const double *py_grad, double *logits_grad, int B, int S, int T,
                                    int R, int C, int termination_symbol, int rnnt_type,
-                                   void *stream);
+                                   int window_only, void *stream);
 
 /*
  * Pruning bounds.  Replaces the device work of get_rnnt_prune_ranges

@@ -400,6 +400,61 @@ def test_pruned_with_every_row_kept_equals_unpruned(gpu_device, kind):
         assert _close(full.grad, a.grad, 1e-4, 1e-4)
 
 
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_losses_do_not_read_logits_outside_the_window(gpu_device, dtype, kind):
+    # rnnt_loss / rnnt_loss_pruned skip the logits rows of cells outside an utterance's
+    # boundary window: NaN planted there (on the GPU side only) must change nothing -- loss
+    # and in-window gradients as the oracle computes them on clean logits, exact zeros outside
+    dev = gpu_device
+    f32 = dtype == torch.float32
+    for n, (B, S, T, C) in enumerate([(3, 9, 20, 12), (2, 40, 70, 1000), (2, 66, 50, 37)]):
+        if kind != "regular" and T < S:
+            continue
+        am, lm, sym, bnd = _case(400 + n, B, S, T, C, dtype, kind)
+        g = torch.Generator().manual_seed(400 + n)
+        logits = torch.randn(B, T, S + 1, C, generator=g, dtype=dtype)
+        s_idx = torch.arange(S + 1).reshape(1, 1, S + 1)
+        t_idx = torch.arange(T).reshape(1, T, 1)
+        inside = (s_idx <= bnd[:, 2].reshape(B, 1, 1)) & (t_idx < bnd[:, 3].reshape(B, 1, 1))
+        poisoned = torch.where(inside.unsqueeze(3), logits, torch.full_like(logits, float("nan")))
+        _say(f"window-only joint {kind} {dtype} shape{n}: {int((~inside).sum())} of "
+             f"{inside.numel()} rows outside")
+        a = logits.clone().requires_grad_(True)
+        want = O.loss_joint(a, sym, 0, boundary=bnd, rnnt_type=kind, reduction="sum")
+        want.backward()
+        d = poisoned.to(dev).requires_grad_(True)
+        got = fast_rnnt_amd.rnnt_loss(d, sym.to(dev), 0, boundary=bnd.to(dev), rnnt_type=kind,
+                                      reduction="sum")
+        got.backward()
+        assert _close(got, want, 0.0, 1e-5 if f32 else 1e-12)
+        grad = d.grad.cpu()
+        assert bool((grad[~inside] == 0).all())
+        assert _close(grad[inside], a.grad[inside], 1e-4 if f32 else 1e-9, 1e-4 if f32 else 1e-9)
+
+        # pruned: ranges of width 4 following the diagonal, rows past S_b / frames past T_b out
+        R = min(4, S + 1)
+        start = (torch.arange(T).reshape(1, T) * (S + 1 - R) // max(T - 1, 1)).expand(B, T)
+        ranges = (start.unsqueeze(2) + torch.arange(R).reshape(1, 1, R)).contiguous()
+        kept = torch.randn(B, T, R, C, generator=g, dtype=dtype)
+        in_p = (ranges <= bnd[:, 2].reshape(B, 1, 1)) & (t_idx < bnd[:, 3].reshape(B, 1, 1))
+        poisoned = torch.where(in_p.unsqueeze(3), kept, torch.full_like(kept, float("nan")))
+        a = kept.clone().requires_grad_(True)
+        want = O.loss_pruned(a, sym, ranges, 0, boundary=bnd, rnnt_type=kind, reduction="none")
+        live = torch.isfinite(want.detach())   # an arbitrary diagonal band may lose every path
+        want[live].sum().backward()
+        d = poisoned.to(dev).requires_grad_(True)
+        got = fast_rnnt_amd.rnnt_loss_pruned(d, sym.to(dev), ranges.to(dev), 0,
+                                             boundary=bnd.to(dev), rnnt_type=kind,
+                                             reduction="none")
+        got[live.to(dev)].sum().backward()
+        assert torch.equal(torch.isfinite(got.detach().cpu()), live)
+        assert _close(got.detach()[live.to(dev)], want.detach()[live], 0.0, 1e-5 if f32 else 1e-12)
+        grad = d.grad.cpu()
+        assert bool((grad[~in_p] == 0).all())
+        assert _close(grad[in_p], a.grad[in_p], 1e-4 if f32 else 1e-9, 1e-4 if f32 else 1e-9)
+
+
 def test_c5_unpruned_full_size(gpu_device):
     dev = gpu_device
     w = workloads.make("c5")
