@@ -317,7 +317,7 @@ def main():
         stream = torch.cuda.current_stream().cuda_stream
         _lib.call("frnnt_simple_logprobs_fwd_f32", lm_c.data_ptr(), am_c.data_ptr(), sym.data_ptr(),
                   bnd.data_ptr(), px.data_ptr(), py.data_ptr(), lm_max.data_ptr(), am_max.data_ptr(),
-                  norm_raw.data_ptr(), B, S, T, C, 0, 0, stream)
+                  norm_raw.data_ptr(), B, S, T, C, 0, 0, 1, stream)
         gpx, gpy = torch.rand_like(px), torch.rand_like(py)
         dmat = torch.empty(B, S + 1, (T + 3) // 4 * 4, **f32)
         row_x, row_y = torch.empty(B, S + 1, **f32), torch.empty(B, S + 1, **f32)
@@ -330,7 +330,7 @@ def main():
                       norm_raw.data_ptr(), None, 0, 1.0, gpx.data_ptr(), gpy.data_ptr(),
                       dmat.data_ptr(), row_x.data_ptr(), row_y.data_ptr(), col_y.data_ptr(),
                       lm_grad.data_ptr() if want_lm else None,
-                      am_grad.data_ptr() if want_am else None, B, S, T, C, 0, 0, stream)
+                      am_grad.data_ptr() if want_am else None, B, S, T, C, 0, 0, 1, stream)
 
         t_prep = _event_time_ms(lambda: grads(False, False), args.kernel_reps)
         one_launch = float(B) * (S + 1) * T * C < 1e9  # the library's rule for a single launch

@@ -30,6 +30,26 @@ namespace {
 
 enum { kRegular = 0, kModified = 1, kConstrained = 2 };
 
+// What the lattice recursion uses of utterance b: rows [s_begin, s_end] and frames
+// [t_begin, t_end) of py, rows [s_begin, s_end) of px.  A caller that goes on to the
+// recursion with the same boundary passes it as `window`: the kernels then leave px / py /
+// the normalizers outside it undefined, and take the gradients to vanish there (the
+// recursion writes exact zeros).  Without a window everything counts.
+struct Limits {
+  int s_begin, t_begin, s_end, t_end;
+};
+__device__ __forceinline__ Limits limits_of(const int64_t *window, int b, int S, int T) {
+  Limits w{0, 0, S, T};
+  if (window) {
+    // clamped: a boundary row outside the lattice must not widen any loop
+    w.s_begin = (int)max((int64_t)0, min(window[4 * b + 0], (int64_t)S));
+    w.t_begin = (int)max((int64_t)0, min(window[4 * b + 1], (int64_t)T));
+    w.s_end = (int)max((int64_t)0, min(window[4 * b + 2], (int64_t)S));
+    w.t_end = (int)max((int64_t)0, min(window[4 * b + 3], (int64_t)T));
+  }
+  return w;
+}
+
 template <typename R>
 __device__ __forceinline__ R wave_max(R v) {
 #pragma unroll
@@ -174,8 +194,9 @@ template <typename R>
 __global__ void __launch_bounds__(256)
     simple_bwd_prep_kernel(const R *__restrict__ gpx, const R *__restrict__ gpy,
                            const R *__restrict__ norm_raw, const int64_t *__restrict__ boundary,
-                           R *__restrict__ dmat, R *__restrict__ row_x, R *__restrict__ row_y,
-                           R *__restrict__ col_y, int B, int S, int T, int ldd, int rnnt_type) {
+                           const int64_t *__restrict__ window, R *__restrict__ dmat,
+                           R *__restrict__ row_x, R *__restrict__ row_y, R *__restrict__ col_y,
+                           int B, int S, int T, int ldd, int rnnt_type) {
   __shared__ R partial[4][kWave];
   const int S1 = S + 1;
   const int T1 = rnnt_type == kRegular ? T + 1 : T;
@@ -188,6 +209,9 @@ __global__ void __launch_bounds__(256)
     if (row >= n_rows) return;
     const int b = (int)(row / S1), s = (int)(row % S1);
     const int t_mask = (rnnt_type == kRegular && boundary) ? (int)boundary[4 * b + 3] : -1;
+    // outside the window nothing is read (the normalizers there may be undefined): D = 0
+    const Limits lim = limits_of(window, b, S, T);
+    const bool row_in = s >= lim.s_begin && s <= lim.s_end;
     const R *gx_row = s < S ? gpx + ((long)b * S + s) * T1 : nullptr;
     const R *gx_prev = (constrained && s >= 1) ? gpx + ((long)b * S + s - 1) * T1 : nullptr;
     const R *gy_row = gpy + row * T;
@@ -199,7 +223,7 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int t = t0 + u * kWave + lane;
-        const bool ok = t < T;
+        const bool ok = t < T && row_in && t >= lim.t_begin && t < lim.t_end;
         gx[u] = (ok && gx_row && t != t_mask) ? gx_row[t] : (R)0;
         gy[u] = ok ? gy_row[t] : (R)0;
         if (ok && gx_prev && t != t_mask) gy[u] += gx_prev[t];
@@ -224,7 +248,8 @@ __global__ void __launch_bounds__(256)
     const long cb = blockIdx.x - row_blocks;
     const int b = (int)(cb / tiles), t = (int)(cb % tiles) * kWave + lane;
     const int t_mask = (rnnt_type == kRegular && boundary) ? (int)boundary[4 * b + 3] : -1;
-    const bool ok = t < T;
+    const Limits lim = limits_of(window, b, S, T);
+    const bool ok = t < T && t >= lim.t_begin && t < lim.t_end;
     R acc = 0;
     for (int s0 = wave; s0 < S1; s0 += 16) {
       R v[4];
@@ -239,7 +264,7 @@ __global__ void __launch_bounds__(256)
     }
     partial[wave][lane] = acc;
     __syncthreads();
-    if (wave == 0 && ok)
+    if (wave == 0 && t < T)
       col_y[(long)b * T + t] = (partial[0][lane] + partial[1][lane]) + (partial[2][lane] + partial[3][lane]);
   }
 }
@@ -424,8 +449,8 @@ __global__ void __launch_bounds__(kPanThreads)
                             const int64_t *__restrict__ boundary,
                             float *__restrict__ lm_max, float *__restrict__ am_max,
                             float *__restrict__ px, float *__restrict__ py,
-                            float *__restrict__ norm_raw, int B, int S, int T, int C, int term,
-                            int rnnt_type) {
+                            float *__restrict__ norm_raw, const int64_t *__restrict__ window,
+                            int B, int S, int T, int C, int term, int rnnt_type) {
   using Shape = PanelShape<kS, kK>;
   constexpr int kPanS = kS, kPanK = kK, kPanRows = Shape::kRows, kPanPitch = Shape::kPitch;
   constexpr int kPanSlab = Shape::kSlab, kPanItems = Shape::kItems;
@@ -445,6 +470,12 @@ __global__ void __launch_bounds__(kPanThreads)
   if (!decode_block(t_tiles * s_tiles, B, b, tile)) return;
   const int s_tile = (tile / t_tiles) * kPanS, t_tile = (tile % t_tiles) * kPanT;
   const int T1 = rnnt_type == kRegular ? T + 1 : T;
+  // With a window only rows <= s_end and frames <= t_end are looked at afterwards (frame
+  // t_end itself only for the -inf that closes the regular lattice): a tile past t_end has
+  // nothing to do -- except the tiles of frame 0, which also store the row maxima of lm
+  // and the lattice's last column -- and 32-row tiles past s_end are not multiplied.
+  const Limits lim = limits_of(window, b, S, T);
+  if (t_tile > lim.t_end && t_tile > 0) return;
   const float *lmb = lm + (long)b * S1 * C;
   const float *amb = am + (long)b * T * C;
   const int64_t *symb = symbols + (long)b * S;
@@ -555,7 +586,7 @@ __global__ void __launch_bounds__(kPanThreads)
   constexpr float kUnset = 3.0e38f;
 #pragma unroll
   for (int j = 0; j < kLoads; ++j) seen[j] = ninf, shift2[j] = kUnset;
-  const int live_tiles = min(kPanS / 32, (S1 - s_tile + 31) / 32);
+  const int live_tiles = min(kPanS / 32, (min(S1, lim.s_end + 1) - s_tile + 31) / 32);
   float *mine = pan_lds + wave * kPanSlab;
   floatx16 acc[kPanS / 32];
 #pragma unroll
@@ -748,7 +779,8 @@ __device__ __forceinline__ void simple_bwd_lm_slab_body(
     const int64_t *__restrict__ symbols, const float *__restrict__ lm_max,
     const float *__restrict__ am_max, const float *__restrict__ dmat,
     const float *__restrict__ row_x, const float *__restrict__ row_y,
-    float *__restrict__ lm_grad, int B, int S, int T, int C, int ldd, int term) {
+    float *__restrict__ lm_grad, const int64_t *__restrict__ window, int B, int S, int T, int C,
+    int ldd, int term) {
   using Shape = LmShape<kS, kK>;
   constexpr int kLmS = kS, kLmK = kK, kLmPitch = Shape::kPitch, kLmSlab = Shape::kSlab;
   constexpr int kLmItems = Shape::kItems;
@@ -767,6 +799,12 @@ __device__ __forceinline__ void simple_bwd_lm_slab_body(
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int half = lane >> 5, r32 = lane & 31;
+  // With a window, D vanishes at frames >= t_end and on rows > s_end: the sum over frames
+  // stops at t_end (the row maxima of later frames may not even be defined) and 32-row
+  // tiles past s_end are left at 0.
+  const Limits lim = limits_of(window, b, S, T);
+  const int t_lim = __builtin_amdgcn_readfirstlane(lim.t_end);
+  const int s_lim = __builtin_amdgcn_readfirstlane(min(S1, lim.s_end + 1));
 
   // what this lane fetches of every slab: D rows sub_a + kRowsA j at k-offset kq_a; am
   // rows (frames) sub + 8 j at vocabulary offset kq
@@ -797,22 +835,24 @@ __device__ __forceinline__ void simple_bwd_lm_slab_body(
     for (int j = 0; j < kLoadsA; ++j)
       sa[j] = as_floats(__builtin_amdgcn_raw_buffer_load_b128(
           d_rs, d_off + (kRowsA * j * ldd + k0) * 4, 0, 0));
-    if (k0 + kLmK > T) {  // (wave-uniform) the slab that holds frame T - 1
+    if (k0 + kLmK > t_lim) {  // (wave-uniform) the slab that holds the last frame
 #pragma unroll
       for (int j = 0; j < kLoadsA; ++j)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (k0 + kq_a + i >= T) sa[j][i] = 0.f;
+          if (k0 + kq_a + i >= t_lim) sa[j][i] = 0.f;
     }
 #pragma unroll
     for (int j = 0; j < kLoadsB; ++j) {
       const int tr = k0 + sub + 8 * j;
       sb[j] = as_floats(__builtin_amdgcn_raw_buffer_load_b128(
           am_rs, am_off + (k0 + 8 * j) * C * 4, 0, 0));
-      shift2[j] = tr < T ? -amx[tr] * kLog2e : 0.f;
+      shift2[j] = tr < t_lim ? -amx[tr] * kLog2e : 0.f;
+      // a frame past the last one meets D = 0; its factor only has to be finite
+      if (tr >= t_lim) sb[j] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
   };
-  const int chunks = (T + kLmK - 1) / kLmK;
+  const int chunks = (t_lim + kLmK - 1) / kLmK;
   int chunk = wave;
   if (chunk < chunks) fetch(chunk * kLmK);
 
@@ -838,7 +878,7 @@ __device__ __forceinline__ void simple_bwd_lm_slab_body(
     row_ry[j] = ok ? row_y[(long)b * S1 + sr] : 0.f;
   }
 
-  const int live_tiles = min(kLmS / 32, (S1 - s_tile + 31) / 32);  // 32-row tiles with lattice rows
+  const int live_tiles = min(kLmS / 32, (s_lim - s_tile + 31) / 32);  // 32-row tiles with rows that count
   float *as = lm_lds + wave * kLmSlab;
   float *bs = as + kLmS * kLmPitch;
   floatx16 acc[kLmS / 32];
@@ -948,8 +988,9 @@ __device__ __forceinline__ void simple_bwd_am_panel_body(
     const int64_t *__restrict__ symbols, const int64_t *__restrict__ boundary,
     const float *__restrict__ lm_max, const float *__restrict__ am_max,
     const float *__restrict__ dmat, const float *__restrict__ gpx,
-    const float *__restrict__ col_y, float *__restrict__ am_grad, int B, int S, int T, int C,
-    int ldd, int term, int rnnt_type, int rows_cap) {
+    const float *__restrict__ col_y, float *__restrict__ am_grad,
+    const int64_t *__restrict__ window, int B, int S, int T, int C, int ldd, int term,
+    int rnnt_type, int rows_cap) {
   using namespace dgemm;
   extern __shared__ float am_lds[];
   int *sym_s = reinterpret_cast<int *>(am_lds);   // [rows_cap] symbols of the pass (-1: none)
@@ -979,23 +1020,44 @@ __device__ __forceinline__ void simple_bwd_am_panel_body(
   const int c_lo = c_tile + wc;  // first vocabulary column of this wave
   // a thread's 16-byte piece of a 64-wide row: row q_row + 16 * step, columns 4 * q_col ..
   const int q_row = tid / kAmQ, q_col = 4 * (tid % kAmQ);
+  // With a window, D vanishes on rows > s_end and at frames >= t_end, where the frames'
+  // maxima may not even be defined: such frames get exact zeros, the sum over the lattice
+  // rows stops at s_end, and a tile without a frame below t_end only stores zeros.
+  const Limits lim = limits_of(window, b, S, T);
+  const int t_lim = lim.t_end, k_lim = min(S1, lim.s_end + 1);
+  if (t_tile >= t_lim) {
+#pragma unroll
+    for (int j = 0; j < kAmT / 16; ++j) {
+      const int t = t_tile + q_row + 16 * j, c = c_tile + q_col;
+      if (t >= T || c >= C) continue;
+      float *dst = am_grad + ((long)b * T + t) * C + c;
+      if (c + 4 <= C) {
+        *reinterpret_cast<floatx4u *>(dst) = floatx4u{0.f, 0.f, 0.f, 0.f};
+      } else {
+        for (int i = 0; i < 4; ++i)
+          if (c + i < C) dst[i] = 0.f;
+      }
+    }
+    return;
+  }
 
   // epilogue inputs: per-frame terms through LDS (visible after the barriers of the
   // first pass), and this thread's pieces of the am tile, rows q_row + 16 * j
   if (tid < kAmT) {
     const int t = t_tile + tid;
-    shift_s[tid] = t < T ? am_max[(long)b * T + t] : 0.f;
-    extra_s[tid] = t < T ? col_y[(long)b * T + t] : 0.f;
+    shift_s[tid] = t < t_lim ? am_max[(long)b * T + t] : 0.f;
+    extra_s[tid] = t < t_lim ? col_y[(long)b * T + t] : 0.f;
   }
   // The panel and tile loads go through buffer resources that cover D[b], lm[b] and
   // am[b]: one instruction each, no branch, any alignment.  A row past the last one lies
   // past the resource and reads as 0; a column past the end of a row belongs to the next
   // row, and only feeds frames >= T or vocabulary entries >= C, which are never written.
   typedef int intx4 __attribute__((ext_vector_type(4)));
+  // (rows that do not count lie past the resources: they read as 0 and move no data)
   const __amdgpu_buffer_rsrc_t d_rs =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(db), 0, S1 * ldd * 4, 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(db), 0, k_lim * ldd * 4, 0x00020000);
   const __amdgpu_buffer_rsrc_t lm_rs =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(lmb), 0, S1 * C * 4, 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(lmb), 0, k_lim * C * 4, 0x00020000);
   const __amdgpu_buffer_rsrc_t am_rs =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(amb), 0, T * C * 4, 0x00020000);
   auto get4 = [](__amdgpu_buffer_rsrc_t rs, int byte_offset) {
@@ -1011,8 +1073,8 @@ __device__ __forceinline__ void simple_bwd_am_panel_body(
   floatx16 acc, hot;
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = hot[v] = 0.f;
-  for (int k0 = 0; k0 < S1; k0 += rows_cap) {
-    const int rows = min(rows_cap, S1 - k0);
+  for (int k0 = 0; k0 < k_lim; k0 += rows_cap) {
+    const int rows = min(rows_cap, k_lim - k0);
     const int pairs = (rows + 1) / 2;
     constexpr int kSteps = kAmRows / 16;
     floatx4 ra[kSteps], rb[kSteps];
@@ -1111,6 +1173,7 @@ __device__ __forceinline__ void simple_bwd_am_panel_body(
     for (int i = 0; i < 4; ++i) {
       res[i] = __expf(am_in[j][i] - shift) * sum[i] + one[i];
       if (c + i == term) res[i] += extra;
+      if (t >= t_lim) res[i] = 0.f;
     }
     float *dst = am_grad + ((long)b * T + t) * C + c;
     if (c + 4 <= C) {
@@ -1128,8 +1191,8 @@ __device__ __forceinline__ void simple_bwd_am_panel_body(
 template <int kS, int kK>
 void launch_fwd_panel(const float *lm, const float *am, const int64_t *symbols,
                       const int64_t *boundary, float *lm_max, float *am_max, float *px,
-                      float *py, float *norm_raw, int B, int S, int T, int C, int term,
-                      int rnnt_type, hipStream_t stream) {
+                      float *py, float *norm_raw, const int64_t *window, int B, int S, int T,
+                      int C, int term, int rnnt_type, hipStream_t stream) {
   using Shape = PanelShape<kS, kK>;
   const int t_tiles = T > 0 ? (T + kPanT - 1) / kPanT : 1;
   const int s_tiles = (S + 1 + kS - 1) / kS;
@@ -1137,26 +1200,27 @@ void launch_fwd_panel(const float *lm, const float *am, const int64_t *symbols,
   (void)allow_lds(reinterpret_cast<const void *>(kernel), Shape::kLdsBytes);
   hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(t_tiles * s_tiles, B)), dim3(kPanThreads),
                      Shape::kLdsBytes, stream, lm, am, symbols, boundary, lm_max, am_max, px, py,
-                     norm_raw, B, S, T, C, term, rnnt_type);
+                     norm_raw, window, B, S, T, C, term, rnnt_type);
 }
 void launch_fwd_gemm(const float *lm, const float *am, const int64_t *symbols,
                      const int64_t *boundary, float *lm_max, float *am_max, float *px,
-                     float *py, float *norm_raw, int B, int S, int T, int C, int term,
-                     int rnnt_type, hipStream_t stream) {
+                     float *py, float *norm_raw, const int64_t *window, int B, int S, int T,
+                     int C, int term, int rnnt_type, hipStream_t stream) {
   // the row count per workgroup that leaves fewer padding rows; 128 on a tie
   const int S1 = S + 1;
   const int padded96 = (S1 + 95) / 96 * 96, padded128 = (S1 + 127) / 128 * 128;
   if (padded96 < padded128)
-    launch_fwd_panel<96, 16>(lm, am, symbols, boundary, lm_max, am_max, px, py, norm_raw, B, S, T,
-                             C, term, rnnt_type, stream);
+    launch_fwd_panel<96, 16>(lm, am, symbols, boundary, lm_max, am_max, px, py, norm_raw, window,
+                             B, S, T, C, term, rnnt_type, stream);
   else
-    launch_fwd_panel<128, 16>(lm, am, symbols, boundary, lm_max, am_max, px, py, norm_raw, B, S,
-                              T, C, term, rnnt_type, stream);
+    launch_fwd_panel<128, 16>(lm, am, symbols, boundary, lm_max, am_max, px, py, norm_raw, window,
+                              B, S, T, C, term, rnnt_type, stream);
 }
 void launch_fwd_gemm(const double *lm, const double *am, const int64_t *symbols,
                      const int64_t *boundary, const double *lm_max, const double *am_max,
-                     double *px, double *py, double *norm_raw, int B, int S, int T, int C,
-                     int term, int rnnt_type, hipStream_t stream) {
+                     double *px, double *py, double *norm_raw, const int64_t *, int B, int S,
+                     int T, int C, int term, int rnnt_type, hipStream_t stream) {
+  // (the double kernels compute the whole lattice whether or not a window is given)
   const int t_tiles = T > 0 ? (T + kTileN - 1) / kTileN : 1;
   const dim3 grid(t_tiles, (S + 1 + kTileM - 1) / kTileM, B);
   hipLaunchKernelGGL(simple_fwd_kernel<double>, grid, dim3(kGemmThreads), 0, stream, lm, am,
@@ -1170,10 +1234,10 @@ __global__ void __launch_bounds__(kLmThreads, 2)
                               const float *__restrict__ lm_max,
                               const float *__restrict__ am_max, const float *__restrict__ dmat,
                               const float *__restrict__ row_x, const float *__restrict__ row_y,
-                              float *__restrict__ lm_grad, int B, int S, int T, int C, int ldd,
-                              int term) {
+                              float *__restrict__ lm_grad, const int64_t *__restrict__ window,
+                              int B, int S, int T, int C, int ldd, int term) {
   simple_bwd_lm_slab_body<kS, kK>((int)blockIdx.x, lm, am, symbols, lm_max, am_max, dmat, row_x,
-                                  row_y, lm_grad, B, S, T, C, ldd, term);
+                                  row_y, lm_grad, window, B, S, T, C, ldd, term);
 }
 __global__ void __launch_bounds__(256, 2)
     simple_bwd_am_panel_kernel(const float *__restrict__ lm, const float *__restrict__ am,
@@ -1182,10 +1246,11 @@ __global__ void __launch_bounds__(256, 2)
                                const float *__restrict__ lm_max,
                                const float *__restrict__ am_max, const float *__restrict__ dmat,
                                const float *__restrict__ gpx, const float *__restrict__ col_y,
-                               float *__restrict__ am_grad, int B, int S, int T, int C, int ldd,
-                               int term, int rnnt_type, int rows_cap) {
+                               float *__restrict__ am_grad, const int64_t *__restrict__ window,
+                               int B, int S, int T, int C, int ldd, int term, int rnnt_type,
+                               int rows_cap) {
   simple_bwd_am_panel_body((int)blockIdx.x, lm, am, symbols, boundary, lm_max, am_max, dmat, gpx,
-                           col_y, am_grad, B, S, T, C, ldd, term, rnnt_type, rows_cap);
+                           col_y, am_grad, window, B, S, T, C, ldd, term, rnnt_type, rows_cap);
 }
 // Both gradient products in one launch: the first lm_blocks workgroups take tiles of
 // lm.grad, the rest tiles of am.grad.  The two only read what the prep kernel left, so
@@ -1204,21 +1269,24 @@ __global__ void __launch_bounds__(256, 2)
                             const float *__restrict__ dmat, const float *__restrict__ gpx,
                             const float *__restrict__ row_x, const float *__restrict__ row_y,
                             const float *__restrict__ col_y, float *__restrict__ lm_grad,
-                            float *__restrict__ am_grad, int B, int S, int T, int C, int ldd,
-                            int term, int rnnt_type, int rows_cap, int lm_blocks) {
+                            float *__restrict__ am_grad, const int64_t *__restrict__ window, int B,
+                            int S, int T, int C, int ldd, int term, int rnnt_type, int rows_cap,
+                            int lm_blocks) {
   if ((int)blockIdx.x < lm_blocks)
     simple_bwd_lm_slab_body<kS, kK>((int)blockIdx.x, lm, am, symbols, lm_max, am_max, dmat, row_x,
-                                    row_y, lm_grad, B, S, T, C, ldd, term);
+                                    row_y, lm_grad, window, B, S, T, C, ldd, term);
   else
     simple_bwd_am_panel_body((int)blockIdx.x - lm_blocks, lm, am, symbols, boundary, lm_max, am_max,
-                             dmat, gpx, col_y, am_grad, B, S, T, C, ldd, term, rnnt_type, rows_cap);
+                             dmat, gpx, col_y, am_grad, window, B, S, T, C, ldd, term, rnnt_type,
+                             rows_cap);
 }
 // lm.grad and am.grad together (float only)
 void launch_bwd_both(const float *lm, const float *am, const int64_t *symbols,
                      const int64_t *boundary, const float *lm_max, const float *am_max,
                      const float *dmat, const float *gpx, const float *row_x, const float *row_y,
-                     const float *col_y, float *lm_grad, float *am_grad, int B, int S, int T, int C,
-                     int ldd, int term, int rnnt_type, hipStream_t stream) {
+                     const float *col_y, float *lm_grad, float *am_grad, const int64_t *window,
+                     int B, int S, int T, int C, int ldd, int term, int rnnt_type,
+                     hipStream_t stream) {
   const int S1 = S + 1;
   const bool rows96 = (S1 + 95) / 96 * 96 < (S1 + 127) / 128 * 128;
   const int rows = rows96 ? 96 : 128;
@@ -1233,17 +1301,17 @@ void launch_bwd_both(const float *lm, const float *am, const int64_t *symbols,
   auto kernel = rows96 ? simple_bwd_am_lm_kernel<96, 16> : simple_bwd_am_lm_kernel<128, 16>;
   (void)allow_lds(reinterpret_cast<const void *>(kernel), lds);
   hipLaunchKernelGGL(kernel, dim3(am_blocks + lm_blocks), dim3(256), lds, stream, lm, am, symbols,
-                     boundary, lm_max, am_max, dmat, gpx, row_x, row_y, col_y, lm_grad, am_grad, B,
-                     S, T, C, ldd, term, rnnt_type, rows_cap, (int)lm_blocks);
+                     boundary, lm_max, am_max, dmat, gpx, row_x, row_y, col_y, lm_grad, am_grad,
+                     window, B, S, T, C, ldd, term, rnnt_type, rows_cap, (int)lm_blocks);
 }
 void launch_bwd_both(const double *, const double *, const int64_t *, const int64_t *,
                      const double *, const double *, const double *, const double *,
-                     const double *, const double *, const double *, double *, double *, int, int,
-                     int, int, int, int, int, hipStream_t) {}
+                     const double *, const double *, const double *, double *, double *,
+                     const int64_t *, int, int, int, int, int, int, int, hipStream_t) {}
 void launch_bwd_lm(const float *lm, const float *am, const int64_t *symbols, const float *lm_max,
                    const float *am_max, const float *dmat, const float *row_x, const float *row_y,
-                   float *lm_grad, int B, int S, int T, int C, int ldd, int term,
-                   hipStream_t stream) {
+                   float *lm_grad, const int64_t *window, int B, int S, int T, int C, int ldd,
+                   int term, hipStream_t stream) {
   // the row count per workgroup that leaves fewer padding rows; 128 on a tie
   const int S1 = S + 1;
   const bool rows96 = (S1 + 95) / 96 * 96 < (S1 + 127) / 128 * 128;
@@ -1253,21 +1321,22 @@ void launch_bwd_lm(const float *lm, const float *am, const int64_t *symbols, con
   const size_t lds = rows96 ? LmShape<96, 32>::kLdsBytes : LmShape<128, 16>::kLdsBytes;
   (void)allow_lds(reinterpret_cast<const void *>(kernel), lds);
   hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(tiles, B)), dim3(kLmThreads), lds, stream, lm,
-                     am, symbols, lm_max, am_max, dmat, row_x, row_y, lm_grad, B, S, T, C, ldd,
-                     term);
+                     am, symbols, lm_max, am_max, dmat, row_x, row_y, lm_grad, window, B, S, T, C,
+                     ldd, term);
 }
 void launch_bwd_lm(const double *lm, const double *am, const int64_t *symbols,
                    const double *lm_max, const double *am_max, const double *dmat,
-                   const double *row_x, const double *row_y, double *lm_grad, int B, int S, int T,
-                   int C, int ldd, int term, hipStream_t stream) {
+                   const double *row_x, const double *row_y, double *lm_grad, const int64_t *, int B,
+                   int S, int T, int C, int ldd, int term, hipStream_t stream) {
   const dim3 grid((C + kTileN - 1) / kTileN, (S + 1 + kTileM - 1) / kTileM, B);
   hipLaunchKernelGGL(simple_bwd_lm_kernel<double>, grid, dim3(kGemmThreads), 0, stream, lm, am,
                      symbols, lm_max, am_max, dmat, row_x, row_y, lm_grad, S, T, C, ldd, term);
 }
 void launch_bwd_am(const float *lm, const float *am, const int64_t *symbols,
                    const int64_t *boundary, const float *lm_max, const float *am_max,
-                   const float *dmat, const float *gpx, const float *col_y, float *am_grad, int B,
-                   int S, int T, int C, int ldd, int term, int rnnt_type, hipStream_t stream) {
+                   const float *dmat, const float *gpx, const float *col_y, float *am_grad,
+                   const int64_t *window, int B, int S, int T, int C, int ldd, int term,
+                   int rnnt_type, hipStream_t stream) {
   const int tiles = ((C + kAmC - 1) / kAmC) * ((T + kAmT - 1) / kAmT);
   // rows of k held in LDS per pass: all of them when they fit
   const int rows_cap = std::min(kAmRows, (S + 2) & ~1);
@@ -1276,13 +1345,13 @@ void launch_bwd_am(const float *lm, const float *am, const int64_t *symbols,
   auto kernel = simple_bwd_am_panel_kernel;
   (void)allow_lds(reinterpret_cast<const void *>(kernel), lds);
   hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(tiles, B)), dim3(256), lds, stream, lm, am,
-                     symbols, boundary, lm_max, am_max, dmat, gpx, col_y, am_grad, B, S, T, C, ldd,
-                     term, rnnt_type, rows_cap);
+                     symbols, boundary, lm_max, am_max, dmat, gpx, col_y, am_grad, window, B, S, T, C,
+                     ldd, term, rnnt_type, rows_cap);
 }
 void launch_bwd_am(const double *lm, const double *am, const int64_t *symbols,
                    const int64_t *boundary, const double *lm_max, const double *am_max,
                    const double *dmat, const double *gpx, const double *col_y, double *am_grad,
-                   int B, int S, int T, int C, int ldd, int term, int rnnt_type,
+                   const int64_t *, int B, int S, int T, int C, int ldd, int term, int rnnt_type,
                    hipStream_t stream) {
   const dim3 grid((C + kTileN - 1) / kTileN, (T + kTileM - 1) / kTileM, B);
   hipLaunchKernelGGL(simple_bwd_am_kernel<double>, grid, dim3(kGemmThreads), 0, stream, lm, am,
@@ -1298,7 +1367,7 @@ void launch_bwd_am(const double *lm, const double *am, const int64_t *symbols,
 template <typename R>
 int fwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *boundary, R *px,
              R *py, R *lm_max, R *am_max, R *norm_raw, int B, int S, int T, int C, int term,
-             int rnnt_type, void *stream_) {
+             int rnnt_type, int window_only, void *stream_) {
   if (B < 0 || S < 0 || T < 0 || C < 1) return fail(FRNNT_EINVAL, "simple_logprobs_fwd: bad size");
   if (rnnt_type < 0 || rnnt_type > 2)
     return fail(FRNNT_EINVAL, "simple_logprobs_fwd: rnnt_type must be 0, 1 or 2");
@@ -1321,8 +1390,8 @@ int fwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
   {
     // (the grid always has at least one column of tiles, so that the -inf column of
     // an empty-frame regular lattice is still written)
-    launch_fwd_gemm(lm, am, symbols, boundary, lm_max, am_max, px, py, norm_raw, B, S, T, C, term,
-                    rnnt_type, stream);
+    launch_fwd_gemm(lm, am, symbols, boundary, lm_max, am_max, px, py, norm_raw,
+                    window_only ? boundary : nullptr, B, S, T, C, term, rnnt_type, stream);
     if (rnnt_type == kConstrained && S > 0 && T > 0) {
       const long total = (long)B * S * T;
       hipLaunchKernelGGL(add_next_row_kernel<R>, dim3((unsigned)((total + 255) / 256)), dim3(256),
@@ -1335,8 +1404,9 @@ int fwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
 template <typename R>
 int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *boundary,
              const R *lm_max, const R *am_max, const R *norm_raw, const R *score_grad,
-             int score_grad_stride, double score_grad_scale, R *px_grad, R *py_grad, R *dmat, R *row_x, R *row_y, R *col_y, R *lm_grad, R *am_grad, int B,
-             int S, int T, int C, int term, int rnnt_type, void *stream_) {
+             int score_grad_stride, double score_grad_scale, R *px_grad, R *py_grad, R *dmat,
+             R *row_x, R *row_y, R *col_y, R *lm_grad, R *am_grad, int B, int S, int T, int C,
+             int term, int rnnt_type, int window_only, void *stream_) {
   if (B < 0 || S < 0 || T < 0 || C < 1) return fail(FRNNT_EINVAL, "simple_logprobs_bwd: bad size");
   if (rnnt_type < 0 || rnnt_type > 2 || term < 0 || term >= C)
     return fail(FRNNT_EINVAL, "simple_logprobs_bwd: bad rnnt_type or termination symbol");
@@ -1362,24 +1432,26 @@ int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
                          (R)score_grad_scale, per_x, per_y, x_blocks);
   }
   const int ldd = (T + 3) & ~3;  // leading dimension of dmat: 16-byte rows
+  // (the double kernels ignore the window: they take the whole lattice as it is)
+  const int64_t *window = (window_only && std::is_same<R, float>::value) ? boundary : nullptr;
   const long prep_blocks = ((long)B * (S + 1) + 3) / 4 + (long)B * ((T + kWave - 1) / kWave);
   hipLaunchKernelGGL(simple_bwd_prep_kernel<R>, dim3((unsigned)prep_blocks), dim3(256), 0, stream,
-                     px_grad, py_grad, norm_raw, boundary, dmat, row_x, row_y, col_y, B, S, T, ldd,
-                     rnnt_type);
+                     px_grad, py_grad, norm_raw, boundary, window, dmat, row_x, row_y, col_y, B, S, T,
+                     ldd, rnnt_type);
   // (one launch for both products while they are short: at B (S+1) T C = 3.2e8 it saves
   // about 1 us of 37; at 3.9e9 the common LDS and register budget costs 8 %)
   if (std::is_same<R, float>::value && lm_grad && am_grad && T > 0 &&
       (double)B * (S + 1) * T * C < 1e9) {
     launch_bwd_both(lm, am, symbols, boundary, lm_max, am_max, dmat, px_grad, row_x, row_y, col_y,
-                    lm_grad, am_grad, B, S, T, C, ldd, term, rnnt_type, stream);
+                    lm_grad, am_grad, window, B, S, T, C, ldd, term, rnnt_type, stream);
     return check_launch("simple_logprobs_bwd");
   }
   if (lm_grad)
-    launch_bwd_lm(lm, am, symbols, lm_max, am_max, dmat, row_x, row_y, lm_grad, B, S, T, C, ldd,
-                  term, stream);
+    launch_bwd_lm(lm, am, symbols, lm_max, am_max, dmat, row_x, row_y, lm_grad, window, B, S, T, C,
+                  ldd, term, stream);
   if (am_grad && T > 0)
-    launch_bwd_am(lm, am, symbols, boundary, lm_max, am_max, dmat, px_grad, col_y, am_grad, B, S,
-                  T, C, ldd, term, rnnt_type, stream);
+    launch_bwd_am(lm, am, symbols, boundary, lm_max, am_max, dmat, px_grad, col_y, am_grad, window,
+                  B, S, T, C, ldd, term, rnnt_type, stream);
   return check_launch("simple_logprobs_bwd");
 }
 
@@ -1431,7 +1503,7 @@ int frnnt_simple_logprobs_bwd_noalloc_f32(const float *lm, const float *am, cons
                                           double score_grad_scale, float *px_grad,
                                           float *py_grad, float *lm_grad, float *am_grad, int B,
                                           int S, int T, int C, int termination_symbol,
-                                          int rnnt_type, void *stream) {
+                                          int rnnt_type, int window_only, void *stream) {
   using frnnt::fail;
   if (B < 0 || S < 0 || T < 0) return fail(FRNNT_EINVAL, "simple_logprobs_bwd_noalloc: bad size");
   // dmat | row_x | row_y | col_y, each starting 16-byte aligned
@@ -1452,22 +1524,24 @@ int frnnt_simple_logprobs_bwd_noalloc_f32(const float *lm, const float *am, cons
   return frnnt::bwd_impl<float>(lm, am, symbols, boundary, lm_max, am_max, norm_raw, score_grad,
                                 score_grad_stride, score_grad_scale, px_grad, py_grad, dmat, row_x,
                                 row_y, col_y, lm_grad, am_grad, B, S, T, C, termination_symbol,
-                                rnnt_type, stream);
+                                rnnt_type, window_only, stream);
 }
 
 int frnnt_simple_logprobs_fwd_f32(const float *lm, const float *am, const int64_t *symbols,
                                   const int64_t *boundary, float *px, float *py, float *lm_max,
                                   float *am_max, float *norm_raw, int B, int S, int T, int C,
-                                  int termination_symbol, int rnnt_type, void *stream) {
+                                  int termination_symbol, int rnnt_type, int window_only,
+                                  void *stream) {
   return frnnt::fwd_impl<float>(lm, am, symbols, boundary, px, py, lm_max, am_max, norm_raw, B, S,
-                                T, C, termination_symbol, rnnt_type, stream);
+                                T, C, termination_symbol, rnnt_type, window_only, stream);
 }
 int frnnt_simple_logprobs_fwd_f64(const double *lm, const double *am, const int64_t *symbols,
                                   const int64_t *boundary, double *px, double *py, double *lm_max,
                                   double *am_max, double *norm_raw, int B, int S, int T, int C,
-                                  int termination_symbol, int rnnt_type, void *stream) {
+                                  int termination_symbol, int rnnt_type, int window_only,
+                                  void *stream) {
   return frnnt::fwd_impl<double>(lm, am, symbols, boundary, px, py, lm_max, am_max, norm_raw, B, S,
-                                 T, C, termination_symbol, rnnt_type, stream);
+                                 T, C, termination_symbol, rnnt_type, window_only, stream);
 }
 int frnnt_simple_logprobs_bwd_f32(const float *lm, const float *am, const int64_t *symbols,
                                   const int64_t *boundary, const float *lm_max,
@@ -1476,10 +1550,12 @@ int frnnt_simple_logprobs_bwd_f32(const float *lm, const float *am, const int64_
                                   double score_grad_scale, float *px_grad, float *py_grad,
                                   float *dmat, float *row_x, float *row_y, float *col_y,
                                   float *lm_grad, float *am_grad, int B, int S, int T, int C,
-                                  int termination_symbol, int rnnt_type, void *stream) {
+                                  int termination_symbol, int rnnt_type, int window_only,
+                                  void *stream) {
   return frnnt::bwd_impl<float>(lm, am, symbols, boundary, lm_max, am_max, norm_raw, score_grad,
-                                score_grad_stride, score_grad_scale, px_grad, py_grad, dmat, row_x, row_y, col_y, lm_grad, am_grad, B,
-                                S, T, C, termination_symbol, rnnt_type, stream);
+                                score_grad_stride, score_grad_scale, px_grad, py_grad, dmat, row_x,
+                                row_y, col_y, lm_grad, am_grad, B, S, T, C, termination_symbol,
+                                rnnt_type, window_only, stream);
 }
 int frnnt_simple_logprobs_bwd_f64(const double *lm, const double *am, const int64_t *symbols,
                                   const int64_t *boundary, const double *lm_max,
@@ -1488,10 +1564,12 @@ int frnnt_simple_logprobs_bwd_f64(const double *lm, const double *am, const int6
                                   double score_grad_scale, double *px_grad, double *py_grad,
                                   double *dmat, double *row_x, double *row_y, double *col_y,
                                   double *lm_grad, double *am_grad, int B, int S, int T, int C,
-                                  int termination_symbol, int rnnt_type, void *stream) {
+                                  int termination_symbol, int rnnt_type, int window_only,
+                                  void *stream) {
   return frnnt::bwd_impl<double>(lm, am, symbols, boundary, lm_max, am_max, norm_raw, score_grad,
-                                 score_grad_stride, score_grad_scale, px_grad, py_grad, dmat, row_x, row_y, col_y, lm_grad, am_grad, B,
-                                 S, T, C, termination_symbol, rnnt_type, stream);
+                                 score_grad_stride, score_grad_scale, px_grad, py_grad, dmat,
+                                 row_x, row_y, col_y, lm_grad, am_grad, B, S, T, C,
+                                 termination_symbol, rnnt_type, window_only, stream);
 }
 
 int frnnt_loss_reduce_f32(const float *scores, float *loss, int B, int reduction, void *stream) {

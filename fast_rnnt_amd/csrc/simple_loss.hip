@@ -16,8 +16,10 @@ int simple_loss_fwd(Logprobs logprobs, Forward forward, Backward backward, Reduc
                     int reduction, void *stream) {
   if ((px_grad == nullptr) != (py_grad == nullptr))
     return fail(FRNNT_EINVAL, "simple_loss_fwd: px_grad and py_grad go together");
+  // px / py only feed the recursion below, with the same boundary: what lies outside an
+  // utterance's window need not be computed
   int rc = logprobs(lm, am, symbols, boundary, px, py, lm_max, am_max, norm_raw, B, S, T, C, term,
-                    rnnt_type, stream);
+                    rnnt_type, boundary != nullptr, stream);
   if (rc != FRNNT_OK) return rc;
   const int modified = rnnt_type != 0;
   rc = forward(px, py, boundary, p, scores, B, S, T, modified, stream);

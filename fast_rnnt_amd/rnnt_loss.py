@@ -108,7 +108,7 @@ class _SimpleLogprobs(torch.autograd.Function):
             _lib.call("frnnt_simple_logprobs_fwd_" + sfx, lm_c.data_ptr(), am_c.data_ptr(),
                       sym_c.data_ptr(), _lib.ptr(bnd_c), px.data_ptr(), py.data_ptr(),
                       lm_max.data_ptr(), am_max.data_ptr(), _lib.ptr(norm_raw), B, S, T, C,
-                      int(termination_symbol), kind, _lib.stream_of(am))
+                      int(termination_symbol), kind, 0, _lib.stream_of(am))
         if need_grad:
             ctx.save_for_backward(lm_c, am_c, sym_c, bnd_c, lm_max, am_max, norm_raw)
             ctx.meta = (B, S, T, C, int(termination_symbol), kind, sfx)
@@ -134,7 +134,7 @@ class _SimpleLogprobs(torch.autograd.Function):
                       norm_raw.data_ptr(), None, 0, 1.0, gpx.data_ptr(), gpy.data_ptr(),
                       dmat.data_ptr(),
                       row_x.data_ptr(), row_y.data_ptr(), col_y.data_ptr(), _lib.ptr(lm_grad),
-                      _lib.ptr(am_grad), B, S, T, C, term, kind, _lib.stream_of(am))
+                      _lib.ptr(am_grad), B, S, T, C, term, kind, 0, _lib.stream_of(am))
         return lm_grad, am_grad, None, None, None, None
 
 
@@ -261,7 +261,7 @@ class _SimpleLoss(torch.autograd.Function):
                 _lib.call("frnnt_simple_logprobs_fwd_" + sfx, lm_c.data_ptr(), am_c.data_ptr(),
                           sym_c.data_ptr(), _lib.ptr(bnd_c), at(o_px), at(o_py), at(o_lmx),
                           at(o_amx), at(o_nr) if need_grad else None, B, S, T, C,
-                          int(termination_symbol), kind, stream)
+                          int(termination_symbol), kind, int(bnd_c is not None), stream)
                 _apply_delay_penalty(px, boundary, rnnt_type, delay_penalty)
                 modified = int(kind != 0)
                 _lib.call("frnnt_mi_forward_" + sfx, at(o_px), at(o_py), _lib.ptr(bnd_c), at(o_p),
@@ -314,7 +314,8 @@ class _SimpleLoss(torch.autograd.Function):
                       wbase + o_nr * item, g.data_ptr(), stride, scale, px_grad.data_ptr(),
                       py_grad.data_ptr(), sbase + o_d * item, sbase + o_rx * item,
                       sbase + o_ry * item, sbase + o_cy * item, _lib.ptr(lm_grad),
-                      _lib.ptr(am_grad), B, S, T, C, term, kind, _lib.stream_of(am))
+                      _lib.ptr(am_grad), B, S, T, C, term, kind, int(bnd is not None),
+                      _lib.stream_of(am))
         return lm_grad, am_grad, None, None, None, None, None, None, None
 
 

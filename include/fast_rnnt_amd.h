@@ -108,15 +108,22 @@ int frnnt_mi_backward_f64(const double *px, const double *py, const int64_t *bou
  *   norm_raw [B][S+1][T] or NULL  out: log(sum_c exp(lm-lm_max) exp(am-am_max) + tiny),
  *                                 needed by the backward entry point
  *   rnnt_type: 0 regular, 1 modified, 2 constrained
+ *   window_only: 0 = every cell is computed.  1 (with a boundary; float32 kernels) = the
+ *   caller goes on to the lattice recursion with the same boundary, which only looks at
+ *   rows <= s_end and frames <= t_end of utterance b: what lies past them in px, py,
+ *   norm_raw and am_max is left undefined (tiles past t_end are not computed at all).
+ *   The backward entry point then needs the same flag.
  */
 int frnnt_simple_logprobs_fwd_f32(const float *lm, const float *am, const int64_t *symbols,
                                   const int64_t *boundary, float *px, float *py, float *lm_max,
                                   float *am_max, float *norm_raw, int B, int S, int T, int C,
-                                  int termination_symbol, int rnnt_type, void *stream);
+                                  int termination_symbol, int rnnt_type, int window_only,
+                                  void *stream);
 int frnnt_simple_logprobs_fwd_f64(const double *lm, const double *am, const int64_t *symbols,
                                   const int64_t *boundary, double *px, double *py, double *lm_max,
                                   double *am_max, double *norm_raw, int B, int S, int T, int C,
-                                  int termination_symbol, int rnnt_type, void *stream);
+                                  int termination_symbol, int rnnt_type, int window_only,
+                                  void *stream);
 
 /*
  * Backward of the above: what autograd derives for rnnt_loss.py:174-225, as one
@@ -132,6 +139,10 @@ int frnnt_simple_logprobs_fwd_f64(const double *lm, const double *am, const int6
  *   dmat [B][S+1][T rounded up to a multiple of 4], row_x [B][S+1], row_y [B][S+1],
  *   col_y [B][T]                                                           scratch
  *   lm_grad [B][S+1][C], am_grad [B][T][C]: out; either may be NULL to skip it
+ *   window_only: 1 (with a boundary) = px_grad / py_grad vanish outside each utterance's
+ *   boundary window, as the recursion's backward leaves them: nothing outside is read,
+ *   the sums stop at s_end / t_end, and am_grad rows of frames >= t_end are stored as
+ *   exact zeros without being computed.  Required when the forward ran with window_only.
  */
 int frnnt_simple_logprobs_bwd_f32(const float *lm, const float *am, const int64_t *symbols,
                                   const int64_t *boundary, const float *lm_max,
@@ -140,7 +151,8 @@ int frnnt_simple_logprobs_bwd_f32(const float *lm, const float *am, const int64_
                                   double score_grad_scale, float *px_grad, float *py_grad,
                                   float *dmat, float *row_x, float *row_y, float *col_y,
                                   float *lm_grad, float *am_grad, int B, int S, int T, int C,
-                                  int termination_symbol, int rnnt_type, void *stream);
+                                  int termination_symbol, int rnnt_type, int window_only,
+                                  void *stream);
 int frnnt_simple_logprobs_bwd_f64(const double *lm, const double *am, const int64_t *symbols,
                                   const int64_t *boundary, const double *lm_max,
                                   const double *am_max, const double *norm_raw,
@@ -148,7 +160,8 @@ int frnnt_simple_logprobs_bwd_f64(const double *lm, const double *am, const int6
                                   double score_grad_scale, double *px_grad, double *py_grad,
                                   double *dmat, double *row_x, double *row_y, double *col_y,
                                   double *lm_grad, double *am_grad, int B, int S, int T, int C,
-                                  int termination_symbol, int rnnt_type, void *stream);
+                                  int termination_symbol, int rnnt_type, int window_only,
+                                  void *stream);
 /*
  * frnnt_simple_logprobs_bwd_f32 for callers that cannot allocate device memory (code under
  * HIP graph capture, serving loops, harnesses that forbid hipMalloc).  It has no
@@ -168,7 +181,7 @@ int frnnt_simple_logprobs_bwd_noalloc_f32(const float *lm, const float *am, cons
                                           double score_grad_scale, float *px_grad,
                                           float *py_grad, float *lm_grad, float *am_grad, int B,
                                           int S, int T, int C, int termination_symbol,
-                                          int rnnt_type, void *stream);
+                                          int rnnt_type, int window_only, void *stream);
 /*
  * The lm-only / am-only smoothing of get_rnnt_logprobs_smoothed (rnnt_loss.py:1135-1369)
  * applied to joint px / py (px_joint, py_joint: outputs of frnnt_simple_logprobs_fwd

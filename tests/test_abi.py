@@ -42,7 +42,7 @@ def test_size_limits_are_reported_without_a_gpu():
     dummy = ctypes.c_void_p(0x1000)
     B, S, T, C = 1, 10, 70000, 8000          # T * C * 4 bytes >= 2 GiB
     rc = lib.frnnt_simple_logprobs_fwd_f32(dummy, dummy, dummy, None, dummy, dummy, dummy, dummy,
-                                           None, B, S, T, C, 0, 0, None)
+                                           None, B, S, T, C, 0, 0, 0, None)
     assert rc == -3 and b"2 GiB" in lib.frnnt_last_error()
     B, S, T = 1, 20000, 20000                # (S+1) * (T+1) * 4 bytes >= 1 GiB
     rc = lib.frnnt_mi_forward_f32(dummy, dummy, None, dummy, dummy, B, S, T, 0, None)

@@ -170,6 +170,42 @@ def test_loss_and_all_gradients(gpu_device, dtype, kind):
             assert _close(gx, wx, gtol) and _close(gy, wy, gtol)
 
 
+@pytest.mark.parametrize("kind", KINDS)
+def test_fused_loss_ignores_frames_past_the_window(gpu_device, kind):
+    # rnnt_loss_simple works on each utterance's window only: NaN planted (on the GPU side)
+    # in the am frames at and past t_end must change nothing -- loss and gradients as the
+    # oracle computes them on clean input, and am.grad exactly zero at those frames.  Shapes
+    # with several frame tiles, row tiles and more than 96 lattice rows.
+    dev = gpu_device
+    for n, (B, S, T, C) in enumerate([(4, 20, 75, 50), (3, 66, 140, 70), (2, 101, 200, 44),
+                                      (3, 80, 250, 500)]):
+        am, lm, sym, bnd = _case(160 + n, B, S, T, C, torch.float32, kind)
+        bnd[0, 3] = T                       # one utterance keeps every frame
+        t_idx = torch.arange(T).reshape(1, T, 1)
+        past = (t_idx >= bnd[:, 3].reshape(B, 1, 1)).expand(B, T, C)
+        _say(f"window-only simple loss {kind} shape{n}: T_b = {bnd[:, 3].tolist()} of {T}, "
+             f"S_b = {bnd[:, 2].tolist()} of {S}")
+        a = am.clone().requires_grad_(True)
+        l = lm.clone().requires_grad_(True)
+        want, (wx, wy) = O.loss_simple(l, a, sym, 0, boundary=bnd, rnnt_type=kind,
+                                       reduction="none", return_grad=True)
+        wx0, wy0 = wx.clone(), wy.clone()
+        want.sum().backward()
+        poisoned = torch.where(past, torch.full_like(am, float("nan")), am)
+        da = poisoned.to(dev).requires_grad_(True)
+        dl = lm.to(dev).requires_grad_(True)
+        got, (gx, gy) = fast_rnnt_amd.rnnt_loss_simple(dl, da, sym.to(dev), 0, boundary=bnd.to(dev),
+                                                       rnnt_type=kind, reduction="none",
+                                                       return_grad=True)
+        gx0, gy0 = gx.clone(), gy.clone()
+        got.sum().backward()
+        assert _close(got, want, 0.0, 1e-5)
+        assert _close(gx0, wx0, 1e-4) and _close(gy0, wy0, 1e-4)
+        assert bool((da.grad.cpu()[past] == 0).all())
+        assert _close(da.grad.cpu()[~past], a.grad[~past], 1e-4, 1e-4)
+        assert _close(dl.grad, l.grad, 1e-4, 1e-4)
+
+
 def test_delay_penalty_and_only_one_input_needs_grad(gpu_device):
     dev = gpu_device
     am, lm, sym, bnd = _case(77, 3, 9, 30, 21, torch.float32, "regular")
@@ -274,7 +310,7 @@ def test_gradient_products_together_and_apart(gpu_device, shape):
     _say(f"gradient products B={B} S={S} T={T} C={C}")
     _lib.call("frnnt_simple_logprobs_fwd_f32", lm.data_ptr(), am.data_ptr(), sym.data_ptr(),
               bnd.data_ptr(), px.data_ptr(), py.data_ptr(), lm_max.data_ptr(), am_max.data_ptr(),
-              norm_raw.data_ptr(), B, S, T, C, 0, 0, stream)
+              norm_raw.data_ptr(), B, S, T, C, 0, 0, 0, stream)
     gpx = torch.rand(B, S, T + 1, generator=g).to(dev)
     gpy = torch.rand(B, S + 1, T, generator=g).to(dev)
     dmat = torch.empty(B, S + 1, (T + 3) // 4 * 4, **f32)
@@ -288,7 +324,7 @@ def test_gradient_products_together_and_apart(gpu_device, shape):
                   bnd.data_ptr(), lm_max.data_ptr(), am_max.data_ptr(), norm_raw.data_ptr(), None,
                   0, 1.0, gpx.data_ptr(), gpy.data_ptr(), dmat.data_ptr(), row_x.data_ptr(),
                   row_y.data_ptr(), col_y.data_ptr(), _lib.ptr(lm_grad), _lib.ptr(am_grad), B, S,
-                  T, C, 0, 0, stream)
+                  T, C, 0, 0, 0, stream)
         torch.cuda.synchronize()
         return lm_grad, am_grad
 

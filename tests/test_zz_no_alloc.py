@@ -38,7 +38,7 @@ def _both_ways(dev, seed, B, S, T, C, rnnt_type, with_boundary, with_score_grad)
     stream = torch.cuda.current_stream().cuda_stream
     _lib.call("frnnt_simple_logprobs_fwd_f32", lm.data_ptr(), am.data_ptr(), sym.data_ptr(),
               _lib.ptr(bnd), px.data_ptr(), py.data_ptr(), lm_max.data_ptr(), am_max.data_ptr(),
-              norm_raw.data_ptr(), B, S, T, C, 0, rnnt_type, stream)
+              norm_raw.data_ptr(), B, S, T, C, 0, rnnt_type, 0, stream)
     gpx = torch.rand(B, S, T1, generator=g).to(dev)
     gpy = torch.rand(B, S + 1, T, generator=g).to(dev)
     score_grad = torch.randn(B, generator=g).to(dev) if with_score_grad else None
@@ -49,7 +49,7 @@ def _both_ways(dev, seed, B, S, T, C, rnnt_type, with_boundary, with_score_grad)
         head = [lm.data_ptr(), am.data_ptr(), sym.data_ptr(), _lib.ptr(bnd), lm_max.data_ptr(),
                 am_max.data_ptr(), norm_raw.data_ptr(), _lib.ptr(score_grad), 1, -0.5,
                 gx.data_ptr(), gy.data_ptr()]
-        tail = [lm_grad.data_ptr(), am_grad.data_ptr(), B, S, T, C, 0, rnnt_type, stream]
+        tail = [lm_grad.data_ptr(), am_grad.data_ptr(), B, S, T, C, 0, rnnt_type, 0, stream]
         if own_scratch:
             _lib.call("frnnt_simple_logprobs_bwd_noalloc_f32", *head, *tail)
         else:
@@ -83,4 +83,4 @@ def test_sizes_beyond_the_array_are_refused(gpu_device):
     B, S, T = 64, 255, 512
     with pytest.raises(RuntimeError, match="scratch"):
         _lib.call("frnnt_simple_logprobs_bwd_noalloc_f32", *([None] * 8), 1, 1.0, *([None] * 4),
-                  B, S, T, 16, 0, 0, None)
+                  B, S, T, 16, 0, 0, 0, None)
