@@ -25,6 +25,7 @@ _D = ctypes.c_double
 _SIGNATURES = {
     "frnnt_version": ([], _I),
     "frnnt_last_error": ([], ctypes.c_char_p),
+    "frnnt_set_spin_limit": ([_I], None),
     "frnnt_mi_forward_f32": ([_P, _P, _P, _P, _P, _I, _I, _I, _I, _P], _I),
     "frnnt_mi_forward_f64": ([_P, _P, _P, _P, _P, _I, _I, _I, _I, _P], _I),
     "frnnt_mi_backward_f32": ([_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P], _I),

@@ -57,7 +57,9 @@ constexpr int kBwdStagers = 3;
 // copy, and more of them slow the sweep waves down (21.4 us with 2, 22.2 with 5, 23.0 with
 // 7 per sweep wave).
 constexpr int kBwdStagersFew = 6;
-constexpr int kSpinLimit = 1 << 22;
+constexpr int kSpinLimit = 1 << 22;   // polls before a wait gives up (seconds, not microseconds)
+// Set by frnnt_set_spin_limit(): lets a test force the give-up path from the host.
+int g_spin_limit = kSpinLimit;
 
 struct Window {
   int s0, t0, ns, nt;  // origin and extent (ns = s_end - s_begin, ...)
@@ -80,11 +82,13 @@ __device__ __forceinline__ Window load_window(const int64_t *boundary, int b, in
 
 // Blocks until the counter reaches `target`; gives up (returns false) after a
 // bounded number of polls so that no wave can spin forever.
-__device__ __forceinline__ bool wait_for(const int *counter, int target) {
+// A wave that gives up must not leave quietly: the callers mark the utterance's outputs
+// (see give_up below), so that a wait that never ends shows as NaN, not as a wrong number.
+__device__ __forceinline__ bool wait_for(const int *counter, int target, int limit) {
   int spins = 0;
   while (__hip_atomic_load(counter, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < target) {
     __builtin_amdgcn_s_sleep(1);
-    if (++spins > kSpinLimit) return false;
+    if (++spins > limit) return false;
   }
   return true;
 }
@@ -202,6 +206,7 @@ __device__ __forceinline__ void push_chunk(R *dst, const R (&src)[kChunk]) {
 }
 
 struct Counters {
+  int failed;                             // set by a wave whose bounded wait ran out
   int ready[kMaxSweep];                   // seam columns published by sweep wave w
   int written[kMaxSweep];                 // tiles whose results sweep wave w has left in LDS
   int loaded[16];                         // tiles staged for sweep wave w by its stager l (index w * stagers + l)
@@ -233,7 +238,7 @@ template <typename R, bool kModified, int kSweepCap, int kStagers, int kBuffers>
 __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
     mi_forward_kernel(const R *__restrict__ px, const R *__restrict__ py,
                       const int64_t *__restrict__ boundary, R *__restrict__ p,
-                      R *__restrict__ ans, int S, int T) {
+                      R *__restrict__ ans, int S, int T, int spin_limit) {
   extern __shared__ __align__(16) unsigned char dyn_lds[];
   __shared__ Counters cnt;
 
@@ -263,6 +268,14 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
   const int seam_pitch = (TP + kSeamSlack + 3) & ~3;  // keeps the tiles 16-byte aligned
   R *tiles = seam + (size_t)nsweep * seam_pitch;  // per sweep wave: kBuffers x tiles, then as many y tiles
   const int band_rows = kWave * nsweep;
+  // A wave whose bounded wait ran out: the utterance's score becomes NaN (also for the
+  // wave that would store it later), so the failure cannot pass for a result.
+  auto give_up = [&]() {
+    if (lane == 0) {
+      publish(&cnt.failed, 1);
+      ans[b] = std::numeric_limits<R>::quiet_NaN();
+    }
+  };
 
   if (wave >= nsweep) {
     // ------------------------------ staging wave -------------------------------
@@ -343,7 +356,10 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
         const int gt = tile_base + m;
         if (gt >= kBuffers) {
           // the buffer still holds p of tile gt - kBuffers
-          if (!wait_for(&cnt.written[w], gt - kBuffers + 1)) return;
+          if (!wait_for(&cnt.written[w], gt - kBuffers + 1, spin_limit)) {
+            give_up();
+            return;
+          }
           drain_buffer(buf);
         }
 #pragma unroll
@@ -383,7 +399,10 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
     const int first_left = max(tile_base - kBuffers, 0);
     buf = first_left % kBuffers;
     for (int gt = first_left; gt < tile_base; ++gt) {
-      if (!wait_for(&cnt.written[w], gt + 1)) return;
+      if (!wait_for(&cnt.written[w], gt + 1, spin_limit)) {
+        give_up();
+        return;
+      }
       drain_buffer(buf);
       buf = buf + 1 == kBuffers ? 0 : buf + 1;
     }
@@ -423,8 +442,10 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
 #pragma unroll
       for (int l = 0; l < kStagers; ++l)
         if (__builtin_amdgcn_readfirstlane(seen_loaded[l]) < gt + 1 &&
-            !wait_for(&cnt.loaded[w * kStagers + l], gt + 1))
+            !wait_for(&cnt.loaded[w * kStagers + l], gt + 1, spin_limit)) {
+          give_up();
           return;
+        }
       // this lane's 32 steps of inputs go to registers in one burst
       R xq[kTileSteps], yq[kTileSteps];
       R *x_row = base + buf * kTileElems + lane * kTilePitch;  // x in, p out
@@ -443,7 +464,7 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
           const int need = min(e0 + kChunk - shift, cols);
           handed = seen_seam;
           if (need > 0 && __builtin_amdgcn_readfirstlane(seen_ready) < up_base + need) {
-            if (!wait_for(&cnt.ready[prev], up_base + need)) {
+            if (!wait_for(&cnt.ready[prev], up_base + need, spin_limit)) {
               alive = false;
               return;
             }
@@ -515,10 +536,13 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
         else
           tile(std::false_type{}, std::false_type{});
       }
-      if (!alive) return;
+      if (!alive) {
+        give_up();
+        return;
+      }
       if (lane == 0) publish_lds_writes(&cnt.written[w], gt + 1);
     }
-    if (lane == fin_lane) ans[b] = fin;
+    if (lane == fin_lane) ans[b] = peek(&cnt.failed) ? std::numeric_limits<R>::quiet_NaN() : fin;
     tile_base += g.ntiles;
   }
 }
@@ -541,7 +565,8 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
     mi_backward_kernel(const R *__restrict__ px, const int64_t *__restrict__ boundary,
                        const R *__restrict__ p, R *ans_grad, R *__restrict__ px_grad,
                        R *__restrict__ py_grad, int S, int T, int overwrite_ans_grad,
-                       const R *__restrict__ scores, R *__restrict__ loss, int B, int reduction) {
+                       const R *__restrict__ scores, R *__restrict__ loss, int B, int reduction,
+                       int spin_limit) {
   extern __shared__ __align__(16) unsigned char dyn_lds[];
   __shared__ Counters cnt;
 
@@ -618,6 +643,21 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
   const int seam_pitch = (TP + kSeamSlack + 3) & ~3;  // keeps the tiles 16-byte aligned
   R *tiles = seam + (size_t)nsweep * seam_pitch;  // per sweep wave: kBuffers d1 tiles, then as many d2 tiles
   const int band_rows = kWave * nsweep;
+  // A wave whose bounded wait ran out leaves NaN where the window starts -- in px_grad,
+  // in py_grad and, when it is written back, in ans_grad -- so that the utterance's
+  // gradients cannot pass for a result; every staging wave repeats that when it is done
+  // and finds the mark, so no later store of a good value covers it up.
+  auto poison = [&]() {
+    if (lane != 0) return;
+    const R nan = std::numeric_limits<R>::quiet_NaN();
+    if (NS > 0) put1(gx_rsrc, (win.s0 * T1 + win.t0) * (int)sizeof(R), nan);
+    if (NT > 0) put1(gy_rsrc, (win.s0 * T + win.t0) * (int)sizeof(R), nan);
+    if (overwrite_ans_grad && ans_grad) ans_grad[b] = nan;
+  };
+  auto give_up = [&]() {
+    if (lane == 0) publish(&cnt.failed, 1);
+    poison();
+  };
 
   if (wave >= nsweep) {
     // ------------------------------ staging wave -------------------------------
@@ -712,7 +752,10 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
         const int gt = tile_base + m;
         if (gt >= kBuffers) {
           // the buffer still holds the gradients of tile gt - kBuffers
-          if (!wait_for(&cnt.written[w], gt - kBuffers + 1)) return;
+          if (!wait_for(&cnt.written[w], gt - kBuffers + 1, spin_limit)) {
+            give_up();
+            return;
+          }
           drain_buffer(buf);
         }
 #pragma unroll
@@ -764,11 +807,15 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
     const int first_left = max(tile_base - kBuffers, 0);
     buf = first_left % kBuffers;
     for (int gt = first_left; gt < tile_base; ++gt) {
-      if (!wait_for(&cnt.written[w], gt + 1)) return;
+      if (!wait_for(&cnt.written[w], gt + 1, spin_limit)) {
+        give_up();
+        return;
+      }
       drain_buffer(buf);
       buf = buf + 1 == kBuffers ? 0 : buf + 1;
     }
     if (!zeroed) zero_outside(wave - nsweep, nwaves - nsweep);
+    if (peek(&cnt.failed)) poison();
     // the loss, if asked for: the scores are the forward kernel's, complete before this
     // kernel started, and this wave has nothing left to do
     if (loss && b == 0 && wave == nsweep) reduce_scores(scores, loss, B, reduction, lane);
@@ -808,8 +855,10 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
 #pragma unroll
       for (int l = 0; l < kStagers; ++l)
         if (__builtin_amdgcn_readfirstlane(seen_loaded[l]) < gt + 1 &&
-            !wait_for(&cnt.loaded[w * kStagers + l], gt + 1))
+            !wait_for(&cnt.loaded[w * kStagers + l], gt + 1, spin_limit)) {
+          give_up();
           return;
+        }
       R d1q[kTileSteps], d2q[kTileSteps];
       R *gx_row = base + buf * kTileElems + lane * kTilePitch;               // d1 in, gx out
       R *gy_row = base + (kBuffers + buf) * kTileElems + lane * kTilePitch;  // d2 in, gy out
@@ -826,7 +875,7 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
           const int need = min(e0 + kChunk - shift, cols);
           handed = seen_seam;
           if (need > 0 && __builtin_amdgcn_readfirstlane(seen_ready) < up_base + need) {
-            if (!wait_for(&cnt.ready[prev], up_base + need)) {
+            if (!wait_for(&cnt.ready[prev], up_base + need, spin_limit)) {
               alive = false;
               return;
             }
@@ -901,10 +950,14 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
         else
           tile(std::false_type{}, std::false_type{});
       }
-      if (!alive) return;
+      if (!alive) {
+        give_up();
+        return;
+      }
       if (lane == 0) publish_lds_writes(&cnt.written[w], gt + 1);
     }
-    if (lane == fin_lane && overwrite_ans_grad && ans_grad) ans_grad[b] = g_origin;
+    if (lane == fin_lane && overwrite_ans_grad && ans_grad)
+      ans_grad[b] = peek(&cnt.failed) ? std::numeric_limits<R>::quiet_NaN() : g_origin;
     tile_base += g.ntiles;
   }
 }
@@ -952,7 +1005,7 @@ int forward_impl(const R *px, const R *py, const int64_t *boundary, R *p, R *ans
   if (!allow_lds(reinterpret_cast<const void *>(kernel), lds))
     return check_launch("mi_forward: hipFuncSetAttribute");
   hipLaunchKernelGGL(kernel, dim3(B), dim3(n * (1 + stagers) * kWave), lds,
-                     static_cast<hipStream_t>(stream), px, py, boundary, p, ans, S, T);
+                     static_cast<hipStream_t>(stream), px, py, boundary, p, ans, S, T, g_spin_limit);
   return check_launch("mi_forward");
 }
 
@@ -992,7 +1045,7 @@ int backward_impl(const R *px, const R *py, const int64_t *boundary, const R *p,
     return check_launch("mi_backward: hipFuncSetAttribute");
   hipLaunchKernelGGL(kernel, dim3(B), dim3(n * (1 + stagers) * kWave), lds,
                      static_cast<hipStream_t>(stream), px, boundary, p, ans_grad, px_grad,
-                     py_grad, S, T, overwrite_ans_grad, scores, loss, B, reduction);
+                     py_grad, S, T, overwrite_ans_grad, scores, loss, B, reduction, g_spin_limit);
   return check_launch("mi_backward");
 }
 
@@ -1014,6 +1067,10 @@ int mi_backward_and_loss(const double *px, const int64_t *boundary, const double
 }  // namespace frnnt
 
 extern "C" {
+
+void frnnt_set_spin_limit(int polls) {
+  frnnt::g_spin_limit = polls > 0 ? polls : frnnt::kSpinLimit;
+}
 
 int frnnt_mi_forward_f32(const float *px, const float *py, const int64_t *boundary, float *p,
                          float *ans, int B, int S, int T, int modified, void *stream) {

@@ -48,6 +48,18 @@ int frnnt_version(void);
 const char *frnnt_last_error(void);
 
 /*
+ * Test hook (no counterpart in the reference).  The recursion kernels synchronise their
+ * waves through counters with BOUNDED waits: a wave that polls `polls` times in vain
+ * gives up, and the utterance's outputs are marked -- ans[b] = NaN from the forward
+ * kernel; NaN at the first cell of the window in px_grad and py_grad (and in ans_grad when
+ * it is written back) from the backward kernel -- so a wait that never ends shows as NaN,
+ * never as a plausible number, and every kernel still exits.  The default (2^22 polls,
+ * seconds) is never reached in normal operation; a tiny value lets a test walk that path.
+ * polls <= 0 restores the default.  Process-wide, not synchronised with running launches.
+ */
+void frnnt_set_spin_limit(int polls);
+
+/*
  * Lattice recursion, forward.  Replaces
  *   _fast_rnnt.mutual_information_forward
  *     (fast_rnnt/python/csrc/mutual_information.cu:27-45), i.e.

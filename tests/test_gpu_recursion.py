@@ -249,3 +249,41 @@ def test_joint_recursion_matches_oracle(gpu_device, dtype, modified):
             for n in range(N):
                 assert (dx[n].grad.cpu() - cx[n].grad).abs().max().item() <= gtol * 3
                 assert (dy[n].grad.cpu() - cy[n].grad).abs().max().item() <= gtol * 3
+
+
+def test_a_wait_that_runs_out_shows_as_nan(gpu_device):
+    # The kernels' waves meet through bounded waits.  With the bound set to one poll from the
+    # host every first wait fails (the staged tiles need a memory round trip to arrive): the
+    # kernels must still exit, and mark what they could not finish -- NaN scores from the
+    # forward kernel, NaN at the window's first cell of px_grad / py_grad and in the
+    # written-back ans_grad from the backward kernel.  Afterwards everything is normal again.
+    from fast_rnnt_amd import _lib
+    dev = gpu_device
+    g = torch.Generator().manual_seed(12)
+    B, S, T = 6, 80, 250
+    px = torch.randn(B, S, T + 1, generator=g).to(dev)
+    py = torch.randn(B, S + 1, T, generator=g).to(dev)
+    bnd = torch.tensor([[0, 0, S, T], [2, 3, 70, 200]] * 3).to(dev)
+    p = torch.empty(B, S + 1, T + 1, device=dev)
+    good = _fast_rnnt.mutual_information_forward(px, py, bnd, p)
+    lib = _lib.load()
+    lib.frnnt_set_spin_limit(1)
+    try:
+        _say("forward with a one-poll bound")
+        q = torch.empty_like(p)
+        ans = _fast_rnnt.mutual_information_forward(px, py, bnd, q)
+        torch.cuda.synchronize()
+        assert torch.isnan(ans).all()
+        _say("backward with a one-poll bound")
+        seed = torch.ones(B, device=dev)
+        gx, gy = _fast_rnnt.mutual_information_backward(px, py, bnd, p, seed)
+        torch.cuda.synchronize()
+        rows = bnd.cpu().tolist()
+        for b, (s0, t0, _, _) in enumerate(rows):
+            assert math.isnan(gx[b, s0, t0].item()) and math.isnan(gy[b, s0, t0].item())
+        assert torch.isnan(seed).all()
+    finally:
+        lib.frnnt_set_spin_limit(0)
+    again = _fast_rnnt.mutual_information_forward(px, py, bnd, torch.empty_like(p))
+    gx, gy = _fast_rnnt.mutual_information_backward(px, py, bnd, p, torch.ones(B, device=dev))
+    assert torch.equal(again, good) and torch.isfinite(gx).all() and torch.isfinite(gy).all()
