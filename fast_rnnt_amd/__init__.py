@@ -21,3 +21,6 @@ from .rnnt_loss import rnnt_loss
 from .rnnt_loss import rnnt_loss_pruned
 from .rnnt_loss import rnnt_loss_simple
 from .rnnt_loss import rnnt_loss_smoothed
+
+# beyond the reference's export list: the joiner's input without the gathered copy
+from .rnnt_loss import pruned_joiner_input

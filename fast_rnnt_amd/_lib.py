@@ -53,6 +53,10 @@ _SIGNATURES = {
     "frnnt_prune_gather_f64": ([_P] * 3 + [_I] * 5 + [_P], _I),
     "frnnt_prune_gather_bwd_f32": ([_P] * 3 + [_I] * 5 + [_P], _I),
     "frnnt_prune_gather_bwd_f64": ([_P] * 3 + [_I] * 5 + [_P], _I),
+    "frnnt_pruned_joiner_fwd_f32": ([_P] * 4 + [_I] * 6 + [_P], _I),
+    "frnnt_pruned_joiner_fwd_f64": ([_P] * 4 + [_I] * 6 + [_P], _I),
+    "frnnt_pruned_joiner_bwd_f32": ([_P] * 5 + [_I] * 6 + [_P], _I),
+    "frnnt_pruned_joiner_bwd_f64": ([_P] * 5 + [_I] * 6 + [_P], _I),
 }
 
 

@@ -244,10 +244,14 @@ constexpr int kScanChunk = 256 * kScanPerThread;
 // a round must be able to take a whole chunk of matches, or it would make no progress
 static_assert(kHitCapacity >= kScanChunk, "a chunk of matches must fit in the list");
 
+// With `act_out` (the tanh outputs the gradient belongs to, same shape as grad) every
+// gradient entry is first multiplied by the activation's derivative 1 - out^2: the adjoint
+// of the fused joiner input below, which never materialises the gathered rows.
 template <typename R>
 __global__ void __launch_bounds__(256)
-    prune_scatter_kernel(const R *__restrict__ grad, const int64_t *__restrict__ ranges,
-                         R *__restrict__ lm_grad, int TR, int S1, int C) {
+    prune_scatter_kernel(const R *__restrict__ grad, const R *__restrict__ act_out,
+                         const int64_t *__restrict__ ranges, R *__restrict__ lm_grad, int TR,
+                         int S1, int C) {
   __shared__ int hits[kHitCapacity];
   __shared__ int wave_count[4];
   __shared__ __align__(16) float meet[4 * 512];  // the four waves' sums of 512 columns
@@ -255,6 +259,7 @@ __global__ void __launch_bounds__(256)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t *rb = ranges + (long)b * TR;
   const R *gb = grad + (long)b * TR * C;
+  const R *ob = act_out ? act_out + (long)b * TR * C : nullptr;
   R *dst = lm_grad + ((long)b * S1 + s) * C;
   bool first_round = true;
   int k_next = 0;
@@ -308,11 +313,19 @@ __global__ void __launch_bounds__(256)
       typedef int intx4 __attribute__((ext_vector_type(4)));
       const __amdgpu_buffer_rsrc_t g_rs = __builtin_amdgcn_make_buffer_rsrc(
           const_cast<float *>(reinterpret_cast<const float *>(gb)), 0, TR * C * 4, 0x00020000);
+      // (without activation outputs the second resource is empty: its loads return 0)
+      const __amdgpu_buffer_rsrc_t o_rs = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<float *>(reinterpret_cast<const float *>(ob ? ob : gb)), 0,
+          ob ? TR * C * 4 : 0, 0x00020000);
       constexpr int kNowhere = (int)0x80000000;
       auto row_piece = [&](int byte_offset) {
         const intx4 w = __builtin_amdgcn_raw_buffer_load_b128(g_rs, byte_offset, 0, 0);
-        return f4{__int_as_float(w[0]), __int_as_float(w[1]), __int_as_float(w[2]),
+        const intx4 o = __builtin_amdgcn_raw_buffer_load_b128(o_rs, byte_offset, 0, 0);
+        f4 g = f4{__int_as_float(w[0]), __int_as_float(w[1]), __int_as_float(w[2]),
                   __int_as_float(w[3])};
+        const f4 y = f4{__int_as_float(o[0]), __int_as_float(o[1]), __int_as_float(o[2]),
+                        __int_as_float(o[3])};
+        return g * (1.f - y * y);  // y = 0 without an activation
       };
       float *df = reinterpret_cast<float *>(dst);
       f4 *meet4 = reinterpret_cast<f4 *>(meet);
@@ -349,23 +362,30 @@ __global__ void __launch_bounds__(256)
         const int c = c0 + tid;
         if (c >= C) continue;
         R acc = first_round ? (R)0 : dst[c];
+        auto entry = [&](int i) -> R {
+          const long at = (long)hits[i] * C + c;
+          const R g = gb[at];
+          if (!ob) return g;
+          const R y = ob[at];
+          return g * ((R)1 - y * y);
+        };
         int i = 0;
         for (; i + 8 <= n; i += 8) {
           R g[8];
 #pragma unroll
-          for (int u = 0; u < 8; ++u) g[u] = gb[(long)hits[i + u] * C + c];
+          for (int u = 0; u < 8; ++u) g[u] = entry(i + u);
 #pragma unroll
           for (int u = 0; u < 8; ++u) acc += g[u];
         }
         if (i + 4 <= n) {
           R g[4];
 #pragma unroll
-          for (int u = 0; u < 4; ++u) g[u] = gb[(long)hits[i + u] * C + c];
+          for (int u = 0; u < 4; ++u) g[u] = entry(i + u);
 #pragma unroll
           for (int u = 0; u < 4; ++u) acc += g[u];
           i += 4;
         }
-        for (; i < n; ++i) acc += gb[(long)hits[i] * C + c];
+        for (; i < n; ++i) acc += entry(i);
         dst[c] = acc;
       }
     }
@@ -445,8 +465,158 @@ int scatter_impl(const R *grad, const int64_t *ranges, R *lm_grad, int B, int S,
   if (!lm_grad || ((long)T * Rr > 0 && (!grad || !ranges)))
     return fail(FRNNT_EINVAL, "prune_gather_bwd: null pointer");
   hipLaunchKernelGGL(prune_scatter_kernel<R>, dim3((unsigned)(B * (S + 1))), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), grad, ranges, lm_grad, T * Rr, S + 1, C);
+                     static_cast<hipStream_t>(stream), grad, (const R *)nullptr, ranges, lm_grad,
+                     T * Rr, S + 1, C);
   return check_launch("prune_gather_bwd");
+}
+
+// ---- the joiner's input without the gathered copy ------------------------------------------
+// out[b,t,j,:] = act(am[b,t,:] + lm[b, ranges[b,t,j], :]) in one pass: what a joiner of the
+// usual form does first with the two tensors do_rnnt_pruning returns (README "pruned
+// rnnt loss" recipe: logits = joiner(am_pruned, lm_pruned)), without lm_pruned [B,T,R,C]
+// ever existing.  One wave per output row; 16-byte accesses when the rows allow.
+enum { kActNone = 0, kActTanh = 1 };
+__device__ __forceinline__ float act_tanh(float x) { return tanhf(x); }
+__device__ __forceinline__ double act_tanh(double x) { return tanh(x); }
+
+template <typename R>
+__global__ void __launch_bounds__(256)
+    joiner_input_kernel(const R *__restrict__ am, const R *__restrict__ lm,
+                        const int64_t *__restrict__ ranges, R *__restrict__ out, long rows, int Rr,
+                        int TR, int S1, int C, int activation) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // in a scalar register
+  const long row = (long)blockIdx.x * 4 + wave;
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const long b = row / TR;
+  const int64_t s = ranges[row];
+  const bool valid = s >= 0 && s < S1;
+  const R *a = am + (row / Rr) * C;
+  const R *l = lm + (b * S1 + (valid ? s : 0)) * C;
+  R *dst = out + row * C;
+  const R nan = std::numeric_limits<R>::quiet_NaN();
+  constexpr int kPer = 16 / (int)sizeof(R);
+  typedef R Piece __attribute__((ext_vector_type(kPer), aligned(sizeof(R))));
+  if (C % kPer == 0) {
+    // two pieces per lane in flight from each source
+    for (int c0 = kPer * lane; c0 < C; c0 += 2 * kPer * kWave) {
+      const int c1 = c0 + kPer * kWave;
+      const bool second = c1 < C;
+      const Piece a0 = *reinterpret_cast<const Piece *>(a + c0);
+      const Piece l0 = *reinterpret_cast<const Piece *>(l + c0);
+      Piece a1 = a0, l1 = l0;
+      if (second) {
+        a1 = *reinterpret_cast<const Piece *>(a + c1);
+        l1 = *reinterpret_cast<const Piece *>(l + c1);
+      }
+      Piece y0, y1;
+#pragma unroll
+      for (int e = 0; e < kPer; ++e) {
+        const R v0 = a0[e] + l0[e], v1 = a1[e] + l1[e];
+        y0[e] = !valid ? nan : (activation == kActTanh ? act_tanh(v0) : v0);
+        y1[e] = !valid ? nan : (activation == kActTanh ? act_tanh(v1) : v1);
+      }
+      *reinterpret_cast<Piece *>(dst + c0) = y0;
+      if (second) *reinterpret_cast<Piece *>(dst + c1) = y1;
+    }
+  } else {
+    for (int c = lane; c < C; c += kWave) {
+      const R v = a[c] + l[c];
+      dst[c] = !valid ? nan : (activation == kActTanh ? act_tanh(v) : v);
+    }
+  }
+}
+
+// am.grad[b,t,:] = sum_j grad[b,t,j,:] * act'(out[b,t,j,:]), j in order: one wave per frame.
+template <typename R>
+__global__ void __launch_bounds__(256)
+    joiner_input_am_grad_kernel(const R *__restrict__ grad, const R *__restrict__ act_out,
+                                R *__restrict__ am_grad, long frames, int Rr, int C) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const long frame = (long)blockIdx.x * 4 + wave;
+  const int lane = threadIdx.x & 63;
+  if (frame >= frames) return;
+  const R *g = grad + frame * Rr * C;
+  const R *o = act_out ? act_out + frame * Rr * C : nullptr;
+  R *dst = am_grad + frame * C;
+  constexpr int kPer = 16 / (int)sizeof(R);
+  typedef R Piece __attribute__((ext_vector_type(kPer), aligned(sizeof(R))));
+  if (C % kPer == 0) {
+    for (int c = kPer * lane; c < C; c += kPer * kWave) {
+      Piece acc;
+#pragma unroll
+      for (int e = 0; e < kPer; ++e) acc[e] = 0;
+      int j = 0;
+      for (; j + 4 <= Rr; j += 4) {  // four rows in flight
+        Piece gv[4], ov[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          gv[u] = *reinterpret_cast<const Piece *>(g + (long)(j + u) * C + c);
+          if (o) ov[u] = *reinterpret_cast<const Piece *>(o + (long)(j + u) * C + c);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int e = 0; e < kPer; ++e)
+            acc[e] += o ? gv[u][e] * ((R)1 - ov[u][e] * ov[u][e]) : gv[u][e];
+      }
+      for (; j < Rr; ++j) {
+        const Piece gv = *reinterpret_cast<const Piece *>(g + (long)j * C + c);
+        Piece ov = gv;
+        if (o) ov = *reinterpret_cast<const Piece *>(o + (long)j * C + c);
+#pragma unroll
+        for (int e = 0; e < kPer; ++e) acc[e] += o ? gv[e] * ((R)1 - ov[e] * ov[e]) : gv[e];
+      }
+      *reinterpret_cast<Piece *>(dst + c) = acc;
+    }
+  } else {
+    for (int c = lane; c < C; c += kWave) {
+      R acc = 0;
+      for (int j = 0; j < Rr; ++j) {
+        const R gv = g[(long)j * C + c];
+        acc += o ? gv * ((R)1 - o[(long)j * C + c] * o[(long)j * C + c]) : gv;
+      }
+      dst[c] = acc;
+    }
+  }
+}
+
+template <typename R>
+int joiner_fwd_impl(const R *am, const R *lm, const int64_t *ranges, R *out, int B, int S, int T,
+                    int Rr, int C, int activation, void *stream) {
+  if (B < 0 || S < 0 || T < 0 || Rr < 0 || C < 0)
+    return fail(FRNNT_EINVAL, "pruned_joiner_fwd: negative size");
+  if (activation != kActNone && activation != kActTanh)
+    return fail(FRNNT_EINVAL, "pruned_joiner_fwd: activation must be 0 (none) or 1 (tanh)");
+  const long rows = (long)B * T * Rr;
+  if (rows == 0 || C == 0) return FRNNT_OK;
+  if (!am || !lm || !ranges || !out) return fail(FRNNT_EINVAL, "pruned_joiner_fwd: null pointer");
+  hipLaunchKernelGGL(joiner_input_kernel<R>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), am, lm, ranges, out, rows, Rr, T * Rr, S + 1,
+                     C, activation);
+  return check_launch("pruned_joiner_fwd");
+}
+
+template <typename R>
+int joiner_bwd_impl(const R *grad, const R *out, const int64_t *ranges, R *am_grad, R *lm_grad,
+                    int B, int S, int T, int Rr, int C, int activation, void *stream) {
+  if (B < 0 || S < 0 || T < 0 || Rr < 0 || C < 0)
+    return fail(FRNNT_EINVAL, "pruned_joiner_bwd: negative size");
+  if (activation != kActNone && activation != kActTanh)
+    return fail(FRNNT_EINVAL, "pruned_joiner_bwd: activation must be 0 (none) or 1 (tanh)");
+  if (B == 0 || C == 0) return FRNNT_OK;
+  const long frames = (long)B * T;
+  if ((long)T * Rr > 0 && (!grad || !ranges || (activation == kActTanh && !out)))
+    return fail(FRNNT_EINVAL, "pruned_joiner_bwd: null pointer");
+  const R *act_out = activation == kActTanh ? out : nullptr;
+  if (am_grad && frames > 0)
+    hipLaunchKernelGGL(joiner_input_am_grad_kernel<R>, dim3((unsigned)((frames + 3) / 4)), dim3(256),
+                       0, static_cast<hipStream_t>(stream), grad, act_out, am_grad, frames, Rr, C);
+  if (lm_grad)
+    hipLaunchKernelGGL(prune_scatter_kernel<R>, dim3((unsigned)(B * (S + 1))), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), grad, act_out, ranges, lm_grad, T * Rr,
+                       S + 1, C);
+  return check_launch("pruned_joiner_bwd");
 }
 
 }  // namespace
@@ -481,6 +651,27 @@ int frnnt_prune_gather_bwd_f32(const float *grad, const int64_t *ranges, float *
 int frnnt_prune_gather_bwd_f64(const double *grad, const int64_t *ranges, double *lm_grad, int B,
                                int S, int T, int R, int C, void *stream) {
   return frnnt::scatter_impl<double>(grad, ranges, lm_grad, B, S, T, R, C, stream);
+}
+int frnnt_pruned_joiner_fwd_f32(const float *am, const float *lm, const int64_t *ranges, float *out,
+                                int B, int S, int T, int R, int C, int activation, void *stream) {
+  return frnnt::joiner_fwd_impl<float>(am, lm, ranges, out, B, S, T, R, C, activation, stream);
+}
+int frnnt_pruned_joiner_fwd_f64(const double *am, const double *lm, const int64_t *ranges,
+                                double *out, int B, int S, int T, int R, int C, int activation,
+                                void *stream) {
+  return frnnt::joiner_fwd_impl<double>(am, lm, ranges, out, B, S, T, R, C, activation, stream);
+}
+int frnnt_pruned_joiner_bwd_f32(const float *grad, const float *out, const int64_t *ranges,
+                                float *am_grad, float *lm_grad, int B, int S, int T, int R, int C,
+                                int activation, void *stream) {
+  return frnnt::joiner_bwd_impl<float>(grad, out, ranges, am_grad, lm_grad, B, S, T, R, C,
+                                       activation, stream);
+}
+int frnnt_pruned_joiner_bwd_f64(const double *grad, const double *out, const int64_t *ranges,
+                                double *am_grad, double *lm_grad, int B, int S, int T, int R, int C,
+                                int activation, void *stream) {
+  return frnnt::joiner_bwd_impl<double>(grad, out, ranges, am_grad, lm_grad, B, S, T, R, C,
+                                        activation, stream);
 }
 
 }  // extern "C"

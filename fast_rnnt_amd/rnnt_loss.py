@@ -555,6 +555,70 @@ def do_rnnt_pruning(am: Tensor, lm: Tensor, ranges: Tensor) -> Tuple[Tensor, Ten
     return am_pruning, lm_pruning
 
 
+_ACTIVATIONS = {None: 0, "none": 0, "tanh": 1}
+
+
+class _PrunedJoinerInput(torch.autograd.Function):
+    """act(am[b,t] + lm[b, ranges[b,t,j]]): frnnt_pruned_joiner_fwd / _bwd."""
+
+    @staticmethod
+    def forward(ctx, am, lm, ranges, activation):
+        B, S1, C = lm.shape
+        _, T, R = ranges.shape
+        sfx = _lib.suffix(lm.dtype)
+        am_c, lm_c, rng_c = am.contiguous(), lm.contiguous(), ranges.contiguous()
+        with _on_device(lm.device):
+            out = torch.empty(B, T, R, C, dtype=lm.dtype, device=lm.device)
+            _lib.call("frnnt_pruned_joiner_fwd_" + sfx, am_c.data_ptr(), lm_c.data_ptr(),
+                      rng_c.data_ptr(), out.data_ptr(), B, S1 - 1, T, R, C, activation,
+                      _lib.stream_of(lm))
+        ctx.save_for_backward(rng_c, out if activation else None)
+        ctx.meta = (B, S1, T, R, C, activation, sfx)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        rng, out = ctx.saved_tensors
+        B, S1, T, R, C, activation, sfx = ctx.meta
+        grad = grad.contiguous()
+        with _on_device(grad.device):
+            am_grad = (torch.empty(B, T, C, dtype=grad.dtype, device=grad.device)
+                       if ctx.needs_input_grad[0] else None)
+            lm_grad = (torch.empty(B, S1, C, dtype=grad.dtype, device=grad.device)
+                       if ctx.needs_input_grad[1] else None)
+            _lib.call("frnnt_pruned_joiner_bwd_" + sfx, grad.data_ptr(), _lib.ptr(out),
+                      rng.data_ptr(), _lib.ptr(am_grad), _lib.ptr(lm_grad), B, S1 - 1, T, R, C,
+                      activation, _lib.stream_of(grad))
+        return am_grad, lm_grad, None, None
+
+
+def pruned_joiner_input(am: Tensor, lm: Tensor, ranges: Tensor,
+                        activation: Optional[str] = "tanh") -> Tensor:
+    """``act(am_pruned + lm_pruned)`` of shape ``(B, T, s_range, C)`` in one pass.
+
+    The usual joiner starts with ``tanh(am_pruned + lm_pruned)`` on the two tensors
+    :func:`do_rnnt_pruning` returns (the reference's recipe, README.md:193-215, with
+    rnnt_loss.py:780-818).  This op consumes ``ranges`` directly::
+
+        out[b, t, j, :] = act(am[b, t, :] + lm[b, ranges[b, t, j], :])
+
+    so the gathered copy ``lm_pruned`` (80 MB at B=32, T=250, s_range=5, C=500) is never
+    written or read back, and the backward pass sums straight into ``am.grad`` and -- with
+    the deterministic per-row segmented sum of the pruning gather's adjoint -- ``lm.grad``.
+    ``activation`` is ``"tanh"`` or ``None`` (the plain sum).  It has no counterpart in the
+    reference, whose callers obtain the same values with two more passes over
+    ``(B, T, s_range, C)``; :func:`do_rnnt_pruning` stays as it is for them.
+    """
+    assert ranges.shape[0] == am.shape[0], (ranges.shape[0], am.shape[0])
+    assert ranges.shape[0] == lm.shape[0], (ranges.shape[0], lm.shape[0])
+    assert am.shape[1] == ranges.shape[1], (am.shape[1], ranges.shape[1])
+    assert am.shape[2] == lm.shape[2], (am.shape[2], lm.shape[2])
+    if activation not in _ACTIVATIONS:
+        raise ValueError(f"activation should be ('tanh' | None), given {activation}")
+    _check_tensors([("am", am), ("lm", lm)], [("ranges", ranges)])
+    return _PrunedJoinerInput.apply(am, lm, ranges, _ACTIVATIONS[activation])
+
+
 def _roll_by_shifts(src: Tensor, shifts: torch.LongTensor):
     """``out[b,t,s] = src[b,t,(s - shifts[b,t]) mod S]`` (rnnt_loss.py:821-853).
     The fused pruned-logprob kernel applies this roll itself; kept for callers."""

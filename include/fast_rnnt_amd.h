@@ -355,6 +355,31 @@ int frnnt_prune_gather_bwd_f32(const float *grad, const int64_t *ranges, float *
 int frnnt_prune_gather_bwd_f64(const double *grad, const int64_t *ranges, double *lm_grad, int B,
                                int S, int T, int R, int C, void *stream);
 
+/*
+ * The joiner's input straight from the pruning bounds:
+ *   out[b][t][j][:] = act(am[b][t][:] + lm[b][ranges[b][t][j]][:])
+ * i.e. what a joiner of the usual form computes first from the two tensors of
+ * do_rnnt_pruning (rnnt_loss.py:780-818; README.md:193-215: logits =
+ * joiner(am_pruned, lm_pruned)), in one pass and without lm_pruned [B][T][R][C] ever
+ * existing.  activation: 0 = none (the plain sum), 1 = tanh.  Rows whose range entry lies
+ * outside [0, S] are NaN, as in frnnt_prune_gather.
+ * Backward: grad is dL/dout, out the forward's result (read for tanh only);
+ *   am_grad[b][t][:] = sum_j grad * act'      lm_grad[b][s][:] = sum over the (t, j) with
+ * ranges[b][t][j] = s of grad * act', in frame order (deterministic, no atomics); either
+ * output may be NULL.
+ */
+int frnnt_pruned_joiner_fwd_f32(const float *am, const float *lm, const int64_t *ranges, float *out,
+                                int B, int S, int T, int R, int C, int activation, void *stream);
+int frnnt_pruned_joiner_fwd_f64(const double *am, const double *lm, const int64_t *ranges,
+                                double *out, int B, int S, int T, int R, int C, int activation,
+                                void *stream);
+int frnnt_pruned_joiner_bwd_f32(const float *grad, const float *out, const int64_t *ranges,
+                                float *am_grad, float *lm_grad, int B, int S, int T, int R, int C,
+                                int activation, void *stream);
+int frnnt_pruned_joiner_bwd_f64(const double *grad, const double *out, const int64_t *ranges,
+                                double *am_grad, double *lm_grad, int B, int S, int T, int R, int C,
+                                int activation, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -455,6 +455,48 @@ def test_losses_do_not_read_logits_outside_the_window(gpu_device, dtype, kind):
         assert _close(grad[in_p], a.grad[in_p], 1e-4 if f32 else 1e-9, 1e-4 if f32 else 1e-9)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_pruned_joiner_input_matches_gather_then_tanh(gpu_device, dtype):
+    # pruned_joiner_input(am, lm, ranges) == tanh(am_pruned + lm_pruned) on the oracle's
+    # do_rnnt_pruning (rnnt_loss.py:780-818), values and both gradients; also the plain sum,
+    # rows that are not multiples of 16 bytes, and range entries outside [0, S] (NaN rows)
+    dev = gpu_device
+    f32 = dtype == torch.float32
+    for n, (B, S, T, R, C) in enumerate([(2, 5, 9, 3, 8), (3, 20, 41, 5, 500), (2, 30, 25, 7, 37),
+                                         (2, 12, 16, 13, 260)]):
+        g = torch.Generator().manual_seed(700 + n)
+        am = torch.randn(B, T, C, generator=g, dtype=dtype)
+        lm = torch.randn(B, S + 1, C, generator=g, dtype=dtype)
+        start = torch.randint(0, S + 2 - R, (B, T), generator=g)
+        ranges = (start.unsqueeze(2) + torch.arange(R).reshape(1, 1, R)).contiguous()
+        weight = torch.randn(B, T, R, C, generator=g, dtype=dtype)
+        for act in ("tanh", None):
+            _say(f"pruned joiner input {dtype} shape{n} activation={act}")
+            a = am.clone().requires_grad_(True)
+            l = lm.clone().requires_grad_(True)
+            am_p, lm_p = O.prune(a, l, ranges)
+            want = torch.tanh(am_p + lm_p) if act else am_p + lm_p
+            (want * weight).sum().backward()
+            da = am.to(dev).requires_grad_(True)
+            dl = lm.to(dev).requires_grad_(True)
+            got = fast_rnnt_amd.pruned_joiner_input(da, dl, ranges.to(dev), activation=act)
+            (got * weight.to(dev)).sum().backward()
+            tol = 2e-6 if f32 else 1e-12
+            assert _close(got, want, tol, tol)
+            assert _close(da.grad, a.grad, 1e-5 if f32 else 1e-11, 1e-5 if f32 else 1e-11)
+            assert _close(dl.grad, l.grad, 2e-5 if f32 else 1e-11, 1e-5 if f32 else 1e-11)
+            # the same numbers as the two-step route through do_rnnt_pruning on the GPU
+            ea = am.to(dev).requires_grad_(True)
+            el = lm.to(dev).requires_grad_(True)
+            p_am, p_lm = fast_rnnt_amd.do_rnnt_pruning(ea, el, ranges.to(dev))
+            two = torch.tanh(p_am + p_lm) if act else p_am + p_lm
+            assert _close(got, two, tol, tol)
+    bad = ranges.clone()
+    bad[0, 0, 0] = S + 1
+    out = fast_rnnt_amd.pruned_joiner_input(am.to(dev), lm.to(dev), bad.to(dev))
+    assert torch.isnan(out[0, 0, 0]).all() and torch.isfinite(out[0, 0, 1]).all()
+
+
 def test_c5_unpruned_full_size(gpu_device):
     dev = gpu_device
     w = workloads.make("c5")
