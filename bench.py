@@ -53,6 +53,9 @@ def _parse():
     ap.add_argument("--kernel-reps", type=int, default=50)
     ap.add_argument("--no-graph", dest="graph", action="store_false",
                     help="skip the graph-replay leg")
+    ap.add_argument("--logits-dtype", default="f32", choices=["f32", "f16", "bf16"],
+                    help="c3 / c5: element type of the logits handed to the loss (the 2-byte "
+                         "types are read as they are and accumulated in float32)")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run device-to-device copies of this size (a reference of known "
                          "traffic for hardware-counter runs)")
@@ -267,8 +270,11 @@ def _bench_lattice(args, w, dev):
     table, traffic_file = _measured_traffic(w.name)
     sym, bnd = w.symbols.to(dev), w.boundary.to(dev)
     extra = {}
+    ldt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[args.logits_dtype]
+    esize = 4 if args.logits_dtype == "f32" else 2
+    sfx = args.logits_dtype
     if w.name == "c5":
-        logits = w.logits.to(dev).requires_grad_(True)
+        logits = w.logits.to(dev).to(ldt).requires_grad_(True)
 
         def step():
             logits.grad = None
@@ -279,7 +285,7 @@ def _bench_lattice(args, w, dev):
         def grads():
             return (logits.grad,)
 
-        cl = w.logits.clone().requires_grad_(True)
+        cl = w.logits.to(ldt).float().requires_grad_(True)
 
         def cpu_step():
             cl.grad = None
@@ -308,7 +314,7 @@ def _bench_lattice(args, w, dev):
             else:
                 am_p, lm_p = fast_rnnt_amd.do_rnnt_pruning(am, lm, rg)
                 hidden = torch.tanh(am_p + lm_p)
-            loss = fast_rnnt_amd.rnnt_loss_pruned(hidden @ W, sym, rg, 0, boundary=bnd,
+            loss = fast_rnnt_amd.rnnt_loss_pruned((hidden @ W).to(ldt), sym, rg, 0, boundary=bnd,
                                                   reduction="sum")
             (simple + loss).backward()
             return loss
@@ -330,8 +336,8 @@ def _bench_lattice(args, w, dev):
                                                return_grad=True)
             rg = O.prune_ranges(gx, gy, w.boundary, w.s_range)
             am_p, lm_p = O.prune(ca, cl, rg)
-            loss = O.loss_pruned(torch.tanh(am_p + lm_p) @ w.joiner, w.symbols, rg, 0,
-                                 boundary=w.boundary, reduction="sum")
+            loss = O.loss_pruned((torch.tanh(am_p + lm_p) @ w.joiner).to(ldt).float(), w.symbols,
+                                 rg, 0, boundary=w.boundary, reduction="sum")
             (simple + loss).backward()
             return loss
 
@@ -340,7 +346,7 @@ def _bench_lattice(args, w, dev):
                 lm, am, sym, 0, 0.25, 0.0, boundary=bnd, reduction="sum", return_grad=True)
             ranges = fast_rnnt_amd.get_rnnt_prune_ranges(gx, gy, bnd, w.s_range)
             hidden = fast_rnnt_amd.pruned_joiner_input(am, lm, ranges, activation="tanh")
-            lg = (hidden @ W).contiguous()
+            lg = (hidden @ W).to(ldt).contiguous()
         R = w.s_range
         what = (f"c3: rnnt_loss_smoothed -> get_rnnt_prune_ranges -> do_rnnt_pruning -> joiner "
                 f"(tanh of the sum, [C,C] projection) -> rnnt_loss_pruned fwd+bwd, B={w.B} T={w.T} "
@@ -351,7 +357,7 @@ def _bench_lattice(args, w, dev):
         fused = _rate(args.steps, _wall_loop(lambda: pipeline(True), args.steps, args.warmup))
         # the caller's joiner (not part of the library): the [B*T*R, C] x [C, C] product,
         # forward and its two backward products
-        g_out = torch.empty_like(lg)
+        g_out = torch.empty_like(lg, dtype=torch.float32)
         h2 = hidden.reshape(-1, w.C)
 
         def joiner_products():
@@ -383,18 +389,18 @@ def _bench_lattice(args, w, dev):
     rp = _lib.ptr(ranges)
 
     def fwd():
-        _lib.call("frnnt_lattice_logprobs_fwd_f32", lg.data_ptr(), sym.data_ptr(), rp,
+        _lib.call("frnnt_lattice_logprobs_fwd_" + sfx, lg.data_ptr(), sym.data_ptr(), rp,
                   bnd.data_ptr(), px.data_ptr(), py.data_ptr(), norm.data_ptr(), xr.data_ptr(),
                   yr.data_ptr(), B, S, T, R, C, 0, 0, 1, stream)
 
     def bwd():
-        _lib.call("frnnt_lattice_logprobs_bwd_f32", lg.data_ptr(), sym.data_ptr(), rp,
+        _lib.call("frnnt_lattice_logprobs_bwd_" + sfx, lg.data_ptr(), sym.data_ptr(), rp,
                   bnd.data_ptr(), norm.data_ptr(), gpx.data_ptr(), gpy.data_ptr(), grad.data_ptr(),
                   B, S, T, R, C, 0, 0, 1, stream)
 
     t_f = _event_time_ms(fwd, args.kernel_reps)
     t_b = _event_time_ms(bwd, args.kernel_reps)
-    nbytes = lg.numel() * 4
+    nbytes = lg.numel() * esize
     # rows of the logits inside the windows: frames < T_b and (c5) lattice rows <= S_b;
     # for c3 the range rows of a frame that fall on lattice rows <= S_b
     if ranges is None:
@@ -405,13 +411,14 @@ def _bench_lattice(args, w, dev):
         t_ok = torch.arange(T).reshape(1, T, 1) < w.boundary[:, 3].reshape(B, 1, 1)
         s_ok = rg <= w.boundary[:, 2].reshape(B, 1, 1)
         rows_in = int((t_ok & s_ok).sum().item())
-    in_bytes = rows_in * C * 4
+    in_bytes = rows_in * C * esize
     # gradient kernel: reads the rows inside the windows, writes every row (zeros outside);
     # normalizer kernel: reads the rows inside the windows
     lines = [
-        _hbm_line(table, "row_grad_regs_kernel", in_bytes + nbytes, t_b,
-                  padded_bytes=2 * nbytes),
-        _hbm_line(table, "row_norm_regs_kernel", in_bytes, t_f, padded_bytes=nbytes,
+        _hbm_line(table, "row_grad_regs_kernel" if esize == 4 else "row_grad_narrow_kernel",
+                  in_bytes + nbytes, t_b, padded_bytes=2 * nbytes),
+        _hbm_line(table, "row_norm_regs_kernel" if esize == 4 else "row_norm_narrow_kernel",
+                  in_bytes, t_f, padded_bytes=nbytes,
                   note="launch time includes the small assemble_kernel of the same entry point"),
     ]
     lines.sort(key=lambda r: -r["avg_launch_us"])
@@ -424,7 +431,8 @@ def _bench_lattice(args, w, dev):
         "value": best["value"], "unit": "calls/sec", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": best["ms_per_step"], "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if esize == 4 else f"f32 arithmetic on {sfx} logits", "data": "synthetic",
         "config": {"workload": what, "logits_bytes": nbytes,
                    "logits_bytes_inside_windows": in_bytes,
                    "mode": "HIP-graph replay of one captured step" if graphed else "eager calls"},

@@ -47,12 +47,20 @@ _SIGNATURES = {
     "frnnt_lattice_logprobs_fwd_f64": ([_P] * 9 + [_I] * 8 + [_P], _I),
     "frnnt_lattice_logprobs_bwd_f32": ([_P] * 8 + [_I] * 8 + [_P], _I),
     "frnnt_lattice_logprobs_bwd_f64": ([_P] * 8 + [_I] * 8 + [_P], _I),
+    "frnnt_lattice_logprobs_fwd_f16": ([_P] * 9 + [_I] * 8 + [_P], _I),
+    "frnnt_lattice_logprobs_fwd_bf16": ([_P] * 9 + [_I] * 8 + [_P], _I),
+    "frnnt_lattice_logprobs_bwd_f16": ([_P] * 8 + [_I] * 8 + [_P], _I),
+    "frnnt_lattice_logprobs_bwd_bf16": ([_P] * 8 + [_I] * 8 + [_P], _I),
     "frnnt_prune_ranges_f32": ([_P] * 4 + [_I] * 5 + [_P], _I),
     "frnnt_prune_ranges_f64": ([_P] * 4 + [_I] * 5 + [_P], _I),
     "frnnt_prune_gather_f32": ([_P] * 3 + [_I] * 5 + [_P], _I),
     "frnnt_prune_gather_f64": ([_P] * 3 + [_I] * 5 + [_P], _I),
     "frnnt_prune_gather_bwd_f32": ([_P] * 3 + [_I] * 5 + [_P], _I),
     "frnnt_prune_gather_bwd_f64": ([_P] * 3 + [_I] * 5 + [_P], _I),
+    "frnnt_prune_gather_f16": ([_P] * 3 + [_I] * 5 + [_P], _I),
+    "frnnt_prune_gather_bf16": ([_P] * 3 + [_I] * 5 + [_P], _I),
+    "frnnt_prune_gather_bwd_f16": ([_P] * 3 + [_I] * 5 + [_P], _I),
+    "frnnt_prune_gather_bwd_bf16": ([_P] * 3 + [_I] * 5 + [_P], _I),
     "frnnt_pruned_joiner_fwd_f32": ([_P] * 4 + [_I] * 6 + [_P], _I),
     "frnnt_pruned_joiner_fwd_f64": ([_P] * 4 + [_I] * 6 + [_P], _I),
     "frnnt_pruned_joiner_bwd_f32": ([_P] * 5 + [_I] * 6 + [_P], _I),
@@ -98,12 +106,18 @@ def stream_of(t: "torch.Tensor"):
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
-def suffix(dtype) -> str:
+def suffix(dtype, narrow: bool = False) -> str:
+    """Entry-point suffix of a tensor type; `narrow` also admits the 2-byte types, for
+    the entry points that have a float16 / bfloat16 form."""
     if dtype == torch.float32:
         return "f32"
     if dtype == torch.float64:
         return "f64"
-    raise RuntimeError(f"fast_rnnt_amd supports float32 and float64 tensors, got {dtype}")
+    if narrow and dtype == torch.float16:
+        return "f16"
+    if narrow and dtype == torch.bfloat16:
+        return "bf16"
+    raise RuntimeError(f"fast_rnnt_amd supports float32 and float64 tensors here, got {dtype}")
 
 
 def ptr(t):

@@ -44,6 +44,52 @@ struct Num<double> {
   static __device__ __forceinline__ double log1p_(double x) { return log1p(x); }
 };
 
+// ---- 2-byte floating-point storage (float16, bfloat16): memory holds the 16-bit
+// patterns, arithmetic is float32; stores round to nearest even.
+struct HalfIO {
+  static __device__ __forceinline__ float load(uint16_t h) {
+    _Float16 v;
+    __builtin_memcpy(&v, &h, 2);
+    return (float)v;
+  }
+  static __device__ __forceinline__ uint16_t store(float f) {
+    const _Float16 v = (_Float16)f;  // round to nearest even
+    uint16_t h;
+    __builtin_memcpy(&h, &v, 2);
+    return h;
+  }
+};
+struct Bf16IO {
+  static __device__ __forceinline__ float load(uint16_t h) {
+    return __uint_as_float((unsigned)h << 16);
+  }
+  static __device__ __forceinline__ uint16_t store(float f) {
+    const unsigned u = __float_as_uint(f);
+    if (f != f) return (uint16_t)((u >> 16) | 0x0040u);        // stays a NaN
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);  // round to nearest even
+  }
+};
+
+// A 2-byte element as a value type, for templates written over the element type: converts
+// to and from float, the arithmetic happens in AccOf<...>::type.
+template <typename IO>
+struct Narrow {
+  uint16_t bits;
+  Narrow() = default;
+  __device__ __forceinline__ Narrow(float f) : bits(IO::store(f)) {}
+  __device__ __forceinline__ operator float() const { return IO::load(bits); }
+};
+using f16_t = Narrow<HalfIO>;
+using bf16_t = Narrow<Bf16IO>;
+template <typename R>
+struct AccOf {
+  typedef R type;
+};
+template <typename IO>
+struct AccOf<Narrow<IO>> {
+  typedef float type;
+};
+
 // log(exp(a) + exp(b)) with the reference's handling of non-finite operands
 // (fast_rnnt/csrc/mutual_information.h:36-65): the larger operand is returned
 // untouched when the difference is not a finite number.

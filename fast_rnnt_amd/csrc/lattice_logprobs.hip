@@ -478,6 +478,344 @@ bool launch_row_grad_regs<float>(const float *logits, const int64_t *symbols, co
   return true;
 }
 
+// ---- 2-byte logits (float16 / bfloat16) ----------------------------------------------
+// The reference's recursion has no half-precision form (mutual_information_cuda.cu:37-38
+// notes the missing half LogAdd), so half or bfloat16 logits there need a float32 copy
+// first.  Here they are read as they are -- half the bytes of the dominant stream -- and
+// everything after the load is float32: the normalizer, the picked log-probs, px / py, the
+// recursion and its gradients.  Only logits.grad goes back out in the 2-byte type.
+// the eight values of a 16-byte piece
+template <typename IO>
+__device__ __forceinline__ void unpack8(intx4 raw, float (&out)[8]) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    out[2 * k] = IO::load((uint16_t)((unsigned)raw[k] & 0xffffu));
+    out[2 * k + 1] = IO::load((uint16_t)((unsigned)raw[k] >> 16));
+  }
+}
+// entry c of a row held as 8-value pieces (c wave-uniform and inside the row)
+template <int kVecs>
+__device__ __forceinline__ float row_entry8(const float (&v)[kVecs][8], int c) {
+  const int piece = c >> 3, e = c & 7, vec = piece / kWave, owner = piece % kWave;
+  float cand = v[0][0];
+#pragma unroll
+  for (int i = 0; i < kVecs; ++i)
+#pragma unroll
+    for (int k = 0; k < 8; ++k) cand = (i == vec && k == e) ? v[i][k] : cand;
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(cand), owner));
+}
+
+// One wave per row, the row in registers as float32 (C a multiple of 8, at most
+// 512 * kVecs entries): the 2-byte counterpart of row_norm_regs_kernel.
+template <typename IO, int kVecs, bool kStream>
+__global__ void __launch_bounds__(256)
+    row_norm_narrow_kernel(const uint16_t *__restrict__ logits, const int64_t *__restrict__ symbols,
+                           const int64_t *__restrict__ ranges, const int64_t *__restrict__ window,
+                           float *__restrict__ norm, float *__restrict__ xr, float *__restrict__ yr,
+                           long rows, int T, int Rr, int S, int C, int term) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const long row = (long)blockIdx.x * 4 + wave;
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  if (live_rows<1>(row, rows, ranges, window, T, Rr) == 0) return;
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t *>(logits + row * C), 0, C * 2, 0x00020000);
+  constexpr int kAux = kStream ? 2 : 0;
+  intx4 raw[kVecs];
+#pragma unroll
+  for (int i = 0; i < kVecs; ++i) {
+    const int c = 8 * (lane + kWave * i);
+    raw[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, c < C ? c * 2 : kOutOfRange, 0, kAux);
+  }
+  const float ninf = -__builtin_huge_valf();
+  float v[kVecs][8];
+#pragma unroll
+  for (int i = 0; i < kVecs; ++i) {
+    unpack8<IO>(raw[i], v[i]);
+    if (8 * (lane + kWave * i) >= C) {  // what lies past the end of the row takes no part
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[i][e] = ninf;
+    }
+  }
+  const int j = (int)(row % Rr);
+  const int b = (int)(row / ((long)Rr * T));
+  const int64_t sym = row_symbol(symbols, ranges, row, b, j, S, term);
+  float m = ninf;
+#pragma unroll
+  for (int i = 0; i < kVecs; ++i)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) m = (v[i][e] > m || v[i][e] != v[i][e]) ? v[i][e] : m;
+  m = wave_max_all(m);
+  const float shift = (m - m == 0) ? m : 0.f;  // torch.logsumexp: infinite max -> shift by 0
+  float sum = 0;
+#pragma unroll
+  for (int i = 0; i < kVecs; ++i)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sum += __expf(v[i][e] - shift);
+  sum = wave_sum_all(sum);
+  const float lse = logf(sum) + shift;
+  const float at_sym = (sym >= 0 && sym < C) ? row_entry8<kVecs>(v, (int)sym) - lse
+                                             : std::numeric_limits<float>::quiet_NaN();
+  const float at_term = row_entry8<kVecs>(v, term) - lse;
+  if (lane == 0) {
+    norm[row] = lse;
+    xr[row] = at_sym;
+    yr[row] = at_term;
+  }
+}
+
+// any row length: lanes stride over the row, two passes (the second hits the cache)
+template <typename IO>
+__global__ void __launch_bounds__(256)
+    row_norm_narrow_any_kernel(const uint16_t *__restrict__ logits,
+                               const int64_t *__restrict__ symbols,
+                               const int64_t *__restrict__ ranges,
+                               const int64_t *__restrict__ window, float *__restrict__ norm,
+                               float *__restrict__ xr, float *__restrict__ yr, long rows, int T,
+                               int Rr, int S, int C, int term) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  if (live_rows<1>(row, rows, ranges, window, T, Rr) == 0) return;
+  const uint16_t *x = logits + row * C;
+  float m = -__builtin_huge_valf();
+  for (int c = lane; c < C; c += kWave) {
+    const float v = IO::load(x[c]);
+    m = (v > m || v != v) ? v : m;
+  }
+  m = wave_max_all(m);
+  const float shift = (m - m == 0) ? m : 0.f;
+  float sum = 0;
+  for (int c = lane; c < C; c += kWave) sum += __expf(IO::load(x[c]) - shift);
+  sum = wave_sum_all(sum);
+  const float lse = logf(sum) + shift;
+  if (lane == 0) {
+    const int j = (int)(row % Rr);
+    const int b = (int)(row / ((long)Rr * T));
+    const int64_t sym = row_symbol(symbols, ranges, row, b, j, S, term);
+    norm[row] = lse;
+    xr[row] = (sym >= 0 && sym < C) ? IO::load(x[sym]) - lse
+                                    : std::numeric_limits<float>::quiet_NaN();
+    yr[row] = IO::load(x[term]) - lse;
+  }
+}
+
+// What the gradient of a logits row needs besides the row (all wave-uniform): the px / py
+// gradients of the lattice cell the row was placed at, its symbol and its normalizer.
+struct RowScalars {
+  float gx, gy, lse;
+  int sym;
+};
+__device__ __forceinline__ RowScalars row_scalars(long row, const int64_t *symbols,
+                                                  const int64_t *ranges, const int64_t *boundary,
+                                                  const float *norm, const float *gpx,
+                                                  const float *gpy, int S, int T, int Rr, int term,
+                                                  int rnnt_type) {
+  const int S1 = S + 1;
+  const int T1 = rnnt_type == kRegular ? T + 1 : T;
+  const int j = (int)(row % Rr);
+  const long frame = row / Rr;
+  const int t = (int)(frame % T), b = (int)(frame / T);
+  const int64_t r0 = ranges ? ranges[frame * Rr] : 0;
+  int64_t s64 = ((int64_t)j + r0) % S1;
+  if (s64 < 0) s64 += S1;
+  const int s = (int)s64;
+  const bool masked = rnnt_type == kRegular && boundary && boundary[4 * b + 3] == t;
+  auto gx_at = [&](int ss) -> float {
+    if (ss < 0 || ss >= S || masked) return 0.f;
+    return gpx[((long)b * S + ss) * T1 + t];
+  };
+  RowScalars r;
+  r.gx = gx_at(s);
+  r.gy = gpy[((long)b * S1 + s) * T + t];
+  if (rnnt_type == kConstrained) r.gy += gx_at(s - 1);
+  r.sym = (int)row_symbol(symbols, ranges, row, b, j, S, term);
+  r.lse = norm[row];
+  return r;
+}
+
+template <typename IO, int kVecs, bool kStream>
+__global__ void __launch_bounds__(256)
+    row_grad_narrow_kernel(const uint16_t *__restrict__ logits, const int64_t *__restrict__ symbols,
+                           const int64_t *__restrict__ ranges, const int64_t *__restrict__ boundary,
+                           const int64_t *__restrict__ window, const float *__restrict__ norm,
+                           const float *__restrict__ gpx, const float *__restrict__ gpy,
+                           uint16_t *__restrict__ glogits, long rows, int S, int T, int Rr, int C,
+                           int term, int rnnt_type) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const long row = (long)blockIdx.x * 4 + wave;
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const bool live = live_rows<1>(row, rows, ranges, window, T, Rr) != 0;  // wave-uniform
+  const __amdgpu_buffer_rsrc_t in_rs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t *>(logits + row * C), 0, C * 2, 0x00020000);
+  const __amdgpu_buffer_rsrc_t out_rs =
+      __builtin_amdgcn_make_buffer_rsrc(glogits + row * C, 0, C * 2, 0x00020000);
+  constexpr int kAux = kStream ? 2 : 0;
+  intx4 raw[kVecs];
+#pragma unroll
+  for (int i = 0; i < kVecs; ++i) {
+    const int c = 8 * (lane + kWave * i);
+    raw[i] = __builtin_amdgcn_raw_buffer_load_b128(in_rs, (live && c < C) ? c * 2 : kOutOfRange, 0,
+                                                   kAux);
+  }
+  RowScalars k{0.f, 0.f, 0.f, -1};
+  if (live)
+    k = row_scalars(row, symbols, ranges, boundary, norm, gpx, gpy, S, T, Rr, term, rnnt_type);
+  const float w = -(k.gx + k.gy);
+#pragma unroll
+  for (int i = 0; i < kVecs; ++i) {
+    const int c = 8 * (lane + kWave * i);
+    float v[8];
+    unpack8<IO>(raw[i], v);
+    intx4 o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      unsigned packed = 0;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int e = 2 * q + h;
+        float g = __expf(v[e] - k.lse) * w;
+        if (c + e == k.sym) g += k.gx;
+        if (c + e == term) g += k.gy;
+        // a row outside the window is not read and gets exact zeros
+        packed |= (unsigned)(live ? IO::store(g) : (uint16_t)0) << (16 * h);
+      }
+      o[q] = (int)packed;
+    }
+    __builtin_amdgcn_raw_buffer_store_b128(o, out_rs, c < C ? c * 2 : kOutOfRange, 0, kAux);
+  }
+}
+
+template <typename IO>
+__global__ void __launch_bounds__(256)
+    row_grad_narrow_any_kernel(const uint16_t *__restrict__ logits,
+                               const int64_t *__restrict__ symbols,
+                               const int64_t *__restrict__ ranges,
+                               const int64_t *__restrict__ boundary,
+                               const int64_t *__restrict__ window, const float *__restrict__ norm,
+                               const float *__restrict__ gpx, const float *__restrict__ gpy,
+                               uint16_t *__restrict__ glogits, long rows, int S, int T, int Rr,
+                               int C, int term, int rnnt_type) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  uint16_t *g = glogits + row * C;
+  if (live_rows<1>(row, rows, ranges, window, T, Rr) == 0) {
+    for (int c = lane; c < C; c += kWave) g[c] = 0;
+    return;
+  }
+  const RowScalars k =
+      row_scalars(row, symbols, ranges, boundary, norm, gpx, gpy, S, T, Rr, term, rnnt_type);
+  const float w = -(k.gx + k.gy);
+  const uint16_t *x = logits + row * C;
+  for (int c = lane; c < C; c += kWave) {
+    float v = __expf(IO::load(x[c]) - k.lse) * w;
+    if (c == k.sym) v += k.gx;
+    if (c == term) v += k.gy;
+    g[c] = IO::store(v);
+  }
+}
+
+template <typename IO>
+int narrow_fwd_impl(const void *logits_, const int64_t *symbols, const int64_t *ranges,
+                    const int64_t *boundary, float *px, float *py, float *norm, float *xr,
+                    float *yr, int B, int S, int T, int Rr, int C, int term, int rnnt_type,
+                    int window_only, void *stream_) {
+  if (B < 0 || S < 0 || T < 0 || Rr < 1 || C < 1)
+    return fail(FRNNT_EINVAL, "lattice_logprobs_fwd: bad size");
+  if (Rr > S + 1) return fail(FRNNT_EINVAL, "lattice_logprobs_fwd: more range rows than S + 1");
+  if (!ranges && Rr != S + 1)
+    return fail(FRNNT_EINVAL, "lattice_logprobs_fwd: without ranges the logits need S + 1 rows");
+  if (rnnt_type < 0 || rnnt_type > 2 || term < 0 || term >= C)
+    return fail(FRNNT_EINVAL, "lattice_logprobs_fwd: bad rnnt_type or termination symbol");
+  if (B == 0) return FRNNT_OK;
+  if (!logits_ || (!symbols && S > 0) || !px || !py || !norm || !xr || !yr)
+    return fail(FRNNT_EINVAL, "lattice_logprobs_fwd: null pointer");
+  const uint16_t *logits = static_cast<const uint16_t *>(logits_);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  const long rows = (long)B * T * Rr;
+  const int64_t *window = window_only ? boundary : nullptr;
+  const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+  const bool big = rows * C * 2 > kStreamBytes;
+#define FRNNT_NARROW_NORM(V)                                                                     \
+  do {                                                                                           \
+    if (big)                                                                                     \
+      hipLaunchKernelGGL((row_norm_narrow_kernel<IO, V, true>), grid, block, 0, stream, logits,  \
+                         symbols, ranges, window, norm, xr, yr, rows, T, Rr, S, C, term);        \
+    else                                                                                         \
+      hipLaunchKernelGGL((row_norm_narrow_kernel<IO, V, false>), grid, block, 0, stream, logits, \
+                         symbols, ranges, window, norm, xr, yr, rows, T, Rr, S, C, term);        \
+  } while (0)
+  if (rows > 0) {
+    if (C % 8 != 0 || C > 512 * 8 || (reinterpret_cast<uintptr_t>(logits) & 15))
+      hipLaunchKernelGGL(row_norm_narrow_any_kernel<IO>, grid, block, 0, stream, logits, symbols,
+                         ranges, window, norm, xr, yr, rows, T, Rr, S, C, term);
+    else if (C <= 512)
+      FRNNT_NARROW_NORM(1);
+    else if (C <= 1024)
+      FRNNT_NARROW_NORM(2);
+    else if (C <= 2048)
+      FRNNT_NARROW_NORM(4);
+    else
+      FRNNT_NARROW_NORM(8);
+  }
+#undef FRNNT_NARROW_NORM
+  const int T1 = rnnt_type == kRegular ? T + 1 : T;
+  const long total = (long)B * S * T1 + (long)B * (S + 1) * T;
+  if (total > 0)
+    hipLaunchKernelGGL(assemble_kernel<float>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                       stream, xr, yr, ranges, boundary, px, py, B, S, T, Rr, rnnt_type);
+  return check_launch("lattice_logprobs_fwd");
+}
+
+template <typename IO>
+int narrow_bwd_impl(const void *logits_, const int64_t *symbols, const int64_t *ranges,
+                    const int64_t *boundary, const float *norm, const float *px_grad,
+                    const float *py_grad, void *logits_grad_, int B, int S, int T, int Rr, int C,
+                    int term, int rnnt_type, int window_only, void *stream_) {
+  if (B < 0 || S < 0 || T < 0 || Rr < 1 || C < 1 || Rr > S + 1 || (!ranges && Rr != S + 1))
+    return fail(FRNNT_EINVAL, "lattice_logprobs_bwd: bad size");
+  if (rnnt_type < 0 || rnnt_type > 2 || term < 0 || term >= C)
+    return fail(FRNNT_EINVAL, "lattice_logprobs_bwd: bad rnnt_type or termination symbol");
+  if (B == 0 || T == 0) return FRNNT_OK;
+  if (!logits_ || (!symbols && S > 0) || !norm || !px_grad || !py_grad || !logits_grad_)
+    return fail(FRNNT_EINVAL, "lattice_logprobs_bwd: null pointer");
+  const uint16_t *logits = static_cast<const uint16_t *>(logits_);
+  uint16_t *glogits = static_cast<uint16_t *>(logits_grad_);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  const long rows = (long)B * T * Rr;
+  const int64_t *window = window_only ? boundary : nullptr;
+  const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+  const bool big = rows * C * 2 > kStreamBytes;
+#define FRNNT_NARROW_GRAD(V)                                                                      \
+  do {                                                                                            \
+    if (big)                                                                                      \
+      hipLaunchKernelGGL((row_grad_narrow_kernel<IO, V, true>), grid, block, 0, stream, logits,   \
+                         symbols, ranges, boundary, window, norm, px_grad, py_grad, glogits,      \
+                         rows, S, T, Rr, C, term, rnnt_type);                                     \
+    else                                                                                          \
+      hipLaunchKernelGGL((row_grad_narrow_kernel<IO, V, false>), grid, block, 0, stream, logits,  \
+                         symbols, ranges, boundary, window, norm, px_grad, py_grad, glogits,      \
+                         rows, S, T, Rr, C, term, rnnt_type);                                     \
+  } while (0)
+  if (C % 8 != 0 || C > 512 * 8 ||
+      ((reinterpret_cast<uintptr_t>(logits) | reinterpret_cast<uintptr_t>(glogits)) & 15))
+    hipLaunchKernelGGL(row_grad_narrow_any_kernel<IO>, grid, block, 0, stream, logits, symbols,
+                       ranges, boundary, window, norm, px_grad, py_grad, glogits, rows, S, T, Rr,
+                       C, term, rnnt_type);
+  else if (C <= 512)
+    FRNNT_NARROW_GRAD(1);
+  else if (C <= 1024)
+    FRNNT_NARROW_GRAD(2);
+  else if (C <= 2048)
+    FRNNT_NARROW_GRAD(4);
+  else
+    FRNNT_NARROW_GRAD(8);
+#undef FRNNT_NARROW_GRAD
+  return check_launch("lattice_logprobs_bwd");
+}
+
 template <typename R>
 int fwd_impl(const R *logits, const int64_t *symbols, const int64_t *ranges,
              const int64_t *boundary, R *px, R *py, R *norm, R *xr, R *yr, int B, int S, int T,
@@ -573,5 +911,28 @@ int frnnt_lattice_logprobs_bwd_f64(const double *logits, const int64_t *symbols,
                                  logits_grad, B, S, T, R, C, termination_symbol, rnnt_type,
                                  window_only, stream);
 }
+
+
+#define FRNNT_NARROW_ENTRY(sfx, IO)                                                              \
+  int frnnt_lattice_logprobs_fwd_##sfx(                                                          \
+      const void *logits, const int64_t *symbols, const int64_t *ranges, const int64_t *boundary, \
+      float *px, float *py, float *norm, float *xr, float *yr, int B, int S, int T, int R, int C, \
+      int termination_symbol, int rnnt_type, int window_only, void *stream) {                    \
+    return frnnt::narrow_fwd_impl<frnnt::IO>(logits, symbols, ranges, boundary, px, py, norm, xr, \
+                                             yr, B, S, T, R, C, termination_symbol, rnnt_type,    \
+                                             window_only, stream);                                \
+  }                                                                                              \
+  int frnnt_lattice_logprobs_bwd_##sfx(                                                          \
+      const void *logits, const int64_t *symbols, const int64_t *ranges, const int64_t *boundary, \
+      const float *norm, const float *px_grad, const float *py_grad, void *logits_grad, int B,    \
+      int S, int T, int R, int C, int termination_symbol, int rnnt_type, int window_only,         \
+      void *stream) {                                                                            \
+    return frnnt::narrow_bwd_impl<frnnt::IO>(logits, symbols, ranges, boundary, norm, px_grad,    \
+                                             py_grad, logits_grad, B, S, T, R, C,                 \
+                                             termination_symbol, rnnt_type, window_only, stream); \
+  }
+FRNNT_NARROW_ENTRY(f16, HalfIO)
+FRNNT_NARROW_ENTRY(bf16, Bf16IO)
+#undef FRNNT_NARROW_ENTRY
 
 }  // extern "C"

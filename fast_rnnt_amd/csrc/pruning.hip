@@ -192,7 +192,8 @@ __global__ void __launch_bounds__(256)
   int64_t s = ranges[row];
   R *dst = out + row * C;
   if (s < 0 || s >= S1) {
-    for (int c = lane; c < C; c += kWave) dst[c] = std::numeric_limits<R>::quiet_NaN();
+    typedef typename AccOf<R>::type A;
+    for (int c = lane; c < C; c += kWave) dst[c] = (R)std::numeric_limits<A>::quiet_NaN();
     return;
   }
   const R *src = lm + (b * S1 + s) * C;
@@ -206,7 +207,8 @@ typedef int words4 __attribute__((ext_vector_type(4), aligned(4)));
 template <int kVecs>
 __global__ void __launch_bounds__(256)
     prune_gather_vec_kernel(const int *__restrict__ lm, const int64_t *__restrict__ ranges,
-                            int *__restrict__ out, long rows, int TR, int S1, int C) {
+                            int *__restrict__ out, long rows, int TR, int S1, int C,
+                            int nan_bits) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // in a scalar register
   const long row = (long)blockIdx.x * 4 + wave;
   const int lane = threadIdx.x & 63;
@@ -215,7 +217,6 @@ __global__ void __launch_bounds__(256)
   const int64_t s = ranges[row];
   const bool valid = s >= 0 && s < S1;
   const int *src = lm + (b * S1 + (valid ? s : 0)) * C;
-  const int nan_bits = 0x7fc00000;
   words4 v[kVecs];
 #pragma unroll
   for (int i = 0; i < kVecs; ++i) {
@@ -361,24 +362,27 @@ __global__ void __launch_bounds__(256)
       for (int c0 = 0; c0 < C; c0 += 256) {
         const int c = c0 + tid;
         if (c >= C) continue;
-        R acc = first_round ? (R)0 : dst[c];
-        auto entry = [&](int i) -> R {
+        // (2-byte elements are summed in float32; a sum that takes several rounds --
+        // more than kHitCapacity rows -- is rounded to the element type between rounds)
+        typedef typename AccOf<R>::type A;
+        A acc = first_round ? (A)0 : (A)dst[c];
+        auto entry = [&](int i) -> A {
           const long at = (long)hits[i] * C + c;
-          const R g = gb[at];
+          const A g = (A)gb[at];
           if (!ob) return g;
-          const R y = ob[at];
-          return g * ((R)1 - y * y);
+          const A y = (A)ob[at];
+          return g * ((A)1 - y * y);
         };
         int i = 0;
         for (; i + 8 <= n; i += 8) {
-          R g[8];
+          A g[8];
 #pragma unroll
           for (int u = 0; u < 8; ++u) g[u] = entry(i + u);
 #pragma unroll
           for (int u = 0; u < 8; ++u) acc += g[u];
         }
         if (i + 4 <= n) {
-          R g[4];
+          A g[4];
 #pragma unroll
           for (int u = 0; u < 4; ++u) g[u] = entry(i + u);
 #pragma unroll
@@ -386,7 +390,7 @@ __global__ void __launch_bounds__(256)
           i += 4;
         }
         for (; i < n; ++i) acc += entry(i);
-        dst[c] = acc;
+        dst[c] = (R)acc;
       }
     }
     first_round = false;
@@ -423,28 +427,32 @@ int ranges_impl(const R *px_grad, const R *py_grad, const int64_t *boundary, int
   return check_launch("prune_ranges");
 }
 
+// nan_words: a quiet NaN of the element type as a 4-byte word (twice, for 2-byte elements)
 template <typename R>
 int gather_impl(const R *lm, const int64_t *ranges, R *out, int B, int S, int T, int Rr, int C,
-                void *stream) {
+                int nan_words, void *stream) {
   if (B < 0 || S < 0 || T < 0 || Rr < 0 || C < 0)
     return fail(FRNNT_EINVAL, "prune_gather: negative size");
   const long rows = (long)B * T * Rr;
   if (rows == 0 || C == 0) return FRNNT_OK;
   if (!lm || !ranges || !out) return fail(FRNNT_EINVAL, "prune_gather: null pointer");
   const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
-  if (sizeof(R) == 4 && C % 4 == 0 && C <= 256 * 16) {
+  // rows as 4-byte words: the elements themselves, or 2-byte elements in pairs
+  const int W = sizeof(R) == 4 ? C : (sizeof(R) == 2 && C % 2 == 0 ? C / 2 : 0);
+  if (W > 0 && W % 4 == 0 && W <= 256 * 16 &&
+      ((reinterpret_cast<uintptr_t>(lm) | reinterpret_cast<uintptr_t>(out)) & 3) == 0) {
     const int *src = reinterpret_cast<const int *>(lm);
     int *dst = reinterpret_cast<int *>(out);
 #define FRNNT_GATHER(V)                                                                          \
   hipLaunchKernelGGL(prune_gather_vec_kernel<V>, grid, block, 0, static_cast<hipStream_t>(stream), \
-                     src, ranges, dst, rows, T * Rr, S + 1, C)
-    if (C <= 256)
+                     src, ranges, dst, rows, T * Rr, S + 1, W, nan_words)
+    if (W <= 256)
       FRNNT_GATHER(1);
-    else if (C <= 512)
+    else if (W <= 512)
       FRNNT_GATHER(2);
-    else if (C <= 1024)
+    else if (W <= 1024)
       FRNNT_GATHER(4);
-    else if (C <= 2048)
+    else if (W <= 2048)
       FRNNT_GATHER(8);
     else
       FRNNT_GATHER(16);
@@ -638,11 +646,11 @@ int frnnt_prune_ranges_f64(const double *px_grad, const double *py_grad, const i
 }
 int frnnt_prune_gather_f32(const float *lm, const int64_t *ranges, float *lm_pruned, int B, int S,
                            int T, int R, int C, void *stream) {
-  return frnnt::gather_impl<float>(lm, ranges, lm_pruned, B, S, T, R, C, stream);
+  return frnnt::gather_impl<float>(lm, ranges, lm_pruned, B, S, T, R, C, 0x7fc00000, stream);
 }
 int frnnt_prune_gather_f64(const double *lm, const int64_t *ranges, double *lm_pruned, int B, int S,
                            int T, int R, int C, void *stream) {
-  return frnnt::gather_impl<double>(lm, ranges, lm_pruned, B, S, T, R, C, stream);
+  return frnnt::gather_impl<double>(lm, ranges, lm_pruned, B, S, T, R, C, 0, stream);
 }
 int frnnt_prune_gather_bwd_f32(const float *grad, const int64_t *ranges, float *lm_grad, int B,
                                int S, int T, int R, int C, void *stream) {
@@ -651,6 +659,30 @@ int frnnt_prune_gather_bwd_f32(const float *grad, const int64_t *ranges, float *
 int frnnt_prune_gather_bwd_f64(const double *grad, const int64_t *ranges, double *lm_grad, int B,
                                int S, int T, int R, int C, void *stream) {
   return frnnt::scatter_impl<double>(grad, ranges, lm_grad, B, S, T, R, C, stream);
+}
+int frnnt_prune_gather_f16(const void *lm, const int64_t *ranges, void *lm_pruned, int B, int S,
+                           int T, int R, int C, void *stream) {
+  return frnnt::gather_impl<frnnt::f16_t>(static_cast<const frnnt::f16_t *>(lm), ranges,
+                                          static_cast<frnnt::f16_t *>(lm_pruned), B, S, T, R, C,
+                                          0x7e007e00, stream);
+}
+int frnnt_prune_gather_bf16(const void *lm, const int64_t *ranges, void *lm_pruned, int B, int S,
+                            int T, int R, int C, void *stream) {
+  return frnnt::gather_impl<frnnt::bf16_t>(static_cast<const frnnt::bf16_t *>(lm), ranges,
+                                           static_cast<frnnt::bf16_t *>(lm_pruned), B, S, T, R, C,
+                                           0x7fc07fc0, stream);
+}
+int frnnt_prune_gather_bwd_f16(const void *grad, const int64_t *ranges, void *lm_grad, int B, int S,
+                               int T, int R, int C, void *stream) {
+  return frnnt::scatter_impl<frnnt::f16_t>(static_cast<const frnnt::f16_t *>(grad), ranges,
+                                           static_cast<frnnt::f16_t *>(lm_grad), B, S, T, R, C,
+                                           stream);
+}
+int frnnt_prune_gather_bwd_bf16(const void *grad, const int64_t *ranges, void *lm_grad, int B,
+                                int S, int T, int R, int C, void *stream) {
+  return frnnt::scatter_impl<frnnt::bf16_t>(static_cast<const frnnt::bf16_t *>(grad), ranges,
+                                            static_cast<frnnt::bf16_t *>(lm_grad), B, S, T, R, C,
+                                            stream);
 }
 int frnnt_pruned_joiner_fwd_f32(const float *am, const float *lm, const int64_t *ranges, float *out,
                                 int B, int S, int T, int R, int C, int activation, void *stream) {

@@ -84,6 +84,22 @@ def _check_tensors(floats, indices) -> None:
     _require_gpu(*(t for _, t in floats + indices))
 
 
+_NARROW = (torch.float16, torch.bfloat16)
+
+
+def _lattice_dtype(dtype):
+    """Element type of px / py (and of the loss) for inputs of type `dtype`: the 2-byte
+    types are accumulated in float32 (the reference's recursion has no half form,
+    mutual_information_cuda.cu:37-38)."""
+    return torch.float32 if dtype in _NARROW else dtype
+
+
+def _widen(*tensors):
+    """float16 / bfloat16 inputs of the additive-joiner losses as float32 (differentiable:
+    the gradients come back in the inputs' type); other types pass through."""
+    return tuple(t.float() if t is not None and t.dtype in _NARROW else t for t in tensors)
+
+
 class _SimpleLogprobs(torch.autograd.Function):
     """(px, py) of the additive-joiner loss: frnnt_simple_logprobs_fwd/bwd."""
 
@@ -160,6 +176,7 @@ def get_rnnt_logprobs(
     validate_st_lengths(S, T, rnnt_type == "regular", boundary)
     assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
     _check_tensors([("am", am), ("lm", lm)], [("symbols", symbols), ("boundary", boundary)])
+    lm, am = _widen(lm, am)
     return _SimpleLogprobs.apply(lm, am, symbols, boundary, termination_symbol, rnnt_type)
 
 
@@ -348,6 +365,7 @@ def rnnt_loss_simple(
             assert 0 <= t_begin <= t_end <= T
     if reduction not in ("none", "mean", "sum"):
         raise ValueError(f"reduction should be ('none' | 'mean' | 'sum'), given {reduction}")
+    lm, am = _widen(lm, am)
     loss, px_grad, py_grad = _SimpleLoss.apply(
         lm, am, symbols, boundary, termination_symbol, rnnt_type, float(delay_penalty),
         bool(return_grad), _REDUCTIONS[reduction])
@@ -366,12 +384,14 @@ class _LatticeLogprobs(torch.autograd.Function):
         B, T, R, C = logits.shape
         S = symbols.shape[1]
         kind = _RNNT_TYPES[rnnt_type]
-        sfx = _lib.suffix(logits.dtype)
+        # float16 / bfloat16 logits are read as they are; px, py and everything after
+        # them are float32
+        sfx = _lib.suffix(logits.dtype, narrow=True)
         lg = logits.contiguous()
         sym_c = symbols.contiguous()
         rng_c = ranges.contiguous() if ranges is not None else None
         bnd_c = boundary.contiguous() if boundary is not None else None
-        opts = dict(dtype=logits.dtype, device=logits.device)
+        opts = dict(dtype=_lattice_dtype(logits.dtype), device=logits.device)
         T1 = T + 1 if kind == 0 else T
         windowed = bool(window_only) and bnd_c is not None
         with torch.cuda.device(logits.device):
@@ -393,7 +413,7 @@ class _LatticeLogprobs(torch.autograd.Function):
     def backward(ctx, gpx, gpy):
         lg, sym, rng, bnd, norm = ctx.saved_tensors
         B, S, T, R, C, term, kind, sfx, windowed = ctx.meta
-        opts = dict(dtype=lg.dtype, device=lg.device)
+        opts = dict(dtype=norm.dtype, device=lg.device)
         T1 = T + 1 if kind == 0 else T
         with torch.cuda.device(lg.device):
             gpx = torch.zeros(B, S, T1, **opts) if gpx is None else gpx.contiguous()
@@ -516,7 +536,7 @@ class _PruneGather(torch.autograd.Function):
     def forward(ctx, lm, ranges):
         B, S1, C = lm.shape
         _, T, R = ranges.shape
-        sfx = _lib.suffix(lm.dtype)
+        sfx = _lib.suffix(lm.dtype, narrow=True)
         lm_c, rng_c = lm.contiguous(), ranges.contiguous()
         with torch.cuda.device(lm.device):
             out = torch.empty(B, T, R, C, dtype=lm.dtype, device=lm.device)
@@ -754,6 +774,7 @@ def get_rnnt_logprobs_smoothed(
     assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
     _check_tensors([("am", am), ("lm", lm)], [("symbols", symbols), ("boundary", boundary)])
 
+    lm, am = _widen(lm, am)
     # joint part, without the boundary / constrained post-processing (applied last)
     base_type = "regular" if rnnt_type == "regular" else "modified"
     px, py = _SimpleLogprobs.apply(lm, am, symbols, None, termination_symbol, base_type)

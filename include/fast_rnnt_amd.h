@@ -324,6 +324,39 @@ int frnnt_lattice_logprobs_bwd_f64(const double *logits, const int64_t *symbols,
                                    int window_only, void *stream);
 
 /*
+ * The two entry points above for 2-byte logits: float16 (_f16) or bfloat16 (_bf16),
+ * passed as void*.  The reference has no such form -- its recursion knows float32 and
+ * float64 only (mutual_information_cuda.cu:37-38 notes the missing half LogAdd), so
+ * half-precision joiner outputs need a float32 copy there.  Here the logits are read as
+ * they are (half the bytes of the dominant stream) and everything after the load is
+ * float32: norm, xr, yr, px, py and the incoming px_grad / py_grad are float32 buffers of
+ * the shapes above, to be used with frnnt_mi_forward_f32 / frnnt_mi_backward_f32; only
+ * logits_grad is written in the logits' type (rounded to nearest even).
+ */
+int frnnt_lattice_logprobs_fwd_f16(const void *logits, const int64_t *symbols,
+                                   const int64_t *ranges, const int64_t *boundary, float *px,
+                                   float *py, float *norm, float *xr, float *yr, int B, int S,
+                                   int T, int R, int C, int termination_symbol, int rnnt_type,
+                                   int window_only, void *stream);
+int frnnt_lattice_logprobs_fwd_bf16(const void *logits, const int64_t *symbols,
+                                    const int64_t *ranges, const int64_t *boundary, float *px,
+                                    float *py, float *norm, float *xr, float *yr, int B, int S,
+                                    int T, int R, int C, int termination_symbol, int rnnt_type,
+                                    int window_only, void *stream);
+int frnnt_lattice_logprobs_bwd_f16(const void *logits, const int64_t *symbols,
+                                   const int64_t *ranges, const int64_t *boundary,
+                                   const float *norm, const float *px_grad, const float *py_grad,
+                                   void *logits_grad, int B, int S, int T, int R, int C,
+                                   int termination_symbol, int rnnt_type, int window_only,
+                                   void *stream);
+int frnnt_lattice_logprobs_bwd_bf16(const void *logits, const int64_t *symbols,
+                                    const int64_t *ranges, const int64_t *boundary,
+                                    const float *norm, const float *px_grad, const float *py_grad,
+                                    void *logits_grad, int B, int S, int T, int R, int C,
+                                    int termination_symbol, int rnnt_type, int window_only,
+                                    void *stream);
+
+/*
  * Pruning bounds.  Replaces the device work of get_rnnt_prune_ranges
  * (rnnt_loss.py:726-777 with _adjust_pruning_lower_bound :584-632).  s_range is
  * the FINAL window size: the caller has already raised it to the regular
@@ -354,6 +387,21 @@ int frnnt_prune_gather_bwd_f32(const float *grad, const int64_t *ranges, float *
                                int S, int T, int R, int C, void *stream);
 int frnnt_prune_gather_bwd_f64(const double *grad, const int64_t *ranges, double *lm_grad, int B,
                                int S, int T, int R, int C, void *stream);
+
+/*
+ * The same for float16 (_f16) / bfloat16 (_bf16) elements, passed as void*: the reference's
+ * do_rnnt_pruning is plain indexing and takes any element type, as half-precision encoder /
+ * predictor outputs under autocast need.  The gather copies bit patterns; the adjoint sums in
+ * float32 and rounds the result to the element type (to nearest even).
+ */
+int frnnt_prune_gather_f16(const void *lm, const int64_t *ranges, void *lm_pruned, int B, int S,
+                           int T, int R, int C, void *stream);
+int frnnt_prune_gather_bf16(const void *lm, const int64_t *ranges, void *lm_pruned, int B, int S,
+                            int T, int R, int C, void *stream);
+int frnnt_prune_gather_bwd_f16(const void *grad, const int64_t *ranges, void *lm_grad, int B, int S,
+                               int T, int R, int C, void *stream);
+int frnnt_prune_gather_bwd_bf16(const void *grad, const int64_t *ranges, void *lm_grad, int B,
+                                int S, int T, int R, int C, void *stream);
 
 /*
  * The joiner's input straight from the pruning bounds:
