@@ -254,6 +254,18 @@ def _recursion_bytes(boundary, S, T, B, backward):
     return 4 * win + 4 * (B * S * (T + 1) + B * (S + 1) * T) + 4 * B + 32 * B
 
 
+def _copy_probe(args, dev):
+    """Device-to-device copies of a known size: the reference against which a hardware-counter
+    run of this script calibrates FETCH_SIZE / WRITE_SIZE."""
+    if args.copy_probe_mib <= 0:
+        return
+    src = torch.empty(args.copy_probe_mib << 20, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    for _ in range(5):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+
+
 def _emit(out):
     print(json.dumps(out))
 
@@ -268,6 +280,7 @@ def _bench_lattice(args, w, dev):
     from oracle import losses as O
 
     table, traffic_file = _measured_traffic(w.name)
+    _copy_probe(args, dev)
     sym, bnd = w.symbols.to(dev), w.boundary.to(dev)
     extra = {}
     ldt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[args.logits_dtype]
@@ -475,12 +488,7 @@ def main():
     sym = w.symbols.to(dev)
     bnd = w.boundary.to(dev)
 
-    if args.copy_probe_mib > 0:
-        src = torch.empty(args.copy_probe_mib << 20, dtype=torch.uint8, device=dev).fill_(1)
-        dst = torch.empty_like(src)
-        for _ in range(5):
-            dst.copy_(src)
-        torch.cuda.synchronize()
+    _copy_probe(args, dev)
 
     def step(boundary=bnd):
         am.grad = None
