@@ -402,6 +402,15 @@ __device__ __forceinline__ dgemm::floatx4 load4_guarded(const float *base, int o
 // exp(x - m) as one fused multiply-add and one v_exp_f32: 2^(x log2(e) - m log2(e)),
 // with shift2 = -m log2(e) prepared per row; x = -inf gives 0.
 constexpr float kLog2e = 1.44269504088896341f;
+// The largest of three, as the one instruction it is.  fmaxf() costs a canonicalising
+// v_max_f32 per operand on top (the compiler quiets signalling NaNs first), which tripled the
+// instruction count of the row maxima in the GEMM loops; v_max3_f32 itself ignores quiet NaNs
+// like fmaxf and quiets signalling ones.
+__device__ __forceinline__ float max3_raw(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
 __device__ __forceinline__ float exp_shifted(float x, float shift2) {
   return __builtin_amdgcn_exp2f(__builtin_fmaf(x, kLog2e, shift2));
 }
@@ -523,10 +532,11 @@ __global__ void __launch_bounds__(kPanThreads)
   auto fetch = [&](floatx4 (&into)[kLoads], int k0) {
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
+      // (the wave-uniform part of the offset rides in a scalar register)
       const intx4 raw = j < kLmLoads
-                            ? __builtin_amdgcn_raw_buffer_load_b128(lm_rs, lm_off + (j * step + k0 * 4), 0, 0)
+                            ? __builtin_amdgcn_raw_buffer_load_b128(lm_rs, lm_off, j * step + k0 * 4, 0)
                             : __builtin_amdgcn_raw_buffer_load_b128(
-                                  am_rs, am_off + ((j - kLmLoads) * step + k0 * 4), 0, 0);
+                                  am_rs, am_off, (j - kLmLoads) * step + k0 * 4, 0);
       into[j] = floatx4{__int_as_float(raw[0]), __int_as_float(raw[1]), __int_as_float(raw[2]),
                         __int_as_float(raw[3])};
     }
@@ -623,7 +633,7 @@ __global__ void __launch_bounds__(kPanThreads)
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
       // two three-input maxima; a row is above its margin exactly when its maximum is
-      seen[j] = fmaxf(fmaxf(fmaxf(slab[j][0], slab[j][1]), slab[j][2]), fmaxf(slab[j][3], seen[j]));
+      seen[j] = max3_raw(max3_raw(slab[j][0], slab[j][1], slab[j][2]), slab[j][3], seen[j]);
       above |= __builtin_fmaf(seen[j], kLog2e, shift2[j]) > kMargin * kLog2e;
     }
     if (__any(above)) raise_shifts();
@@ -834,7 +844,7 @@ __device__ __forceinline__ void simple_bwd_lm_slab_body(
 #pragma unroll
     for (int j = 0; j < kLoadsA; ++j)
       sa[j] = as_floats(__builtin_amdgcn_raw_buffer_load_b128(
-          d_rs, d_off + (kRowsA * j * ldd + k0) * 4, 0, 0));
+          d_rs, d_off, (kRowsA * j * ldd + k0) * 4, 0));  // (uniform part: scalar register)
     if (k0 + kLmK > t_lim) {  // (wave-uniform) the slab that holds the last frame
 #pragma unroll
       for (int j = 0; j < kLoadsA; ++j)
@@ -846,7 +856,7 @@ __device__ __forceinline__ void simple_bwd_lm_slab_body(
     for (int j = 0; j < kLoadsB; ++j) {
       const int tr = k0 + sub + 8 * j;
       sb[j] = as_floats(__builtin_amdgcn_raw_buffer_load_b128(
-          am_rs, am_off + (k0 + 8 * j) * C * 4, 0, 0));
+          am_rs, am_off, (k0 + 8 * j) * C * 4, 0));
       shift2[j] = tr < t_lim ? -amx[tr] * kLog2e : 0.f;
       // a frame past the last one meets D = 0; its factor only has to be finite
       if (tr >= t_lim) sb[j] = floatx4{0.f, 0.f, 0.f, 0.f};
