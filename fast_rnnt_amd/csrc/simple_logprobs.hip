@@ -982,17 +982,25 @@ __device__ __forceinline__ void simple_bwd_lm_slab_body(
 // requested before the dense product so that they arrive under it.
 constexpr int kAmT = 64;       // frames per workgroup
 constexpr int kAmC = 64;       // vocabulary entries per workgroup
-constexpr int kAmRows = 128;   // lattice rows per LDS pass (even)
 constexpr int kAmHotAhead = 8; // per-symbol pairs whose gx values are requested ahead
 constexpr int kAmOutPitch = 68;  // row pitch of the result tiles staged in LDS
 constexpr int kAmQ = kAmT / 4;   // 16-byte pieces per panel row (kAmT == kAmC)
 
+constexpr int kAmCap = 64;     // most lattice rows per pass
+// rows of k per pass: passes of equal (even) size, none above kAmCap
+int am_rows_per_pass(int S) {
+  const int passes = (S + 1 + kAmCap - 1) / kAmCap;
+  return std::min(kAmCap, ((S + 1 + passes - 1) / passes + 1) & ~1);
+}
 size_t am_panel_lds_bytes(int rows_cap) {
   const size_t panels = (size_t)rows_cap * (kAmT + kAmC) * sizeof(float);
   const size_t staging = (size_t)2 * kAmT * kAmOutPitch * sizeof(float);
   return std::max(panels, staging) + (size_t)(2 * rows_cap + 2 * kAmT) * sizeof(float);
 }
 
+// kCap: most lattice rows a pass may hold (the launch's rows_cap is at most that); it sets
+// how many panel pieces a thread keeps in registers.
+template <int kCap>
 __device__ __forceinline__ void simple_bwd_am_panel_body(
     int block_id, const float *__restrict__ lm, const float *__restrict__ am,
     const int64_t *__restrict__ symbols, const int64_t *__restrict__ boundary,
@@ -1083,17 +1091,24 @@ __device__ __forceinline__ void simple_bwd_am_panel_body(
   floatx16 acc, hot;
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = hot[v] = 0.f;
-  for (int k0 = 0; k0 < k_lim; k0 += rows_cap) {
-    const int rows = min(rows_cap, k_lim - k0);
-    const int pairs = (rows + 1) / 2;
-    constexpr int kSteps = kAmRows / 16;
-    floatx4 ra[kSteps], rb[kSteps];
+  constexpr int kSteps = kCap / 16;
+  constexpr int kNowhere = (int)0x80000000;  // an offset outside every resource: reads 0, moves nothing
+  floatx4 ra[kSteps], rb[kSteps];
+  // a pass's pieces of the two panels: rows k0 + q_row + 16 j of D and of lm, while they
+  // belong to the pass
+  auto request = [&](int k0) {
+    const int end = min(k0 + rows_cap, k_lim);
 #pragma unroll
     for (int j = 0; j < kSteps; ++j) {
       const int k = k0 + q_row + 16 * j;
-      ra[j] = get4(d_rs, (k * ldd + t_tile + q_col) * 4);
-      rb[j] = get4(lm_rs, (k * C + c_tile + q_col) * 4);
+      ra[j] = get4(d_rs, k < end ? (k * ldd + t_tile + q_col) * 4 : kNowhere);
+      rb[j] = get4(lm_rs, k < end ? (k * C + c_tile + q_col) * 4 : kNowhere);
     }
+  };
+  request(0);
+  for (int k0 = 0; k0 < k_lim; k0 += rows_cap) {
+    const int rows = min(rows_cap, k_lim - k0);
+    const int pairs = (rows + 1) / 2;
     if (k0 > 0) __syncthreads();  // the previous pass's readers are done with the panels
     for (int k = tid; k < 2 * pairs; k += 256) {
       sym_s[k] = (k0 + k < S) ? sym_lo[2 * (k0 + k)] : -1;
@@ -1141,6 +1156,8 @@ __device__ __forceinline__ void simple_bwd_am_panel_body(
       for (int i = 0; i < 4; ++i) e[i] = (k < rows && c + i < C) ? __expf(rb[j][i] - mx) : 0.f;
       *reinterpret_cast<floatx4 *>(Bs + k * kAmC + q_col) = e;
     }
+    // the next pass's panels are on their way while this one is multiplied
+    if (k0 + rows_cap < k_lim) request(k0 + rows_cap);
     __syncthreads();
     // dense product
     const float *ap = As + half * kAmT + wt + r32;
@@ -1249,7 +1266,8 @@ __global__ void __launch_bounds__(kLmThreads, 2)
   simple_bwd_lm_slab_body<kS, kK>((int)blockIdx.x, lm, am, symbols, lm_max, am_max, dmat, row_x,
                                   row_y, lm_grad, window, B, S, T, C, ldd, term);
 }
-__global__ void __launch_bounds__(256, 2)
+template <int kCap, int kPerCu>
+__global__ void __launch_bounds__(256, kPerCu)
     simple_bwd_am_panel_kernel(const float *__restrict__ lm, const float *__restrict__ am,
                                const int64_t *__restrict__ symbols,
                                const int64_t *__restrict__ boundary,
@@ -1259,8 +1277,9 @@ __global__ void __launch_bounds__(256, 2)
                                float *__restrict__ am_grad, const int64_t *__restrict__ window,
                                int B, int S, int T, int C, int ldd, int term, int rnnt_type,
                                int rows_cap) {
-  simple_bwd_am_panel_body((int)blockIdx.x, lm, am, symbols, boundary, lm_max, am_max, dmat, gpx,
-                           col_y, am_grad, window, B, S, T, C, ldd, term, rnnt_type, rows_cap);
+  simple_bwd_am_panel_body<kCap>((int)blockIdx.x, lm, am, symbols, boundary, lm_max, am_max, dmat,
+                                 gpx, col_y, am_grad, window, B, S, T, C, ldd, term, rnnt_type,
+                                 rows_cap);
 }
 // Both gradient products in one launch: the first lm_blocks workgroups take tiles of
 // lm.grad, the rest tiles of am.grad.  The two only read what the prep kernel left, so
@@ -1286,7 +1305,7 @@ __global__ void __launch_bounds__(256, 2)
     simple_bwd_lm_slab_body<kS, kK>((int)blockIdx.x, lm, am, symbols, lm_max, am_max, dmat, row_x,
                                     row_y, lm_grad, window, B, S, T, C, ldd, term);
   else
-    simple_bwd_am_panel_body((int)blockIdx.x - lm_blocks, lm, am, symbols, boundary, lm_max, am_max,
+    simple_bwd_am_panel_body<kAmCap>((int)blockIdx.x - lm_blocks, lm, am, symbols, boundary, lm_max, am_max,
                              dmat, gpx, col_y, am_grad, window, B, S, T, C, ldd, term, rnnt_type,
                              rows_cap);
 }
@@ -1302,7 +1321,7 @@ void launch_bwd_both(const float *lm, const float *am, const int64_t *symbols,
   const int rows = rows96 ? 96 : 128;
   const int lm_tiles = ((C + kLmC - 1) / kLmC) * ((S1 + rows - 1) / rows);
   const int am_tiles = ((C + kAmC - 1) / kAmC) * ((T + kAmT - 1) / kAmT);
-  const int rows_cap = std::min(kAmRows, (S + 2) & ~1);
+  const int rows_cap = am_rows_per_pass(S);
   // (frames in slabs of 16 here also for the 96-row form: its LDS is then 50 KB, not 67,
   // and three workgroups fit on a CU whichever product they work on: 33.4 us against 36.2)
   const size_t lm_lds = rows96 ? LmShape<96, 16>::kLdsBytes : LmShape<128, 16>::kLdsBytes;
@@ -1349,10 +1368,16 @@ void launch_bwd_am(const float *lm, const float *am, const int64_t *symbols,
                    int rnnt_type, hipStream_t stream) {
   const int tiles = ((C + kAmC - 1) / kAmC) * ((T + kAmT - 1) / kAmT);
   // rows of k held in LDS per pass: all of them when they fit
-  const int rows_cap = std::min(kAmRows, (S + 2) & ~1);
+  // Rows of k held in LDS per pass: at most 64, in passes of equal size.  The workgroup's
+  // phases (panels in, exp, products, results out) do not overlap inside it, so the compute
+  // unit needs several of them; 64 rows of panels leave room for four (128 rows: two), and the
+  // next pass's panels are requested before the current one is multiplied (B = 16, S + 1 = 121,
+  // T = 400, C = 5000: 154 us with one pass of 122 rows, 138 with two of 64 as three workgroups
+  // per compute unit).
+  const int rows_cap = am_rows_per_pass(S);
   const size_t lds = am_panel_lds_bytes(rows_cap);
   // (the 16-byte accesses need no alignment)
-  auto kernel = simple_bwd_am_panel_kernel;
+  auto kernel = simple_bwd_am_panel_kernel<kAmCap, 4>;
   (void)allow_lds(reinterpret_cast<const void *>(kernel), lds);
   hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(tiles, B)), dim3(256), lds, stream, lm, am,
                      symbols, boundary, lm_max, am_max, dmat, gpx, col_y, am_grad, window, B, S, T, C,
