@@ -41,6 +41,10 @@ _SIGNATURES = {
     "frnnt_smoothed_logprobs_bwd_f64": ([_P] * 20 + [_I] * 6 + [_D, _D, _P], _I),
     "frnnt_simple_loss_fwd_f32": ([_P] * 14 + [_I] * 7 + [_P], _I),
     "frnnt_simple_loss_fwd_f64": ([_P] * 14 + [_I] * 7 + [_P], _I),
+    "frnnt_mi_loss_fwd_f32": ([_P] * 8 + [_I] * 5 + [_P], _I),
+    "frnnt_mi_loss_fwd_f64": ([_P] * 8 + [_I] * 5 + [_P], _I),
+    "frnnt_mi_scale_grads_f32": ([_P] * 3 + [_I, _D] + [_I] * 4 + [_P], _I),
+    "frnnt_mi_scale_grads_f64": ([_P] * 3 + [_I, _D] + [_I] * 4 + [_P], _I),
     "frnnt_loss_reduce_f32": ([_P, _P, _I, _I, _P], _I),
     "frnnt_loss_reduce_f64": ([_P, _P, _I, _I, _P], _I),
     "frnnt_lattice_logprobs_fwd_f32": ([_P] * 9 + [_I] * 8 + [_P], _I),

@@ -1490,6 +1490,27 @@ int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
   return check_launch("simple_logprobs_bwd");
 }
 
+// px_grad[b] and py_grad[b] times score_grad_scale * score_grad[b * stride], in place: the
+// scaling step of the recursion's autograd backward (mutual_information.py:173-181).
+template <typename R>
+int scale_grads_impl(R *px_grad, R *py_grad, const R *score_grad, int score_grad_stride,
+                     double score_grad_scale, int B, int S, int T, int modified, void *stream) {
+  if (B < 0 || S < 0 || T < 0) return fail(FRNNT_EINVAL, "mi_scale_grads: negative size");
+  if (score_grad_stride != 0 && score_grad_stride != 1)
+    return fail(FRNNT_EINVAL, "mi_scale_grads: score_grad_stride must be 0 or 1");
+  if (B == 0) return FRNNT_OK;
+  if (!px_grad || !py_grad || !score_grad)
+    return fail(FRNNT_EINVAL, "mi_scale_grads: null pointer");
+  const int T1 = modified ? T : T + 1;
+  const int per_x = S * T1, per_y = (S + 1) * T;
+  const int x_blocks = (per_x + 1023) / 1024, y_blocks = (per_y + 1023) / 1024;
+  if (x_blocks + y_blocks > 0)
+    hipLaunchKernelGGL(scale_by_batch_kernel<R>, dim3(x_blocks + y_blocks, B), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), px_grad, py_grad, score_grad,
+                       score_grad_stride, (R)score_grad_scale, per_x, per_y, x_blocks);
+  return check_launch("mi_scale_grads");
+}
+
 template <typename R>
 int reduce_impl(const R *scores, R *loss, int B, int reduction, void *stream) {
   if (B < 0 || reduction < 0 || reduction > 2)
@@ -1607,6 +1628,18 @@ int frnnt_simple_logprobs_bwd_f64(const double *lm, const double *am, const int6
                                  termination_symbol, rnnt_type, window_only, stream);
 }
 
+int frnnt_mi_scale_grads_f32(float *px_grad, float *py_grad, const float *score_grad,
+                             int score_grad_stride, double score_grad_scale, int B, int S, int T,
+                             int modified, void *stream) {
+  return frnnt::scale_grads_impl<float>(px_grad, py_grad, score_grad, score_grad_stride,
+                                        score_grad_scale, B, S, T, modified, stream);
+}
+int frnnt_mi_scale_grads_f64(double *px_grad, double *py_grad, const double *score_grad,
+                             int score_grad_stride, double score_grad_scale, int B, int S, int T,
+                             int modified, void *stream) {
+  return frnnt::scale_grads_impl<double>(px_grad, py_grad, score_grad, score_grad_stride,
+                                         score_grad_scale, B, S, T, modified, stream);
+}
 int frnnt_loss_reduce_f32(const float *scores, float *loss, int B, int reduction, void *stream) {
   return frnnt::reduce_impl<float>(scores, loss, B, reduction, stream);
 }

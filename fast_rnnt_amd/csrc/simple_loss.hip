@@ -36,10 +36,47 @@ int simple_loss_fwd(Logprobs logprobs, Forward forward, Backward backward, Reduc
   return rc;
 }
 
+// The tail every loss function shares (e.g. rnnt_loss.py:326-340): the recursion, its
+// backward with a gradient of ones when the occupation gradients are wanted, the reduction.
+template <typename R, typename Forward, typename Backward, typename Reduce>
+int mi_loss_fwd(Forward forward, Backward backward, Reduce reduce, const R *px, const R *py,
+                const int64_t *boundary, R *p, R *scores, R *px_grad, R *py_grad, R *loss, int B,
+                int S, int T, int modified, int reduction, void *stream) {
+  if ((px_grad == nullptr) != (py_grad == nullptr))
+    return fail(FRNNT_EINVAL, "mi_loss_fwd: px_grad and py_grad go together");
+  int rc = forward(px, py, boundary, p, scores, B, S, T, modified, stream);
+  if (rc != FRNNT_OK) return rc;
+  if (px_grad) {
+    // with a loss to form, the backward kernel reduces the scores on its way
+    if (loss && B > 0)
+      return mi_backward_and_loss(px, boundary, p, px_grad, py_grad, scores, loss, B, S, T,
+                                  modified, reduction, stream);
+    rc = backward(px, py, boundary, p, nullptr, px_grad, py_grad, B, S, T, modified, 0, stream);
+    if (rc != FRNNT_OK) return rc;
+  }
+  if (loss) rc = reduce(scores, loss, B, reduction, stream);
+  return rc;
+}
+
 }  // namespace
 }  // namespace frnnt
 
 extern "C" {
+
+int frnnt_mi_loss_fwd_f32(const float *px, const float *py, const int64_t *boundary, float *p,
+                          float *scores, float *px_grad, float *py_grad, float *loss, int B, int S,
+                          int T, int modified, int reduction, void *stream) {
+  return frnnt::mi_loss_fwd<float>(frnnt_mi_forward_f32, frnnt_mi_backward_f32,
+                                   frnnt_loss_reduce_f32, px, py, boundary, p, scores, px_grad,
+                                   py_grad, loss, B, S, T, modified, reduction, stream);
+}
+int frnnt_mi_loss_fwd_f64(const double *px, const double *py, const int64_t *boundary, double *p,
+                          double *scores, double *px_grad, double *py_grad, double *loss, int B,
+                          int S, int T, int modified, int reduction, void *stream) {
+  return frnnt::mi_loss_fwd<double>(frnnt_mi_forward_f64, frnnt_mi_backward_f64,
+                                    frnnt_loss_reduce_f64, px, py, boundary, p, scores, px_grad,
+                                    py_grad, loss, B, S, T, modified, reduction, stream);
+}
 
 int frnnt_simple_loss_fwd_f32(const float *lm, const float *am, const int64_t *symbols,
                               const int64_t *boundary, float *px, float *py, float *lm_max,

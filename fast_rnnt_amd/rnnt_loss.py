@@ -194,25 +194,83 @@ def _apply_delay_penalty(px: Tensor, boundary: Optional[Tensor], rnnt_type: str,
     px += penalty.to(px.dtype)
 
 
+_REDUCTIONS = {"none": 0, "mean": 1, "sum": 2}
+
+
+class _RecursionLoss(torch.autograd.Function):
+    """The tail the loss functions share, behind one autograd node: the lattice recursion, --
+    as its autograd wrapper does whenever gradients will be wanted
+    (mutual_information.py:159-168) -- its backward with a gradient of ones, and the
+    reduction of the scores to the loss (rnnt_loss.py:326-340).  backward() scales the
+    occupation gradients in place by the loss's gradient, sign and 1/B of the reduction
+    included, exactly as MutualInformationRecursionFunction.backward does to the tensors
+    it handed out (mutual_information.py:173-181), and passes them on as the gradients of
+    px / py.  Same arithmetic as mutual_information_recursion followed by the torch
+    reduction; one library call each way instead of a dozen small kernels."""
+
+    @staticmethod
+    def forward(ctx, px, py, boundary, want_grads, reduction):
+        B, S, T1 = px.shape
+        T = py.shape[2]
+        sfx = _lib.suffix(px.dtype)
+        bnd_c = boundary.contiguous() if boundary is not None else None
+        opts = dict(dtype=px.dtype, device=px.device)
+        need_grad = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        ctx.set_materialize_grads(False)
+        with _on_device(px.device):
+            p = torch.empty(B, S + 1, T + 1, **opts)
+            scores = torch.empty(B, **opts)
+            px_grad = py_grad = None
+            if want_grads or need_grad:
+                px_grad = torch.empty(B, S, T1, **opts)
+                py_grad = torch.empty(B, S + 1, T, **opts)
+            loss = torch.empty((B,) if reduction == 0 else (), **opts)
+            _lib.call("frnnt_mi_loss_fwd_" + sfx, px.data_ptr(), py.data_ptr(), _lib.ptr(bnd_c),
+                      p.data_ptr(), scores.data_ptr(), _lib.ptr(px_grad), _lib.ptr(py_grad),
+                      loss.data_ptr(), B, S, T, int(T1 == T), reduction, _lib.stream_of(px))
+        if need_grad:
+            ctx.save_for_backward(px_grad, py_grad)
+            ctx.meta = (B, S, T, int(T1 == T), sfx, reduction)
+        if px_grad is None:
+            return loss, None, None
+        ctx.mark_non_differentiable(px_grad, py_grad)
+        return loss, px_grad, py_grad
+
+    @staticmethod
+    def backward(ctx, g_loss, _gx, _gy):
+        if g_loss is None:
+            return (None,) * 5
+        px_grad, py_grad = ctx.saved_tensors
+        B, S, T, modified, sfx, reduction = ctx.meta
+        with _on_device(px_grad.device):
+            g = g_loss.contiguous()
+            stride = 1 if reduction == 0 else 0
+            scale = -1.0 / B if reduction == 1 else -1.0
+            _lib.call("frnnt_mi_scale_grads_" + sfx, px_grad.data_ptr(), py_grad.data_ptr(),
+                      g.data_ptr(), stride, scale, B, S, T, modified, _lib.stream_of(px_grad))
+        return px_grad, py_grad, None, None, None
+
+
 def _recursion_and_reduce(px, py, boundary, rnnt_type, delay_penalty, reduction, return_grad):
     """Shared tail of the four losses (e.g. rnnt_loss.py:309-340)."""
     if delay_penalty > 0.0:
         _apply_delay_penalty(px, boundary, rnnt_type, delay_penalty)
-    scores_and_grads = mutual_information_recursion(
-        px=px, py=py, boundary=boundary, return_grad=return_grad)
-    negated_loss = scores_and_grads[0] if return_grad else scores_and_grads
-    if reduction == "none":
-        loss = -negated_loss
-    elif reduction == "mean":
-        loss = -torch.mean(negated_loss)
-    elif reduction == "sum":
-        loss = -torch.sum(negated_loss)
-    else:
+    if reduction not in _REDUCTIONS:
+        # (the reference finds this out after the recursion has run: same exception)
         raise ValueError(f"reduction should be ('none' | 'mean' | 'sum'), given {reduction}")
-    return (loss, scores_and_grads[1]) if return_grad else loss
-
-
-_REDUCTIONS = {"none": 0, "mean": 1, "sum": 2}
+    # the argument checks of mutual_information_recursion (mutual_information.py:271-289)
+    assert px.ndim == 3
+    B, S, T1 = px.shape
+    T = py.shape[-1]
+    assert px.shape[-1] in [T, T + 1]
+    assert py.shape == (B, S + 1, T)
+    assert px.dtype == py.dtype
+    if boundary is not None:
+        _assert_boundary(boundary, B, S, T)
+    _require_gpu(px, py)
+    loss, px_grad, py_grad = _RecursionLoss.apply(px.contiguous(), py.contiguous(), boundary,
+                                                  bool(return_grad), _REDUCTIONS[reduction])
+    return (loss, (px_grad, py_grad)) if return_grad else loss
 
 
 def _on_device(device):
@@ -500,12 +558,21 @@ def get_rnnt_prune_ranges(px_grad: Tensor, py_grad: Tensor, boundary: Tensor,
     _check_tensors([("px_grad", px_grad), ("py_grad", py_grad)], [("boundary", boundary)])
 
     if is_regular:
-        Ss = boundary[:, 2]
-        Ts = boundary[:, 3]
-        s_range_min = Ss.sub(1).div(Ts, rounding_mode="trunc").add(2).max().item()
-        if s_range < s_range_min:
+        # max over the batch of trunc((S_b - 1) / T_b) + 2 (rnnt_loss.py:696-710), from the
+        # host copy of the boundary rows that the loss call before this one has usually left
+        # behind: no kernels and no wait for the device here
+        s_range_min = None
+        for _s_begin, _t_begin, s_end, t_end in boundary_rows(boundary):
+            if t_end == 0:
+                raise RuntimeError("ZeroDivisionError")  # what the reference's integer division raises
+            quotient = abs(s_end - 1) // abs(t_end)
+            if (s_end - 1 < 0) != (t_end < 0):
+                quotient = -quotient
+            s_range_min = quotient + 2 if s_range_min is None else max(s_range_min, quotient + 2)
+        if s_range_min is not None and s_range < s_range_min:
             print(f"Warning: get_rnnt_prune_ranges - got s_range={s_range} "
-                  f"for boundaries S={Ss}, T={Ts}. Adjusting to {s_range_min}")
+                  f"for boundaries S={boundary[:, 2]}, T={boundary[:, 3]}. "
+                  f"Adjusting to {s_range_min}")
             s_range = s_range_min
     if s_range > S:
         s_range = S + 1

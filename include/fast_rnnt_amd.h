@@ -264,6 +264,32 @@ int frnnt_simple_loss_fwd_f64(const double *lm, const double *am, const int64_t 
                               void *stream);
 
 /*
+ * The tail every loss function shares (rnnt_loss.py:326-340, :535-547, :1119-1132, :1481-1494)
+ * in one call: frnnt_mi_forward, then -- when px_grad / py_grad are given -- frnnt_mi_backward
+ * with a gradient of ones (mutual_information.py:159-168), then -- when loss is given --
+ * frnnt_loss_reduce (the backward kernel reduces the scores on its way: no extra launch).
+ * p [B][S+1][T+1] and scores [B] are outputs as well.
+ */
+int frnnt_mi_loss_fwd_f32(const float *px, const float *py, const int64_t *boundary, float *p,
+                          float *scores, float *px_grad, float *py_grad, float *loss, int B, int S,
+                          int T, int modified, int reduction, void *stream);
+int frnnt_mi_loss_fwd_f64(const double *px, const double *py, const int64_t *boundary, double *p,
+                          double *scores, double *px_grad, double *py_grad, double *loss, int B,
+                          int S, int T, int modified, int reduction, void *stream);
+/*
+ * The backward of that tail: px_grad[b] and py_grad[b] are multiplied IN PLACE by
+ * score_grad_scale * score_grad[b * score_grad_stride] -- what the recursion's autograd
+ * backward does to the tensors it handed out (mutual_information.py:173-181), with the
+ * reduction's sign and 1/B in score_grad_scale (stride 0: one scalar for all utterances).
+ */
+int frnnt_mi_scale_grads_f32(float *px_grad, float *py_grad, const float *score_grad,
+                             int score_grad_stride, double score_grad_scale, int B, int S, int T,
+                             int modified, void *stream);
+int frnnt_mi_scale_grads_f64(double *px_grad, double *py_grad, const double *score_grad,
+                             int score_grad_stride, double score_grad_scale, int B, int S, int T,
+                             int modified, void *stream);
+
+/*
  * The reduction at the end of every loss function (rnnt_loss.py:160-169, :330-340):
  * loss = -scores (reduction 0, [B]), -mean(scores) (1, one value) or -sum(scores)
  * (2, one value), summed in a fixed order by one workgroup.
