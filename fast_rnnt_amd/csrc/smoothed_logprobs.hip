@@ -190,7 +190,8 @@ __global__ void __launch_bounds__(256)
 template <typename R>
 __global__ void __launch_bounds__(256)
     smoothed_combine_kernel(const R *__restrict__ lm, const R *__restrict__ am,
-                            const int64_t *__restrict__ symbols, const R *__restrict__ pxj,
+                            const int64_t *__restrict__ symbols,
+                            const int64_t *__restrict__ boundary, const R *__restrict__ pxj,
                             const R *__restrict__ pyj, const R *__restrict__ lm_max,
                             const R *__restrict__ lm_sum, const R *__restrict__ am_max,
                             const R *__restrict__ am_z, const R *__restrict__ unigram,
@@ -216,7 +217,11 @@ __global__ void __launch_bounds__(256)
       const R an = log(am_z[arow]) + am_max[arow];
       am_only = ((in ? am[arow * C + sym] : nan) + (in ? log(unigram[sym]) : nan)) - an;
     }
-    px[idx] = pxj[idx] * k_joint + lm_only * k_lm + am_only * k_am;
+    R v = pxj[idx] * k_joint + lm_only * k_lm + am_only * k_am;
+    // nothing can be emitted after an utterance's last frame (fix_for_boundary,
+    // rnnt_loss.py:45-63, applied by the reference after the interpolation)
+    if (boundary && regular && boundary[4 * b + 3] == t) v = Num<R>::neg_inf();
+    px[idx] = v;
   } else if (idx < n_px + n_py) {
     const long j = idx - n_px;
     const int t = (int)(j % T);
@@ -506,7 +511,8 @@ __global__ void __launch_bounds__(256)
 }
 
 template <typename R>
-int fwd_impl(const R *lm, const R *am, const int64_t *symbols, const R *pxj, const R *pyj, R *px,
+int fwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *boundary,
+             const R *pxj, const R *pyj, R *px,
              R *py, R *lm_max, R *lm_sum, R *am_max, R *am_z, R *unigram, R *partial, int B, int S,
              int T, int C, int term, int regular, double lm_only_scale, double am_only_scale,
              void *stream_) {
@@ -535,7 +541,7 @@ int fwd_impl(const R *lm, const R *am, const int64_t *symbols, const R *pxj, con
   const R k_joint = (R)(1.0 - lm_only_scale - am_only_scale);
   if (total > 0)
     hipLaunchKernelGGL(smoothed_combine_kernel<R>, dim3((unsigned)((total + 255) / 256)),
-                       dim3(256), 0, stream, lm, am, symbols, pxj, pyj, lm_max, lm_sum, am_max,
+                       dim3(256), 0, stream, lm, am, symbols, boundary, pxj, pyj, lm_max, lm_sum, am_max,
                        am_z, unigram, px, py, B, S, T, C, term, regular, k_joint, k_lm, k_am);
   return check_launch("smoothed_logprobs_fwd");
 }
@@ -599,22 +605,24 @@ int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const R *lm_max, 
 extern "C" {
 
 int frnnt_smoothed_logprobs_fwd_f32(const float *lm, const float *am, const int64_t *symbols,
+                                    const int64_t *boundary,
                                     const float *px_joint, const float *py_joint, float *px,
                                     float *py, float *lm_max, float *lm_sum, float *am_max,
                                     float *am_z, float *unigram, float *partial, int B, int S,
                                     int T, int C, int termination_symbol, int regular,
                                     double lm_only_scale, double am_only_scale, void *stream) {
-  return frnnt::fwd_impl<float>(lm, am, symbols, px_joint, py_joint, px, py, lm_max, lm_sum, am_max,
+  return frnnt::fwd_impl<float>(lm, am, symbols, boundary, px_joint, py_joint, px, py, lm_max, lm_sum, am_max,
                                 am_z, unigram, partial, B, S, T, C, termination_symbol, regular,
                                 lm_only_scale, am_only_scale, stream);
 }
 int frnnt_smoothed_logprobs_fwd_f64(const double *lm, const double *am, const int64_t *symbols,
+                                    const int64_t *boundary,
                                     const double *px_joint, const double *py_joint, double *px,
                                     double *py, double *lm_max, double *lm_sum, double *am_max,
                                     double *am_z, double *unigram, double *partial, int B, int S,
                                     int T, int C, int termination_symbol, int regular,
                                     double lm_only_scale, double am_only_scale, void *stream) {
-  return frnnt::fwd_impl<double>(lm, am, symbols, px_joint, py_joint, px, py, lm_max, lm_sum,
+  return frnnt::fwd_impl<double>(lm, am, symbols, boundary, px_joint, py_joint, px, py, lm_max, lm_sum,
                                  am_max, am_z, unigram, partial, B, S, T, C, termination_symbol,
                                  regular, lm_only_scale, am_only_scale, stream);
 }

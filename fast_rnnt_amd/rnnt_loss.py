@@ -761,12 +761,17 @@ class _SmoothedCombine(torch.autograd.Function):
     (rnnt_loss.py:1264-1355): frnnt_smoothed_logprobs_fwd/bwd."""
 
     @staticmethod
-    def forward(ctx, pxj, pyj, lm, am, symbols, termination_symbol, regular, k_lm, k_am):
+    def forward(ctx, pxj, pyj, lm, am, symbols, boundary, termination_symbol, regular, k_lm,
+                k_am):
+        # boundary (regular lattice): px[b, :, t_end] = -inf, the reference's
+        # fix_for_boundary after the interpolation (rnnt_loss.py:1364-1365); the gradient
+        # the recursion returns for those cells is zero, so backward() has nothing to mask
         B, T, C = am.shape
         S = lm.shape[1] - 1
         sfx = _lib.suffix(am.dtype)
         lm_c, am_c, sym_c = lm.contiguous(), am.contiguous(), symbols.contiguous()
         pxj_c, pyj_c = pxj.contiguous(), pyj.contiguous()
+        bnd_c = boundary.contiguous() if (boundary is not None and regular) else None
         opts = dict(dtype=am.dtype, device=am.device)
         n_lm, n_am = B * (S + 1), B * T
         # kept for the backward: lm_max | lm_sum | am_max | am_z | unigram
@@ -778,7 +783,8 @@ class _SmoothedCombine(torch.autograd.Function):
             partial = torch.empty((n_lm + 15) // 16 * C, **opts)
             base, item = stats.data_ptr(), stats.element_size()
             _lib.call("frnnt_smoothed_logprobs_fwd_" + sfx, lm_c.data_ptr(), am_c.data_ptr(),
-                      sym_c.data_ptr(), pxj_c.data_ptr(), pyj_c.data_ptr(), px.data_ptr(),
+                      sym_c.data_ptr(), _lib.ptr(bnd_c), pxj_c.data_ptr(), pyj_c.data_ptr(),
+                      px.data_ptr(),
                       py.data_ptr(), base + o_lmx * item, base + o_lms * item,
                       base + o_amx * item, base + o_amz * item, base + o_u * item,
                       partial.data_ptr(), B, S, T, C, int(termination_symbol), int(regular),
@@ -812,13 +818,14 @@ class _SmoothedCombine(torch.autograd.Function):
                       sb + o_rx * item, sb + o_ry * item, sb + o_cy * item, sb + o_cg * item,
                       sb + o_gu * item, sb + o_p * item, B, S, T, C, term, regular, k_lm, k_am,
                       _lib.stream_of(am))
-        return gxj, gyj, lm_grad, am_grad, None, None, None, None, None
+        return gxj, gyj, lm_grad, am_grad, None, None, None, None, None, None
 
 
 def get_rnnt_logprobs_smoothed(
     lm: Tensor, am: Tensor, symbols: Tensor, termination_symbol: int,
     lm_only_scale: float = 0.1, am_only_scale: float = 0.1,
     boundary: Optional[Tensor] = None, rnnt_type: str = "regular",
+    _mask_in_kernel: bool = False,
 ) -> Tuple[Tensor, Tensor]:
     """(px, py) interpolating the joint model with an lm-only and an am-only
     (unigram-lm) model (rnnt_loss.py:1135-1369)::
@@ -851,12 +858,19 @@ def get_rnnt_logprobs_smoothed(
         lm_only_scale = 1.0e-20
     if am_only_scale == 0.0:
         am_only_scale = 1.0e-20
+    # _mask_in_kernel (rnnt_loss_smoothed): the caller feeds (px, py) to the recursion with
+    # this boundary, whose gradient at the cells fix_for_boundary sets to -inf is zero -- the
+    # kernel then writes those -inf itself and no masking node is needed on the way back.
+    # The public helper keeps the reference's scatter_, whose backward zeroes whatever
+    # gradient a caller sends in there.
+    fused_mask = _mask_in_kernel and rnnt_type == "regular" and boundary is not None
     px_interp, py_interp = _SmoothedCombine.apply(
-        px, py, lm, am, symbols, termination_symbol, rnnt_type == "regular",
-        float(lm_only_scale), float(am_only_scale))
+        px, py, lm, am, symbols, boundary if fused_mask else None, termination_symbol,
+        rnnt_type == "regular", float(lm_only_scale), float(am_only_scale))
 
     if rnnt_type == "regular":
-        px_interp = fix_for_boundary(px_interp, boundary)
+        if not fused_mask:
+            px_interp = fix_for_boundary(px_interp, boundary)
     elif rnnt_type == "constrained":
         px_interp += py_interp[:, 1:, :]
     return (px_interp, py_interp)
@@ -872,6 +886,6 @@ def rnnt_loss_smoothed(
     px, py = get_rnnt_logprobs_smoothed(
         lm=lm, am=am, symbols=symbols, termination_symbol=termination_symbol,
         lm_only_scale=lm_only_scale, am_only_scale=am_only_scale, boundary=boundary,
-        rnnt_type=rnnt_type)
+        rnnt_type=rnnt_type, _mask_in_kernel=True)
     return _recursion_and_reduce(px, py, boundary, rnnt_type, delay_penalty, reduction,
                                  return_grad)

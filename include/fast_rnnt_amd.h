@@ -201,8 +201,10 @@ int frnnt_simple_logprobs_bwd_noalloc_f32(const float *lm, const float *am, cons
  *   px = px_joint * (1 - l - a) + lm_only_px * l + am_only_px * a     (same for py)
  * with l = lm_only_scale, a = am_only_scale, the lm-only model log_softmax(lm) and the
  * am-only model am + log(unigram) normalised per frame, unigram = mean over all
- * (b, s) of softmax(lm[b,s,:]) + tiny.  The boundary / constrained post-processing of
- * the reference (rnnt_loss.py:1357-1367) is left to the caller.
+ * (b, s) of softmax(lm[b,s,:]) + tiny.  With a boundary (regular lattice) px[b][:][t_end] is
+ * set to -inf after the interpolation (fix_for_boundary, rnnt_loss.py:1364-1365; the
+ * gradient that comes back for those cells is zero, so the backward entry point needs
+ * nothing for it); the constrained "px += py[:, 1:]" step is left to the caller.
  *   lm_max, lm_sum [B][S+1], am_max, am_z [B][T], unigram [C]: out, kept for the backward
  *   partial [ceil(B*(S+1)/16)][C] (forward), [ceil(B*T/16)][C] (backward): scratch
  * Backward: px_grad / py_grad are the gradients of px / py; out are the gradients of
@@ -211,13 +213,13 @@ int frnnt_simple_logprobs_bwd_noalloc_f32(const float *lm, const float *am, cons
  * row_x, row_y [B][S+1], col_y, col_g [B][T], g_unigram [C]: scratch.
  */
 int frnnt_smoothed_logprobs_fwd_f32(const float *lm, const float *am, const int64_t *symbols,
-                                    const float *px_joint, const float *py_joint, float *px,
+                                    const int64_t *boundary, const float *px_joint, const float *py_joint, float *px,
                                     float *py, float *lm_max, float *lm_sum, float *am_max,
                                     float *am_z, float *unigram, float *partial, int B, int S,
                                     int T, int C, int termination_symbol, int regular,
                                     double lm_only_scale, double am_only_scale, void *stream);
 int frnnt_smoothed_logprobs_fwd_f64(const double *lm, const double *am, const int64_t *symbols,
-                                    const double *px_joint, const double *py_joint, double *px,
+                                    const int64_t *boundary, const double *px_joint, const double *py_joint, double *px,
                                     double *py, double *lm_max, double *lm_sum, double *am_max,
                                     double *am_z, double *unigram, double *partial, int B, int S,
                                     int T, int C, int termination_symbol, int regular,
