@@ -497,6 +497,86 @@ def test_pruned_joiner_input_matches_gather_then_tanh(gpu_device, dtype):
     assert torch.isnan(out[0, 0, 0]).all() and torch.isfinite(out[0, 0, 1]).all()
 
 
+@pytest.mark.parametrize("reduction", ["none", "mean", "sum"])
+@pytest.mark.parametrize("which", ["joint", "pruned", "smoothed"])
+def test_loss_tail_reductions_weights_and_returned_gradients(gpu_device, which, reduction):
+    """The part the three losses share after px, py: delay penalty, recursion, reduction.
+
+    The loss is weighted per utterance before backward() (for "none"), so that the
+    gradient of the scores is not a constant; px_grad / py_grad are compared as returned
+    (the occupation counts) and after backward(), which scales them in place as the
+    reference's recursion does (mutual_information.py:162-178).
+    """
+    dev = gpu_device
+    kind = "regular"
+    B, S, T, C, R = 4, 7, 19, 11, 4
+    am, lm, sym, bnd = _case(300, B, S, T, C, torch.float64, kind)
+    w = torch.tensor([0.5, -1.25, 2.0, 0.0], dtype=torch.float64)
+
+    def run(mod_losses, to):
+        a = to(am).requires_grad_(True)
+        l = to(lm).requires_grad_(True)
+        kw = dict(boundary=to(bnd), rnnt_type=kind, delay_penalty=0.02, reduction=reduction,
+                  return_grad=True)
+        if which == "smoothed":
+            loss, (gx, gy) = mod_losses["smoothed"](l, a, to(sym), 2, 0.3, 0.1, **kw)
+        elif which == "joint":
+            logits = torch.tanh(a.unsqueeze(2) + l.unsqueeze(1)) * 2
+            loss, (gx, gy) = mod_losses["joint"](logits, to(sym), 2, **kw)
+        else:
+            start = torch.clamp(torch.arange(T) * (S + 1 - R) // T, 0, S + 1 - R)
+            ranges = to((start.reshape(1, T, 1) + torch.arange(R).reshape(1, 1, R))
+                        .expand(B, T, R).contiguous())
+            lp = torch.gather(l.unsqueeze(1).expand(B, T, S + 1, C), 2,
+                              ranges.unsqueeze(3).expand(B, T, R, C))
+            logits = torch.tanh(a.unsqueeze(2) + lp) * 2
+            loss, (gx, gy) = mod_losses["pruned"](logits, to(sym), ranges, 2, **kw)
+        before = gx.detach().clone(), gy.detach().clone()
+        total = (loss * to(w)).sum() if reduction == "none" else loss * 1.5
+        total.backward()
+        return loss, before, (gx.detach(), gy.detach()), a.grad, l.grad
+
+    want = run({"smoothed": O.loss_smoothed, "joint": O.loss_joint, "pruned": O.loss_pruned},
+               lambda x: x.clone())
+    got = run({"smoothed": fast_rnnt_amd.rnnt_loss_smoothed, "joint": fast_rnnt_amd.rnnt_loss,
+               "pruned": fast_rnnt_amd.rnnt_loss_pruned}, lambda x: x.to(dev))
+    _say(f"loss tail {which} {reduction}")
+    assert got[0].shape == want[0].shape and _close(got[0], want[0], 0.0, 1e-6)
+    for i in (0, 1):
+        assert _close(got[1][i], want[1][i], 1e-7), "occupation counts as returned"
+        assert _close(got[2][i], want[2][i], 1e-7), "the same tensors after backward()"
+    # backward() did rescale them: by -w[b], -1.5/B or -1.5
+    scale = {"none": -w, "mean": torch.full((B,), -1.5 / B, dtype=torch.float64),
+             "sum": torch.full((B,), -1.5, dtype=torch.float64)}[reduction]
+    assert _close(got[2][0], got[1][0].cpu() * scale.reshape(B, 1, 1), 1e-12)
+    assert _close(got[3], want[3], 1e-7, 1e-7) and _close(got[4], want[4], 1e-7, 1e-7)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_smoothed_loss_equals_helper_then_recursion(gpu_device, kind):
+    """rnnt_loss_smoothed writes the -inf beyond the last frame inside its kernel; the public
+    get_rnnt_logprobs_smoothed followed by the recursion (rnnt_loss.py:1357-1362, 1466-1473)
+    must give the same loss and gradients."""
+    dev = gpu_device
+    am, lm, sym, bnd = _case(310, 3, 9, 26, 15, torch.float64, kind)
+    res = []
+    for direct in (True, False):
+        a = am.to(dev).requires_grad_(True)
+        l = lm.to(dev).requires_grad_(True)
+        if direct:
+            loss = fast_rnnt_amd.rnnt_loss_smoothed(l, a, sym.to(dev), 1, 0.2, 0.1,
+                                                    boundary=bnd.to(dev), rnnt_type=kind,
+                                                    reduction="none")
+        else:
+            px, py = fast_rnnt_amd.get_rnnt_logprobs_smoothed(l, a, sym.to(dev), 1, 0.2, 0.1,
+                                                              boundary=bnd.to(dev), rnnt_type=kind)
+            loss = -fast_rnnt_amd.mutual_information_recursion(px, py, bnd.to(dev))
+        loss.sum().backward()
+        res.append((loss.detach(), a.grad, l.grad))
+    for x, y in zip(*res):
+        assert _close(x, y, 1e-12, 1e-12)
+
+
 def test_c5_unpruned_full_size(gpu_device):
     dev = gpu_device
     w = workloads.make("c5")
