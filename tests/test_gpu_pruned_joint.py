@@ -555,7 +555,7 @@ def test_loss_tail_reductions_weights_and_returned_gradients(gpu_device, which, 
 @pytest.mark.parametrize("kind", KINDS)
 def test_smoothed_loss_equals_helper_then_recursion(gpu_device, kind):
     """rnnt_loss_smoothed writes the -inf beyond the last frame inside its kernel; the public
-    get_rnnt_logprobs_smoothed followed by the recursion (rnnt_loss.py:1357-1362, 1466-1473)
+    get_rnnt_logprobs_smoothed followed by the recursion (rnnt_loss.py:1364-1365, 1480-1494)
     must give the same loss and gradients."""
     dev = gpu_device
     am, lm, sym, bnd = _case(310, 3, 9, 26, 15, torch.float64, kind)
