@@ -368,15 +368,15 @@ def _bench_lattice(args, w, dev):
         # the same step with pruned_joiner_input in the place of do_rnnt_pruning and the
         # caller's add + tanh: lm_pruned is never written or read back
         fused = _rate(args.steps, _wall_loop(lambda: pipeline(True), args.steps, args.warmup))
-        # the caller's joiner (not part of the library): the [B*T*R, C] x [C, C] product,
-        # forward and its two backward products
+        # the caller's joiner (not part of the library): the [B*T*R, C] x [C, C] product and
+        # the product that takes the gradient back to the joiner's input (the projection is a
+        # constant of the workload, so the step forms no gradient for it)
         g_out = torch.empty_like(lg, dtype=torch.float32)
         h2 = hidden.reshape(-1, w.C)
 
         def joiner_products():
             torch.matmul(h2, W)
             torch.matmul(g_out.reshape(-1, w.C), W.t())
-            torch.matmul(h2.t(), g_out.reshape(-1, w.C))
 
         t_join = _event_time_ms(joiner_products, max(5, args.kernel_reps // 5))
         extra = {"with_pruned_joiner_input": fused,
