@@ -3,8 +3,9 @@
 // prune_ranges (fast_rnnt/python/fast_rnnt/rnnt_loss.py:638-777, helpers
 // :550-632): for every frame pick the window start s that maximises
 //   sum_{j<R} py_grad[b,s+j,t] - px_grad[b,s-1,t]        (0 for s = 0)
-// with the window sum formed strictly left to right in the input precision and
-// ties resolved to the first maximum, replace the starts of frames at or beyond
+// with the window sum formed in the input precision in the order of the reference's
+// torch.sum on the CPU (left to right up to 16 values, in stretches of 16 beyond: see
+// window_sum below) and ties resolved to the first maximum, replace the starts of frames at or beyond
 // T_b - 1 by max(S_b - R + 1, 0), then make the starts non-decreasing, starting
 // at 0, with steps smaller than r (r = R for the regular lattice, 2 otherwise)
 // by two suffix-minimum passes.  Two kernels: one lane per frame for the window
@@ -47,6 +48,44 @@ __device__ __forceinline__ void suffix_min_inplace(int *v, int n, int lane) {
   __syncthreads();
 }
 
+// The sum of the s_range values of one window, in the order in which the reference's
+// torch.sum adds them on the CPU (rnnt_loss.py:726-734 reduces a strided view over the
+// window axis; ATen's outer-sum loop, SumKernel.cpp multi_row_sum): left to right in
+// stretches of 16, each stretch's sum added to a second accumulator, that one to a third
+// after 16 stretches and to a fourth after 256, the remainder left to right, and at the
+// end the four added in order.  Up to 16 values that is plain left to right.  The order
+// matters: when the window is wider than the band of the lattice that holds the
+// alignment's mass, neighbouring window starts tie up to rounding, and the first maximum
+// among them is whatever the rounding makes it.  `at(j)` is the window's j-th value.
+template <typename R, typename F>
+__device__ __forceinline__ R window_sum(int width, F at) {
+  if (width <= 16) {
+    R sum = at(0);
+    for (int j = 1; j < width; ++j) sum = sum + at(j);
+    return sum;
+  }
+  R a1 = 0, a2 = 0, a3 = 0;
+  int i = 0;
+  while (i + 16 <= width) {
+    R c = at(i);
+#pragma unroll
+    for (int j = 1; j < 16; ++j) c = c + at(i + j);
+    i += 16;
+    a1 = a1 + c;
+    if ((i & 0xF0) == 0) {
+      a2 = a2 + a1;
+      a1 = 0;
+      if ((i & 0xF00) == 0) {
+        a3 = a3 + a2;
+        a2 = 0;
+      }
+    }
+  }
+  R rest = 0;
+  for (; i < width; ++i) rest = rest + at(i);
+  return ((rest + a1) + a2) + a3;
+}
+
 // Step 1, one lane per frame: the best window start of frame (b, t), left in
 // ranges[b][t][0].
 template <typename R>
@@ -72,8 +111,7 @@ __global__ void __launch_bounds__(kWave)
     }
   };
   auto score_of = [&](int s) {
-    R sum = gy[(long)s * T];
-    for (int j = 1; j < Rr; ++j) sum = sum + gy[(long)(s + j) * T];
+    const R sum = window_sum<R>(Rr, [&](int j) { return gy[(long)(s + j) * T]; });
     const R below = s >= 1 ? gx[(long)(s - 1) * T1] : (R)0;
     return sum - below;
   };
@@ -142,8 +180,7 @@ __global__ void __launch_bounds__(256)
     }
   };
   for (int s = lo; s < hi; ++s) {
-    R sum = ty[s * kWave + lane];
-    for (int j = 1; j < Rr; ++j) sum = sum + ty[(s + j) * kWave + lane];
+    const R sum = window_sum<R>(Rr, [&](int j) { return ty[(s + j) * kWave + lane]; });
     const R below = s >= 1 ? tx[(s - 1) * kWave + lane] : (R)0;
     consider(s, sum - below);
   }

@@ -389,7 +389,10 @@ int frnnt_lattice_logprobs_bwd_bf16(const void *logits, const int64_t *symbols,
  * (rnnt_loss.py:726-777 with _adjust_pruning_lower_bound :584-632).  s_range is
  * the FINAL window size: the caller has already raised it to the regular
  * lattice's minimum and capped it at S+1 (rnnt_loss.py:696-724), so
- * 1 <= s_range <= S+1.
+ * 1 <= s_range <= S+1.  The window sums are formed in the input precision and in the
+ * order of torch.sum on the CPU (left to right up to 16 rows, stretches of 16 merged
+ * upwards beyond), first maximum wins, NaN counts as the maximum: given the same
+ * gradients the ranges are those of the reference's CPU run, near-ties included.
  *   px_grad [B][S][T+1] (modified: [B][S][T]), py_grad [B][S+1][T], boundary [B][4]  in
  *   ranges int64 [B][T][s_range]                                                     out
  */

@@ -231,10 +231,42 @@ def adjust_lower_bound(s_begin: Tensor, r: int) -> Tensor:
     return ramp - y
 
 
+def window_sums_in_torch_cpu_order(py_grad: Tensor, n: int, width: int) -> Tensor:
+    """sum_j py_grad[:, s + j, :] for s < n, j < width, added in the order of ATen's CPU
+    loop for a sum over a strided axis whose neighbour axis is contiguous
+    (aten/src/ATen/native/cpu/SumKernel.cpp, multi_row_sum): left to right in stretches of
+    16 into a first accumulator, which is added to a second after every stretch, that one
+    to a third after 16 stretches and to a fourth after 256, the remainder left to right,
+    and at the end the four added in order.  Up to 16 values this is plain left to right.
+    torch.sum itself deviates from this for the last few output elements of each chunk
+    of its loop (those that do not fill four SIMD vectors are summed as four interleaved
+    partial sums), so which elements those are depends on the host's SIMD width and
+    thread count."""
+    B, _, T = py_grad.shape
+    zero = py_grad.new_zeros(B, n, T)
+    acc = [zero.clone() for _ in range(4)]
+    i = 0
+    while i + 16 <= width:
+        for _ in range(16):
+            acc[0] = acc[0] + py_grad[:, i:i + n, :]
+            i += 1
+        for level in range(1, 4):
+            acc[level] = acc[level] + acc[level - 1]
+            acc[level - 1] = zero.clone()
+            if i & (0xF << (4 * level)):
+                break
+    while i < width:
+        acc[0] = acc[0] + py_grad[:, i:i + n, :]
+        i += 1
+    return ((acc[0] + acc[1]) + acc[2]) + acc[3]
+
+
 def prune_ranges(px_grad, py_grad, boundary, s_range: int, window_sum: str = "torch") -> Tensor:
     """rnnt_loss.py:638-777.  ``window_sum='torch'`` reduces the strided window
     view with torch.sum exactly as the reference does (:726-734);
-    ``'ltr'`` adds the window rows strictly left to right in the input dtype."""
+    ``'ltr'`` adds the window rows strictly left to right in the input dtype;
+    ``'cascade'`` is window_sums_in_torch_cpu_order, the host-independent restatement of
+    what torch.sum does there."""
     B, S, T1 = px_grad.shape
     T = py_grad.shape[-1]
     regular = T1 != T
@@ -256,6 +288,8 @@ def prune_ranges(px_grad, py_grad, boundary, s_range: int, window_sum: str = "to
         sb, ss, st = py_grad.stride()
         win = torch.as_strided(py_grad, (B, n, s_range, T), (sb, ss, ss, st))
         blk = torch.sum(win, axis=2)
+    elif window_sum == "cascade":
+        blk = window_sums_in_torch_cpu_order(py_grad, n, s_range)
     else:
         blk = py_grad[:, 0:n, :].clone()
         for j in range(1, s_range):

@@ -127,6 +127,34 @@ def test_prune_ranges_random_bit_exact(gpu_device, dtype, kind):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_prune_ranges_wide_windows_bit_exact(gpu_device, dtype):
+    """s_range above 16, where the reference's torch.sum no longer adds the window left to
+    right (ATen's CPU loop sums in stretches of 16), on occupancies of short targets in a
+    tall lattice: the window covers the whole band that holds the alignment's mass, so
+    neighbouring window starts tie up to rounding and the summation order picks the
+    winner.  Against the oracle's torch.sum (frame counts that fill whole SIMD vectors,
+    where it has no differently summed tail) and against its host-independent
+    restatement of that order."""
+    dev = gpu_device
+    for seed, (B, S, T) in enumerate([(3, 69, 128), (2, 100, 64), (2, 150, 64)]):
+        g = torch.Generator().manual_seed(40 + seed)
+        am = torch.randn(B, T, 12, generator=g, dtype=dtype)
+        lm = torch.randn(B, S + 1, 12, generator=g, dtype=dtype)
+        sym = torch.randint(1, 12, (B, S), generator=g)
+        Sb = torch.randint(S // 4, S // 2, (B,), generator=g)
+        Tb = torch.randint(T // 2, T + 1, (B,), generator=g)
+        z = torch.zeros(B, dtype=torch.int64)
+        bnd = torch.stack([z, z, Sb, Tb], 1)
+        _, (gx, gy) = O.loss_simple(lm, am, sym, 0, boundary=bnd, reduction="sum",
+                                    return_grad=True)
+        for R in (16, 17, 19, 33, 40, 64):
+            _say(f"wide windows {dtype} B={B} S={S} T={T} R={R}")
+            got = fast_rnnt_amd.get_rnnt_prune_ranges(gx.to(dev), gy.to(dev), bnd.to(dev), R).cpu()
+            assert torch.equal(got, O.prune_ranges(gx, gy, bnd, R, window_sum="cascade"))
+            assert torch.equal(got, O.prune_ranges(gx, gy, bnd, R))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 def test_prune_ranges_ties_nans_and_long_targets(gpu_device, dtype):
     """Window scores with exact ties and NaNs (first maximum wins, NaN counts as the maximum,
     as torch.argmax in rnnt_loss.py:735-741), on targets short enough for the kernel that

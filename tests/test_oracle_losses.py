@@ -238,3 +238,54 @@ def test_golden_prune_ranges(capsys):
             assert torch.equal(px, c["px"]) and torch.equal(py, c["py"]), name
     assert "Adjusting to 4" in capsys.readouterr().out
     assert data["ties"]["ranges"][0, :, 0].tolist()[0] == 0
+
+
+def _occupancies(seed, B, S, T, C, dtype):
+    g = torch.Generator().manual_seed(seed)
+    am = torch.randn(B, T, C, generator=g, dtype=dtype)
+    lm = torch.randn(B, S + 1, C, generator=g, dtype=dtype)
+    sym = torch.randint(1, C, (B, S), generator=g)
+    # short targets in a tall lattice: a wide window covers the whole band that holds the
+    # alignment's mass, so neighbouring window starts tie up to rounding
+    Sb = torch.randint(S // 4, S // 2, (B,), generator=g)
+    Tb = torch.randint(T // 2, T + 1, (B,), generator=g)
+    z = torch.zeros(B, dtype=torch.int64)
+    bnd = torch.stack([z, z, Sb, Tb], 1)
+    _, (gx, gy) = losses.loss_simple(lm, am, sym, 0, boundary=bnd, reduction="sum",
+                                     return_grad=True)
+    return gx, gy, bnd
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_window_sums_follow_torch_cpu_order(dtype):
+    """The restatement of torch.sum's order over the window axis (what decides near-ties
+    between window starts once s_range exceeds 16) against torch.sum itself, on one thread
+    and with frame counts that fill whole SIMD vectors, where torch.sum has no differently
+    summed tail; and the prune ranges that follow from either."""
+    threads = torch.get_num_threads()
+    torch.set_num_threads(1)
+    try:
+        for n_case, (B, S, T, R) in enumerate([(2, 30, 64, 5), (2, 30, 64, 16), (2, 30, 64, 17),
+                                               (3, 69, 128, 19), (2, 80, 64, 33), (1, 300, 64, 70),
+                                               (1, 700, 64, 300), (1, 600, 64, 513),
+                                               (1, 5000, 64, 4500)]):
+            g = torch.Generator().manual_seed(n_case)
+            py = torch.rand(B, S + 1, T, generator=g, dtype=dtype) ** 3
+            n = S + 2 - R
+            sb, ss, st = py.stride()
+            want = torch.sum(torch.as_strided(py, (B, n, R, T), (sb, ss, ss, st)), axis=2)
+            got = losses.window_sums_in_torch_cpu_order(py, n, R)
+            assert torch.equal(got, want), (B, S, T, R)
+            if R <= 16:
+                ltr = py[:, 0:n, :].clone()
+                for j in range(1, R):
+                    ltr = ltr + py[:, j:j + n, :]
+                assert torch.equal(got, ltr)
+        for seed, (B, S, T) in enumerate([(3, 69, 128), (2, 100, 64)]):
+            gx, gy, bnd = _occupancies(40 + seed, B, S, T, 12, dtype)
+            for R in (17, 19, 33, 40):
+                a = losses.prune_ranges(gx, gy, bnd, R)
+                b = losses.prune_ranges(gx, gy, bnd, R, window_sum="cascade")
+                assert torch.equal(a, b), (B, S, T, R)
+    finally:
+        torch.set_num_threads(threads)
