@@ -37,8 +37,8 @@ _SIGNATURES = {
     "frnnt_simple_logprobs_bwd_noalloc_f32": ([_P] * 8 + [_I, _D] + [_P] * 4 + [_I] * 7 + [_P], _I),
     "frnnt_smoothed_logprobs_fwd_f32": ([_P] * 14 + [_I] * 6 + [_D, _D, _P], _I),
     "frnnt_smoothed_logprobs_fwd_f64": ([_P] * 14 + [_I] * 6 + [_D, _D, _P], _I),
-    "frnnt_smoothed_logprobs_bwd_f32": ([_P] * 20 + [_I] * 6 + [_D, _D, _P], _I),
-    "frnnt_smoothed_logprobs_bwd_f64": ([_P] * 20 + [_I] * 6 + [_D, _D, _P], _I),
+    "frnnt_smoothed_logprobs_bwd_f32": ([_P] * 21 + [_I] * 6 + [_D, _D, _P], _I),
+    "frnnt_smoothed_logprobs_bwd_f64": ([_P] * 21 + [_I] * 6 + [_D, _D, _P], _I),
     "frnnt_simple_loss_fwd_f32": ([_P] * 14 + [_I] * 7 + [_P], _I),
     "frnnt_simple_loss_fwd_f64": ([_P] * 14 + [_I] * 7 + [_P], _I),
     "frnnt_mi_loss_fwd_f32": ([_P] * 8 + [_I] * 5 + [_P], _I),

@@ -241,9 +241,14 @@ __global__ void __launch_bounds__(256)
 // Row sums rx, ry (one wave per lattice row; rx over all T1 columns) and column sums
 // cy = sum_s gy, G = sum_s (gx + gy) over the frames (64 frames per block, waves split
 // the rows); also the gradients of the joint inputs, k * (gx, gy).
+// t_masks (optional): per utterance the frame whose px the forward kernel set to -inf for
+// the regular lattice; like the reference's scatter_ there (rnnt_loss.py:45-63) that cuts
+// the gradient, whatever the recursion left in px_grad at those cells (1 when no path
+// exists at all, 0 otherwise).
 template <typename R>
 __global__ void __launch_bounds__(256)
     smoothed_bwd_sums_kernel(const R *__restrict__ gpx, const R *__restrict__ gpy,
+                             const int64_t *__restrict__ boundary,
                              R *__restrict__ gxj, R *__restrict__ gyj, R *__restrict__ row_x,
                              R *__restrict__ row_y, R *__restrict__ col_y, R *__restrict__ col_g,
                              int B, int S, int T, int T1, R k_joint) {
@@ -256,11 +261,12 @@ __global__ void __launch_bounds__(256)
     const long row = (long)blockIdx.x * 4 + wave;
     if (row >= n_rows) return;
     const int b = (int)(row / S1), s = (int)(row % S1);
+    const int t_mask = boundary ? (int)boundary[4 * b + 3] : -1;
     R sx = 0, sy = 0;
     if (s < S) {
       const long o = ((long)b * S + s) * T1;
       for (int t = lane; t < T1; t += kWave) {
-        const R v = gpx[o + t];
+        const R v = t == t_mask ? (R)0 : gpx[o + t];
         gxj[o + t] = v * k_joint;
         sx += v;
       }
@@ -282,11 +288,12 @@ __global__ void __launch_bounds__(256)
     const long cb = blockIdx.x - row_blocks;
     const int b = (int)(cb / tiles), t = (int)(cb % tiles) * kWave + lane;
     const bool ok = t < T;
+    const bool masked = boundary && boundary[4 * b + 3] == t;
     R ax = 0, ay = 0;
     for (int s = wave; s < S1; s += 4) {
       if (ok) {
         ay += gpy[((long)b * S1 + s) * T + t];
-        if (s < S) ax += gpx[((long)b * S + s) * T1 + t];
+        if (s < S && !masked) ax += gpx[((long)b * S + s) * T1 + t];
       }
     }
     part[0][wave][lane] = ax;
@@ -422,8 +429,10 @@ __global__ void __launch_bounds__(256)
 template <typename R>
 __global__ void __launch_bounds__(256)
     smoothed_bwd_symbols_kernel(const R *__restrict__ gpx, const int64_t *__restrict__ symbols,
-                                R *__restrict__ am_grad, int S, int T, int T1, int C, R k_am) {
+                                const int64_t *__restrict__ boundary, R *__restrict__ am_grad,
+                                int S, int T, int T1, int C, R k_am) {
   const int b = blockIdx.x / S, s = blockIdx.x % S;
+  const int t_mask = boundary ? (int)boundary[4 * b + 3] : -1;
   const int64_t *sym_b = symbols + (long)b * S;
   const int64_t sym = sym_b[s];
   if (sym < 0 || sym >= C) return;
@@ -432,7 +441,7 @@ __global__ void __launch_bounds__(256)
   for (int t = threadIdx.x; t < T; t += 256) {
     R acc = 0;
     for (int k = s; k < S; ++k)
-      if (sym_b[k] == sym) acc += gpx[((long)b * S + k) * T1 + t];
+      if (sym_b[k] == sym && t != t_mask) acc += gpx[((long)b * S + k) * T1 + t];
     am_grad[((long)b * T + t) * C + sym] += k_am * acc;
   }
 }
@@ -453,8 +462,8 @@ __global__ void __launch_bounds__(256)
                                const R *__restrict__ am_z, const R *__restrict__ unigram,
                                const R *__restrict__ col_y, const R *__restrict__ col_g,
                                const R *__restrict__ gpx, const int64_t *__restrict__ symbols,
-                               R *__restrict__ am_grad, long rows, int S, int T, int T1, int C,
-                               int term, R k_am) {
+                               const int64_t *__restrict__ boundary, R *__restrict__ am_grad,
+                               long rows, int S, int T, int T1, int C, int term, R k_am) {
   extern __shared__ __align__(16) unsigned char sym_lds[];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // in a scalar register
   const long row = (long)blockIdx.x * 4 + wave;
@@ -463,6 +472,7 @@ __global__ void __launch_bounds__(256)
   R *extra = reinterpret_cast<R *>(sym_lds) + (size_t)wave * C;
   int *first = reinterpret_cast<int *>(sym_lds + (size_t)4 * C * sizeof(R)) + (size_t)wave * C;
   const int b = (int)(row / T), t = (int)(row % T);
+  const bool masked = boundary && boundary[4 * b + 3] == t;  // (wave-uniform)
   int sym[kSymRowsPerLane];
   R gx[kSymRowsPerLane];
 #pragma unroll
@@ -470,7 +480,7 @@ __global__ void __launch_bounds__(256)
     const int s = q * kWave + lane;
     const int64_t y = s < S ? symbols[(long)b * S + s] : -1;
     sym[q] = (y >= 0 && y < C) ? (int)y : -1;
-    gx[q] = s < S ? gpx[((long)b * S + s) * T1 + t] : (R)0;
+    gx[q] = (s < S && !masked) ? gpx[((long)b * S + s) * T1 + t] : (R)0;
   }
   for (int c = lane; c < C; c += kWave) {
     extra[c] = 0;
@@ -547,7 +557,8 @@ int fwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
 }
 
 template <typename R>
-int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const R *lm_max, const R *lm_sum,
+int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *boundary,
+             const R *lm_max, const R *lm_sum,
              const R *am_max, const R *am_z, const R *unigram, const R *px_grad, const R *py_grad,
              R *pxj_grad, R *pyj_grad, R *lm_grad, R *am_grad, R *row_x, R *row_y, R *col_y,
              R *col_g, R *g_unigram, R *partial, int B, int S, int T, int C, int term, int regular,
@@ -565,10 +576,11 @@ int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const R *lm_max, 
   const long n_lm = (long)B * (S + 1), n_am = (long)B * T;
   const R k_lm = (R)lm_only_scale, k_am = (R)am_only_scale;
   const R k_joint = (R)(1.0 - lm_only_scale - am_only_scale);
+  const int64_t *t_masks = regular ? boundary : nullptr;
   const long sums_blocks = (n_lm + 3) / 4 + (long)B * ((T + kWave - 1) / kWave);
   hipLaunchKernelGGL(smoothed_bwd_sums_kernel<R>, dim3((unsigned)sums_blocks), dim3(256), 0, stream,
-                     px_grad, py_grad, pxj_grad, pyj_grad, row_x, row_y, col_y, col_g, B, S, T, T1,
-                     k_joint);
+                     px_grad, py_grad, t_masks, pxj_grad, pyj_grad, row_x, row_y, col_y, col_g, B, S,
+                     T, T1, k_joint);
   const int blocks = (int)((n_am + kRowsPerBlock - 1) / kRowsPerBlock);
   if (n_am > 0)
     hipLaunchKernelGGL(weighted_column_partial_kernel<R>, dim3(blocks), dim3(256), 0, stream, am,
@@ -586,14 +598,14 @@ int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const R *lm_max, 
         allow_lds(reinterpret_cast<const void *>(smoothed_bwd_am_sym_kernel<R>), sym_lds)) {
       hipLaunchKernelGGL(smoothed_bwd_am_sym_kernel<R>, dim3((unsigned)((n_am + 3) / 4)), dim3(256),
                          sym_lds, stream, am, am_max, am_z, unigram, col_y, col_g, px_grad, symbols,
-                         am_grad, n_am, S, T, T1, C, term, k_am);
+                         t_masks, am_grad, n_am, S, T, T1, C, term, k_am);
     } else {
       hipLaunchKernelGGL(smoothed_bwd_am_kernel<R>, dim3((unsigned)((n_am + 3) / 4)), dim3(256), 0,
                          stream, am, am_max, am_z, unigram, col_y, col_g, am_grad, n_am, C, term,
                          k_am);
       if (S > 0)
         hipLaunchKernelGGL(smoothed_bwd_symbols_kernel<R>, dim3((unsigned)(B * S)), dim3(256), 0,
-                           stream, px_grad, symbols, am_grad, S, T, T1, C, k_am);
+                           stream, px_grad, symbols, t_masks, am_grad, S, T, T1, C, k_am);
     }
   }
   return check_launch("smoothed_logprobs_bwd");
@@ -627,7 +639,7 @@ int frnnt_smoothed_logprobs_fwd_f64(const double *lm, const double *am, const in
                                  regular, lm_only_scale, am_only_scale, stream);
 }
 int frnnt_smoothed_logprobs_bwd_f32(const float *lm, const float *am, const int64_t *symbols,
-                                    const float *lm_max, const float *lm_sum, const float *am_max,
+                                    const int64_t *boundary, const float *lm_max, const float *lm_sum, const float *am_max,
                                     const float *am_z, const float *unigram, const float *px_grad,
                                     const float *py_grad, float *px_joint_grad,
                                     float *py_joint_grad, float *lm_grad, float *am_grad,
@@ -635,13 +647,13 @@ int frnnt_smoothed_logprobs_bwd_f32(const float *lm, const float *am, const int6
                                     float *g_unigram, float *partial, int B, int S, int T, int C,
                                     int termination_symbol, int regular, double lm_only_scale,
                                     double am_only_scale, void *stream) {
-  return frnnt::bwd_impl<float>(lm, am, symbols, lm_max, lm_sum, am_max, am_z, unigram, px_grad,
+  return frnnt::bwd_impl<float>(lm, am, symbols, boundary, lm_max, lm_sum, am_max, am_z, unigram, px_grad,
                                 py_grad, px_joint_grad, py_joint_grad, lm_grad, am_grad, row_x,
                                 row_y, col_y, col_g, g_unigram, partial, B, S, T, C,
                                 termination_symbol, regular, lm_only_scale, am_only_scale, stream);
 }
 int frnnt_smoothed_logprobs_bwd_f64(const double *lm, const double *am, const int64_t *symbols,
-                                    const double *lm_max, const double *lm_sum,
+                                    const int64_t *boundary, const double *lm_max, const double *lm_sum,
                                     const double *am_max, const double *am_z,
                                     const double *unigram, const double *px_grad,
                                     const double *py_grad, double *px_joint_grad,
@@ -650,7 +662,7 @@ int frnnt_smoothed_logprobs_bwd_f64(const double *lm, const double *am, const in
                                     double *g_unigram, double *partial, int B, int S, int T, int C,
                                     int termination_symbol, int regular, double lm_only_scale,
                                     double am_only_scale, void *stream) {
-  return frnnt::bwd_impl<double>(lm, am, symbols, lm_max, lm_sum, am_max, am_z, unigram, px_grad,
+  return frnnt::bwd_impl<double>(lm, am, symbols, boundary, lm_max, lm_sum, am_max, am_z, unigram, px_grad,
                                  py_grad, px_joint_grad, py_joint_grad, lm_grad, am_grad, row_x,
                                  row_y, col_y, col_g, g_unigram, partial, B, S, T, C,
                                  termination_symbol, regular, lm_only_scale, am_only_scale, stream);

@@ -764,8 +764,9 @@ class _SmoothedCombine(torch.autograd.Function):
     def forward(ctx, pxj, pyj, lm, am, symbols, boundary, termination_symbol, regular, k_lm,
                 k_am):
         # boundary (regular lattice): px[b, :, t_end] = -inf, the reference's
-        # fix_for_boundary after the interpolation (rnnt_loss.py:1364-1365); the gradient
-        # the recursion returns for those cells is zero, so backward() has nothing to mask
+        # fix_for_boundary after the interpolation (rnnt_loss.py:1364-1365); backward() lets
+        # no gradient through those cells, as the scatter_ there does (the recursion leaves
+        # 1 in px_grad at them when the lattice has no path at all)
         B, T, C = am.shape
         S = lm.shape[1] - 1
         sfx = _lib.suffix(am.dtype)
@@ -790,6 +791,7 @@ class _SmoothedCombine(torch.autograd.Function):
                       partial.data_ptr(), B, S, T, C, int(termination_symbol), int(regular),
                       k_lm, k_am, _lib.stream_of(am))
         ctx.save_for_backward(lm_c, am_c, sym_c, stats)
+        ctx.masked_at = bnd_c
         ctx.meta = (B, S, T, C, int(termination_symbol), int(regular), k_lm, k_am, sfx,
                     (o_lmx, o_lms, o_amx, o_amz, o_u))
         return px, py
@@ -812,7 +814,8 @@ class _SmoothedCombine(torch.autograd.Function):
             scratch = torch.empty(total, **opts)
             sb, wb, item = scratch.data_ptr(), stats.data_ptr(), stats.element_size()
             _lib.call("frnnt_smoothed_logprobs_bwd_" + sfx, lm.data_ptr(), am.data_ptr(),
-                      sym.data_ptr(), wb + o_lmx * item, wb + o_lms * item, wb + o_amx * item,
+                      sym.data_ptr(), _lib.ptr(ctx.masked_at), wb + o_lmx * item,
+                      wb + o_lms * item, wb + o_amx * item,
                       wb + o_amz * item, wb + o_u * item, gpx.data_ptr(), gpy.data_ptr(),
                       gxj.data_ptr(), gyj.data_ptr(), lm_grad.data_ptr(), am_grad.data_ptr(),
                       sb + o_rx * item, sb + o_ry * item, sb + o_cy * item, sb + o_cg * item,
@@ -825,7 +828,6 @@ def get_rnnt_logprobs_smoothed(
     lm: Tensor, am: Tensor, symbols: Tensor, termination_symbol: int,
     lm_only_scale: float = 0.1, am_only_scale: float = 0.1,
     boundary: Optional[Tensor] = None, rnnt_type: str = "regular",
-    _mask_in_kernel: bool = False,
 ) -> Tuple[Tensor, Tensor]:
     """(px, py) interpolating the joint model with an lm-only and an am-only
     (unigram-lm) model (rnnt_loss.py:1135-1369)::
@@ -858,20 +860,15 @@ def get_rnnt_logprobs_smoothed(
         lm_only_scale = 1.0e-20
     if am_only_scale == 0.0:
         am_only_scale = 1.0e-20
-    # _mask_in_kernel (rnnt_loss_smoothed): the caller feeds (px, py) to the recursion with
-    # this boundary, whose gradient at the cells fix_for_boundary sets to -inf is zero -- the
-    # kernel then writes those -inf itself and no masking node is needed on the way back.
-    # The public helper keeps the reference's scatter_, whose backward zeroes whatever
-    # gradient a caller sends in there.
-    fused_mask = _mask_in_kernel and rnnt_type == "regular" and boundary is not None
+    # fix_for_boundary (rnnt_loss.py:1364-1365) happens inside the node for the regular
+    # lattice: its forward kernel writes the -inf of px[b, :, t_end], its backward kernels let
+    # no gradient through those cells -- what the reference's in-place scatter_ does in both
+    # directions, without the three launches and the index tensor.
     px_interp, py_interp = _SmoothedCombine.apply(
-        px, py, lm, am, symbols, boundary if fused_mask else None, termination_symbol,
-        rnnt_type == "regular", float(lm_only_scale), float(am_only_scale))
+        px, py, lm, am, symbols, boundary if rnnt_type == "regular" else None,
+        termination_symbol, rnnt_type == "regular", float(lm_only_scale), float(am_only_scale))
 
-    if rnnt_type == "regular":
-        if not fused_mask:
-            px_interp = fix_for_boundary(px_interp, boundary)
-    elif rnnt_type == "constrained":
+    if rnnt_type == "constrained":
         px_interp += py_interp[:, 1:, :]
     return (px_interp, py_interp)
 
@@ -886,6 +883,6 @@ def rnnt_loss_smoothed(
     px, py = get_rnnt_logprobs_smoothed(
         lm=lm, am=am, symbols=symbols, termination_symbol=termination_symbol,
         lm_only_scale=lm_only_scale, am_only_scale=am_only_scale, boundary=boundary,
-        rnnt_type=rnnt_type, _mask_in_kernel=True)
+        rnnt_type=rnnt_type)
     return _recursion_and_reduce(px, py, boundary, rnnt_type, delay_penalty, reduction,
                                  return_grad)

@@ -202,9 +202,10 @@ int frnnt_simple_logprobs_bwd_noalloc_f32(const float *lm, const float *am, cons
  * with l = lm_only_scale, a = am_only_scale, the lm-only model log_softmax(lm) and the
  * am-only model am + log(unigram) normalised per frame, unigram = mean over all
  * (b, s) of softmax(lm[b,s,:]) + tiny.  With a boundary (regular lattice) px[b][:][t_end] is
- * set to -inf after the interpolation (fix_for_boundary, rnnt_loss.py:1364-1365; the
- * gradient that comes back for those cells is zero, so the backward entry point needs
- * nothing for it); the constrained "px += py[:, 1:]" step is left to the caller.
+ * set to -inf after the interpolation (fix_for_boundary, rnnt_loss.py:1364-1365); the
+ * backward entry point then takes the same boundary and lets no gradient through those
+ * cells, as the reference's scatter_ does (px_grad holds 1 there when the lattice has no
+ * path at all; NULL when the caller masks outside); the constrained "px += py[:, 1:]" step is left to the caller.
  *   lm_max, lm_sum [B][S+1], am_max, am_z [B][T], unigram [C]: out, kept for the backward
  *   partial [ceil(B*(S+1)/16)][C] (forward), [ceil(B*T/16)][C] (backward): scratch
  * Backward: px_grad / py_grad are the gradients of px / py; out are the gradients of
@@ -225,7 +226,7 @@ int frnnt_smoothed_logprobs_fwd_f64(const double *lm, const double *am, const in
                                     int T, int C, int termination_symbol, int regular,
                                     double lm_only_scale, double am_only_scale, void *stream);
 int frnnt_smoothed_logprobs_bwd_f32(const float *lm, const float *am, const int64_t *symbols,
-                                    const float *lm_max, const float *lm_sum, const float *am_max,
+                                    const int64_t *boundary, const float *lm_max, const float *lm_sum, const float *am_max,
                                     const float *am_z, const float *unigram, const float *px_grad,
                                     const float *py_grad, float *px_joint_grad,
                                     float *py_joint_grad, float *lm_grad, float *am_grad,
@@ -234,7 +235,7 @@ int frnnt_smoothed_logprobs_bwd_f32(const float *lm, const float *am, const int6
                                     int termination_symbol, int regular, double lm_only_scale,
                                     double am_only_scale, void *stream);
 int frnnt_smoothed_logprobs_bwd_f64(const double *lm, const double *am, const int64_t *symbols,
-                                    const double *lm_max, const double *lm_sum,
+                                    const int64_t *boundary, const double *lm_max, const double *lm_sum,
                                     const double *am_max, const double *am_z,
                                     const double *unigram, const double *px_grad,
                                     const double *py_grad, double *px_joint_grad,

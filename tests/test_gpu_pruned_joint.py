@@ -605,6 +605,90 @@ def test_smoothed_loss_equals_helper_then_recursion(gpu_device, kind):
         assert _close(x, y, 1e-12, 1e-12)
 
 
+@pytest.mark.parametrize("which", ["simple", "smoothed", "joint", "pruned"])
+def test_windows_without_a_path(gpu_device, which):
+    """Boundary rows that leave no alignment: an empty range of frames behind a symbol range
+    that is not (regular lattice: the -inf column is all there is to emit on), or none of
+    either.  The loss is +inf or finite as in the reference, and the gradients that reach
+    the inputs are the reference's -- the recursion leaves 1, not 0, in px_grad at the
+    masked cells of a lattice without a path, which the -inf masking must not let through
+    (rnnt_loss.py:45-63: scatter_ cuts the gradient)."""
+    dev = gpu_device
+    B, S, T, C, R = 4, 12, 20, 9, 4
+    g = torch.Generator().manual_seed(77)
+    am = torch.randn(B, T, C, generator=g, dtype=torch.float64)
+    lm = torch.randn(B, S + 1, C, generator=g, dtype=torch.float64)
+    sym = torch.randint(0, C, (B, S), generator=g)
+    bnd = torch.tensor([[2, 1, 9, 1], [0, 0, 12, 20], [3, 5, 3, 5], [0, 7, 6, 7]])
+    start = torch.clamp(torch.arange(T) * (S + 1 - R) // (T - 1), 0, S + 1 - R)
+    ranges = (start.reshape(1, T, 1) + torch.arange(R).reshape(1, 1, R)).expand(B, T, R).contiguous()
+    w = torch.tensor([1.0, 0.5, -2.0, 0.25], dtype=torch.float64)
+
+    def run(fns, to):
+        a = to(am).requires_grad_(True)
+        l = to(lm).requires_grad_(True)
+        kw = dict(boundary=to(bnd), reduction="none", return_grad=True)
+        if which == "simple":
+            loss, (gx, gy) = fns[0](l, a, to(sym), 0, **kw)
+        elif which == "smoothed":
+            loss, (gx, gy) = fns[1](l, a, to(sym), 0, 0.2, 0.1, **kw)
+        elif which == "joint":
+            loss, (gx, gy) = fns[2](torch.tanh(a.unsqueeze(2) + l.unsqueeze(1)), to(sym), 0, **kw)
+        else:
+            rg = to(ranges)
+            lp = torch.gather(l.unsqueeze(1).expand(B, T, S + 1, C), 2,
+                              rg.unsqueeze(3).expand(B, T, R, C))
+            loss, (gx, gy) = fns[3](torch.tanh(a.unsqueeze(2) + lp), to(sym), rg, 0, **kw)
+        occ = gx.detach().clone(), gy.detach().clone()
+        # (utterances without a path have an infinite loss; their gradients still flow)
+        (torch.where(torch.isfinite(loss), loss, torch.zeros_like(loss)) * to(w)).sum().backward()
+        return loss.detach(), occ, a.grad, l.grad
+
+    want = run((O.loss_simple, O.loss_smoothed, O.loss_joint, O.loss_pruned), lambda x: x.clone())
+    got = run((fast_rnnt_amd.rnnt_loss_simple, fast_rnnt_amd.rnnt_loss_smoothed,
+               fast_rnnt_amd.rnnt_loss, fast_rnnt_amd.rnnt_loss_pruned), lambda x: x.to(dev))
+    _say(f"no path {which}: losses {want[0].tolist()}")
+    assert torch.isinf(want[0][0]) and torch.isfinite(want[0][1])
+    assert _close(got[0], want[0], 0.0, 1e-9)
+    assert _close(got[1][0], want[1][0], 1e-9) and _close(got[1][1], want[1][1], 1e-9)
+    assert _close(got[2], want[2], 1e-9, 1e-9) and _close(got[3], want[3], 1e-9, 1e-9)
+
+
+@pytest.mark.parametrize("which", ["simple", "smoothed", "joint"])
+def test_gradient_of_a_loss_without_a_path(gpu_device, which):
+    """The same with the infinite losses left in the sum: their utterances' occupation
+    gradients (1 at the masked cells) are scaled and passed back like any others, and must
+    stop where the reference's scatter_ stops them."""
+    dev = gpu_device
+    B, S, T, C = 2, 10, 16, 7
+    g = torch.Generator().manual_seed(78)
+    am = torch.randn(B, T, C, generator=g, dtype=torch.float64)
+    lm = torch.randn(B, S + 1, C, generator=g, dtype=torch.float64)
+    sym = torch.randint(0, C, (B, S), generator=g)
+    bnd = torch.tensor([[2, 1, 9, 1], [0, 0, 10, 16]])
+    res = []
+    for gpu_side in (False, True):
+        to = (lambda x: x.to(dev)) if gpu_side else (lambda x: x.clone())
+        a = to(am).requires_grad_(True)
+        l = to(lm).requires_grad_(True)
+        kw = dict(boundary=to(bnd), reduction="none")
+        if which == "simple":
+            f = fast_rnnt_amd.rnnt_loss_simple if gpu_side else O.loss_simple
+            loss = f(l, a, to(sym), 0, **kw)
+        elif which == "smoothed":
+            f = fast_rnnt_amd.rnnt_loss_smoothed if gpu_side else O.loss_smoothed
+            loss = f(l, a, to(sym), 0, 0.2, 0.1, **kw)
+        else:
+            f = fast_rnnt_amd.rnnt_loss if gpu_side else O.loss_joint
+            loss = f(a.unsqueeze(2) + l.unsqueeze(1), to(sym), 0, **kw)
+        loss.backward(torch.ones_like(loss))
+        res.append((loss.detach(), a.grad, l.grad))
+    _say(f"infinite loss {which}: {res[0][0].tolist()}")
+    assert torch.isinf(res[0][0][0])
+    for x, y in zip(res[1], res[0]):
+        assert _close(x, y, 1e-9, 1e-9)
+
+
 def test_c5_unpruned_full_size(gpu_device):
     dev = gpu_device
     w = workloads.make("c5")
