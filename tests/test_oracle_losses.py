@@ -213,12 +213,14 @@ def test_golden_smoothed_logprobs():
         px, py = losses.lattice_logprobs_smoothed(
             c["lm"], c["am"], c["symbols"], 0, c["lm_only_scale"], c["am_only_scale"],
             boundary=c["boundary"], rnnt_type=c["kind"])
-        assert torch.equal(px, c["px"]), name
-        assert torch.equal(py, c["py"]), name
+        # (bit for bit on the host that wrote the vectors; torch's matmul and logsumexp add in
+        # an order that depends on the host's thread count, hence the last-bit tolerance)
+        assert torch.allclose(px, c["px"], rtol=2e-6, atol=2e-6), name
+        assert torch.allclose(py, c["py"], rtol=2e-6, atol=2e-6), name
         loss = losses.loss_smoothed(
             c["lm"], c["am"], c["symbols"], 0, c["lm_only_scale"], c["am_only_scale"],
             boundary=c["boundary"], rnnt_type=c["kind"], reduction="none")
-        assert torch.equal(loss, c["loss"]), name
+        assert torch.allclose(loss, c["loss"], rtol=2e-6, atol=0), name
 
 
 def test_golden_prune_ranges(capsys):
@@ -235,7 +237,9 @@ def test_golden_prune_ranges(capsys):
             px, py = losses.lattice_logprobs_pruned(
                 c["logits"], c["symbols"], c["ranges"], 0, boundary=c["boundary"],
                 rnnt_type=c["kind"])
-            assert torch.equal(px, c["px"]) and torch.equal(py, c["py"]), name
+            # (last-bit tolerance: logsumexp's summation order follows the host's threads)
+            assert torch.allclose(px, c["px"], rtol=2e-6, atol=2e-6), name
+            assert torch.allclose(py, c["py"], rtol=2e-6, atol=2e-6), name
     assert "Adjusting to 4" in capsys.readouterr().out
     assert data["ties"]["ranges"][0, :, 0].tolist()[0] == 0
 
