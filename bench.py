@@ -385,7 +385,7 @@ def _bench_lattice(args, w, dev):
                                                               4)}
 
     replay = None
-    if args.graph and w.name == "c5":
+    if args.graph:
         replay = _graph_replay(step, grads, args)
 
     # the two logits kernels alone, through the C ABI, with events on the launch stream; as
