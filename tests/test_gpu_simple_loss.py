@@ -288,12 +288,15 @@ def test_baseline_configs(gpu_device, name):
         assert _close(da.grad, a.grad, bound, 1e-4) and _close(dl.grad, l.grad, bound, 1e-4)
 
 
-@pytest.mark.parametrize("shape", [(3, 80, 250, 500), (2, 100, 130, 96), (2, 7, 9, 5)])
-def test_gradient_products_together_and_apart(gpu_device, shape):
+@pytest.mark.parametrize("ragged", [False, True])
+@pytest.mark.parametrize("shape", [(3, 80, 250, 500), (2, 100, 130, 96), (2, 7, 9, 5),
+                                   (2, 20, 130, 2100), (3, 100, 200, 2048), (2, 127, 70, 2500)])
+def test_gradient_products_together_and_apart(gpu_device, shape, ragged):
     # frnnt_simple_logprobs_bwd forms lm.grad and am.grad in one launch while the products
     # are short, and in two launches when only one of them is asked for: the same tiles,
     # so am.grad must come out bit for bit the same, and lm.grad (whose tiles take the
-    # frames in shorter slabs inside the common launch) to rounding.
+    # frames in shorter slabs inside the common launch) to rounding.  ragged: boundary
+    # windows, and nothing computed outside them.
     from fast_rnnt_amd import _lib
     dev = gpu_device
     B, S, T, C = shape
@@ -302,7 +305,13 @@ def test_gradient_products_together_and_apart(gpu_device, shape):
     lm = torch.randn(B, S + 1, C, generator=g).to(dev)
     am = torch.randn(B, T, C, generator=g).to(dev)
     sym = torch.randint(0, C, (B, S), generator=g).to(dev)
-    bnd = torch.tensor([[0, 0, S, T]] * B, dtype=torch.int64).to(dev)
+    if ragged:
+        bnd = torch.stack([torch.zeros(B, dtype=torch.int64), torch.zeros(B, dtype=torch.int64),
+                           torch.randint(max(1, S // 2), S + 1, (B,), generator=g),
+                           torch.randint(max(1, T // 3), T + 1, (B,), generator=g)], 1).to(dev)
+    else:
+        bnd = torch.tensor([[0, 0, S, T]] * B, dtype=torch.int64).to(dev)
+    window_only = int(ragged)
     px, py = torch.empty(B, S, T + 1, **f32), torch.empty(B, S + 1, T, **f32)
     lm_max, am_max = torch.empty(B, S + 1, **f32), torch.empty(B, T, **f32)
     norm_raw = torch.empty(B, S + 1, T, **f32)
@@ -310,9 +319,15 @@ def test_gradient_products_together_and_apart(gpu_device, shape):
     _say(f"gradient products B={B} S={S} T={T} C={C}")
     _lib.call("frnnt_simple_logprobs_fwd_f32", lm.data_ptr(), am.data_ptr(), sym.data_ptr(),
               bnd.data_ptr(), px.data_ptr(), py.data_ptr(), lm_max.data_ptr(), am_max.data_ptr(),
-              norm_raw.data_ptr(), B, S, T, C, 0, 0, 0, stream)
+              norm_raw.data_ptr(), B, S, T, C, 0, 0, window_only, stream)
     gpx = torch.rand(B, S, T + 1, generator=g).to(dev)
     gpy = torch.rand(B, S + 1, T, generator=g).to(dev)
+    if ragged:  # what the recursion leaves outside a window: exact zeros
+        rows = torch.arange(S + 1, device=dev).reshape(1, S + 1, 1)
+        cols = torch.arange(T + 1, device=dev).reshape(1, 1, T + 1)
+        s_end, t_end = bnd[:, 2].reshape(B, 1, 1), bnd[:, 3].reshape(B, 1, 1)
+        gpx *= ((rows[:, :S] < s_end) & (cols <= t_end)).float()
+        gpy *= ((rows <= s_end) & (cols[:, :, :T] < t_end)).float()
     dmat = torch.empty(B, S + 1, (T + 3) // 4 * 4, **f32)
     row_x, row_y = torch.empty(B, S + 1, **f32), torch.empty(B, S + 1, **f32)
     col_y = torch.empty(B, T, **f32)
@@ -324,7 +339,7 @@ def test_gradient_products_together_and_apart(gpu_device, shape):
                   bnd.data_ptr(), lm_max.data_ptr(), am_max.data_ptr(), norm_raw.data_ptr(), None,
                   0, 1.0, gpx.data_ptr(), gpy.data_ptr(), dmat.data_ptr(), row_x.data_ptr(),
                   row_y.data_ptr(), col_y.data_ptr(), _lib.ptr(lm_grad), _lib.ptr(am_grad), B, S,
-                  T, C, 0, 0, 0, stream)
+                  T, C, 0, 0, window_only, stream)
         torch.cuda.synchronize()
         return lm_grad, am_grad
 
