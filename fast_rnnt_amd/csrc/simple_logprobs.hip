@@ -609,7 +609,14 @@ __global__ void __launch_bounds__(kPanThreads)
     for (int off = 1; off < kRowLanes; off <<= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
     return v;
   };
-  auto raise_shifts = [&]() {
+  // (sums_are_zero: the wave's first slab, which always comes here -- nothing to scale yet)
+  auto raise_shifts = [&](bool sums_are_zero) {
+    if (sums_are_zero) {
+#pragma unroll
+      for (int j = 0; j < kLoads; ++j)
+        shift2[j] = fminf(shift2[j], -across_row(seen[j]) * kLog2e);
+      return;
+    }
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
       const float now = fminf(shift2[j], -across_row(seen[j]) * kLog2e);
@@ -628,7 +635,7 @@ __global__ void __launch_bounds__(kPanThreads)
   };
   // one slab: exp(x - shift) to LDS, the request for the slab that will take these
   // registers next, then the products (32-row tiles without lattice rows are skipped)
-  auto consume = [&](floatx4 (&slab)[kLoads], int next_chunk) {
+  auto consume = [&](floatx4 (&slab)[kLoads], int next_chunk, bool first) {
     bool above = false;
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
@@ -636,7 +643,7 @@ __global__ void __launch_bounds__(kPanThreads)
       seen[j] = max3_raw(max3_raw(slab[j][0], slab[j][1], slab[j][2]), slab[j][3], seen[j]);
       above |= __builtin_fmaf(seen[j], kLog2e, shift2[j]) > kMargin * kLog2e;
     }
-    if (__any(above)) raise_shifts();
+    if (__any(above)) raise_shifts(first);
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
       float *d = mine + (sub + kRowsPerLoad * j) * kPanPitch + kq;
@@ -656,7 +663,8 @@ __global__ void __launch_bounds__(kPanThreads)
                                                         0, 0, 0);
     }
   };
-  for (int chunk = wave; chunk < chunks; chunk += kPanWaves) consume(slab, chunk + kPanWaves);
+  for (int chunk = wave; chunk < chunks; chunk += kPanWaves)
+    consume(slab, chunk + kPanWaves, chunk == wave);
 
   // ---- the waves meet: maxima first ...
 #pragma unroll
