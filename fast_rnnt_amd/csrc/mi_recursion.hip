@@ -313,38 +313,48 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
       }
     };
     // p of tile pm of the band that starts at row0, left by the sweep wave in buffer `buf`:
-    // element (row r, step q) is the cell (row0 + r, 32 pm + q - r) of the window.
-    auto drain = [&](int row0, int pm, int buf) {
-      const R *ps = base + buf * kTileElems + r_first * kTilePitch + q;
-      const int i0 = row0 + r_first;
-      const int j0 = pm * kTileSteps + q - r_first;
-      const int o0 = ((win.s0 + i0) * TP + win.t0 + j0) * kSize;
+    // element (row r, step q) is the cell (row0 + r, 32 pm + q - r) of the window.  Taking
+    // it out of the buffer and storing it are two steps: a wave's wait for a load also
+    // waits for every store it has issued before, so the stores of a tile go out after
+    // the buffer has been refilled and handed back to the sweep wave, not before.
+    struct Drained {
       R v[kRows];
+      int row0, pm;
+    };
+    auto take = [&](Drained &d, int row0, int pm, int buf) {
+      const R *ps = base + buf * kTileElems + r_first * kTilePitch + q;
+      d.row0 = row0;
+      d.pm = pm;
 #pragma unroll
       for (int u = 0; u < kRows; ++u) {
         if (r_first + kStep * u >= kWave) continue;
-        v[u] = ps[u * kStep * kTilePitch];
+        d.v[u] = ps[u * kStep * kTilePitch];
       }
+    };
+    auto store = [&](const Drained &d) {
+      const int i0 = d.row0 + r_first;
+      const int j0 = d.pm * kTileSteps + q - r_first;
+      const int o0 = ((win.s0 + i0) * TP + win.t0 + j0) * kSize;
 #pragma unroll
       for (int u = 0; u < kRows; ++u) {
         if (r_first + kStep * u >= kWave) continue;
         const int i = i0 + kStep * u, j = j0 - kStep * u;
         const bool ok = i <= NS && (unsigned)j <= (unsigned)NT;
-        put1(p_rsrc, ok ? o0 + u * (kStep * (TP - 1) * kSize) : kDropped, v[u]);
+        put1(p_rsrc, ok ? o0 + u * (kStep * (TP - 1) * kSize) : kDropped, d.v[u]);
       }
     };
     // which tile each buffer holds: its band's first row and its number in the band
     int held_row0[kBuffers], held_m[kBuffers];
 #pragma unroll
     for (int k = 0; k < kBuffers; ++k) held_row0[k] = held_m[k] = 0;
-    auto drain_buffer = [&](int buf) {
+    auto take_buffer = [&](Drained &d, int buf) {
       int row0 = held_row0[0], pm = held_m[0];
 #pragma unroll
       for (int k = 1; k < kBuffers; ++k) {
         row0 = buf == k ? held_row0[k] : row0;
         pm = buf == k ? held_m[k] : pm;
       }
-      drain(row0, pm, buf);
+      take(d, row0, pm, buf);
     };
     int tile_base = 0, buf = 0;  // buf = tile number modulo kBuffers
     for (int band = 0; band * band_rows <= NS; ++band) {
@@ -354,13 +364,15 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
       fetch(cur, g, 0);
       for (int m = 0; m < g.ntiles; ++m) {
         const int gt = tile_base + m;
-        if (gt >= kBuffers) {
+        Drained out;
+        const bool refill = gt >= kBuffers;
+        if (refill) {
           // the buffer still holds p of tile gt - kBuffers
           if (!wait_for(&cnt.written[w], gt - kBuffers + 1, spin_limit)) {
             give_up();
             return;
           }
-          drain_buffer(buf);
+          take_buffer(out, buf);
         }
 #pragma unroll
         for (int k = 0; k < kBuffers; ++k) {
@@ -389,6 +401,7 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
         }
         // every lane's LDS writes precede the release by lane 0 of the same wave
         if (lane == 0) publish(my_loaded, gt + 1);
+        if (refill) store(out);
         // the next tile's inputs, fetched while this wave waits for its buffer
         if (m + 1 < g.ntiles) fetch(cur, g, m + 1);
         buf = buf + 1 == kBuffers ? 0 : buf + 1;
@@ -403,7 +416,9 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
         give_up();
         return;
       }
-      drain_buffer(buf);
+      Drained out;
+      take_buffer(out, buf);
+      store(out);
       buf = buf + 1 == kBuffers ? 0 : buf + 1;
     }
     return;
@@ -456,9 +471,13 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
       // One chunk of kChunk steps, specialised at compile time on whether the wave
       // receives a seam (kUp) and feeds one (kDown).
       bool alive = true;
-      auto chunk = [&](auto up_c, auto down_c, int c4, int e0) __attribute__((always_inline)) {
+      // kPlain: a tile whose 32 steps all exist and do not hold the answer's step; a single
+      // wave pays for every instruction it issues, scalar tests and branches included, so
+      // such tiles run without the two tests per chunk.
+      auto chunk = [&](auto up_c, auto down_c, auto plain_c, int c4, int e0) __attribute__((always_inline)) {
         constexpr bool kUp = decltype(up_c)::value;
         constexpr bool kDown = decltype(down_c)::value;
+        constexpr bool kPlain = decltype(plain_c)::value;
         R handed = ninf;  // lane k: the seam value lane 0 needs at step e0 + k
         if (kUp) {
           const int need = min(e0 + kChunk - shift, cols);
@@ -501,11 +520,13 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
           own2 = own;
           own = v;
         }
-        const int kf = fin_step - e0;  // wave-uniform
-        if ((unsigned)kf < (unsigned)kChunk) {
+        if (!kPlain) {
+          const int kf = fin_step - e0;  // wave-uniform
+          if ((unsigned)kf < (unsigned)kChunk) {
 #pragma unroll
-          for (int k = 0; k < kChunk; ++k)
-            if (k == kf) fin = vals[k];
+            for (int k = 0; k < kChunk; ++k)
+              if (k == kf) fin = vals[k];
+          }
         }
         // seam: the last lane's columns e0 - 63 ... (the pads take what falls outside)
         if (kDown && e0 + kChunk > kWave - 1) {
@@ -518,23 +539,32 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
         // the chunk's p takes the place of its x in the tile
         push_chunk(x_row + c4 * kChunk, vals);
       };
-      auto tile = [&](auto up_c, auto down_c) __attribute__((always_inline)) {
+      auto tile = [&](auto up_c, auto down_c, auto plain_c) __attribute__((always_inline)) {
 #pragma unroll
         for (int c4 = 0; c4 < kTileSteps / kChunk; ++c4) {
           const int e0 = m * kTileSteps + c4 * kChunk;
-          if (e0 < g.nsteps && (!decltype(up_c)::value || alive)) chunk(up_c, down_c, c4, e0);
+          if ((decltype(plain_c)::value || e0 < g.nsteps) && (!decltype(up_c)::value || alive))
+            chunk(up_c, down_c, plain_c, c4, e0);
         }
+      };
+      auto tile_of = [&](auto up_c, auto down_c) __attribute__((always_inline)) {
+        const bool plain = (m + 1) * kTileSteps <= g.nsteps &&
+                           (unsigned)(fin_step - m * kTileSteps) >= (unsigned)kTileSteps;
+        if (plain)
+          tile(up_c, down_c, std::true_type{});
+        else
+          tile(up_c, down_c, std::false_type{});
       };
       if (has_up) {
         if (has_down)
-          tile(std::true_type{}, std::true_type{});
+          tile_of(std::true_type{}, std::true_type{});
         else
-          tile(std::true_type{}, std::false_type{});
+          tile_of(std::true_type{}, std::false_type{});
       } else {
         if (has_down)
-          tile(std::false_type{}, std::true_type{});
+          tile_of(std::false_type{}, std::true_type{});
         else
-          tile(std::false_type{}, std::false_type{});
+          tile_of(std::false_type{}, std::false_type{});
       }
       if (!alive) {
         give_up();
@@ -701,21 +731,31 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
     // The straight-line form below (every row group handled alike, borders by select) is
     // faster than variants that skip the rows past the window's top or branch to a
     // mask-free copy for tiles inside the window: those were 1 to 5 us slower per launch.
-    auto drain = [&](int pg_row0, int pm, int buf) {
+    // Taking a tile's gradients out of the buffer and storing them are two steps: a wave's
+    // wait for a load also waits for every store it has issued before, so the stores go
+    // out after the buffer has been refilled and handed back to the sweep wave.
+    struct Drained {
+      R vx[kRows], vy[kRows];
+      int row0, pm;
+    };
+    auto take = [&](Drained &d, int pg_row0, int pm, int buf) {
       const R *gxs = base + buf * kTileElems + r_first * kTilePitch + q;
       const R *gys = gxs + kBuffers * kTileElems;
-      constexpr int kMinX = kModified ? 1 : 0;
-      const int i0 = NS - pg_row0 - r_first;                // lattice row of u = 0
-      const int j0 = NT - (pm * kTileSteps + q - r_first);  // and its column
-      const int x0 = ((win.s0 + i0 - 1) * T1 + win.t0 - shift + j0) * kSize;
-      const int y0 = ((win.s0 + i0) * T + win.t0 - 1 + j0) * kSize;
-      R vx[kRows], vy[kRows];
+      d.row0 = pg_row0;
+      d.pm = pm;
 #pragma unroll
       for (int u = 0; u < kRows; ++u) {
         if (r_first + kStep * u >= kWave) continue;
-        vx[u] = gxs[u * kStep * kTilePitch];
-        vy[u] = gys[u * kStep * kTilePitch];
+        d.vx[u] = gxs[u * kStep * kTilePitch];
+        d.vy[u] = gys[u * kStep * kTilePitch];
       }
+    };
+    auto store = [&](const Drained &d) {
+      constexpr int kMinX = kModified ? 1 : 0;
+      const int i0 = NS - d.row0 - r_first;                   // lattice row of u = 0
+      const int j0 = NT - (d.pm * kTileSteps + q - r_first);  // and its column
+      const int x0 = ((win.s0 + i0 - 1) * T1 + win.t0 - shift + j0) * kSize;
+      const int y0 = ((win.s0 + i0) * T + win.t0 - 1 + j0) * kSize;
 #pragma unroll
       for (int u = 0; u < kRows; ++u) {
         if (r_first + kStep * u >= kWave) continue;
@@ -724,22 +764,22 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
         const int i = i0 - kStep * u, j = j0 + kStep * u;
         const bool okx = i > 0 && (unsigned)(j - kMinX) < (unsigned)(NT + 1 - kMinX);
         const bool oky = i >= 0 && (unsigned)(j - 1) < (unsigned)NT;
-        put1(gx_rsrc, okx ? xo : kDropped, vx[u]);
-        put1(gy_rsrc, oky ? yo : kDropped, vy[u]);
+        put1(gx_rsrc, okx ? xo : kDropped, d.vx[u]);
+        put1(gy_rsrc, oky ? yo : kDropped, d.vy[u]);
       }
     };
     // which tile each buffer holds: its band's first row and its number in the band
     int held_row0[kBuffers], held_m[kBuffers];
 #pragma unroll
     for (int k = 0; k < kBuffers; ++k) held_row0[k] = held_m[k] = 0;
-    auto drain_buffer = [&](int buf) {
+    auto take_buffer = [&](Drained &d, int buf) {
       int row0 = held_row0[0], pm = held_m[0];
 #pragma unroll
       for (int k = 1; k < kBuffers; ++k) {
         row0 = buf == k ? held_row0[k] : row0;
         pm = buf == k ? held_m[k] : pm;
       }
-      drain(row0, pm, buf);
+      take(d, row0, pm, buf);
     };
     int tile_base = 0, buf = 0;  // buf = tile number modulo kBuffers
     bool zeroed = false;
@@ -750,13 +790,15 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
       fetch(cur, g, 0);
       for (int m = 0; m < g.ntiles; ++m) {
         const int gt = tile_base + m;
-        if (gt >= kBuffers) {
+        Drained out;
+        const bool refill = gt >= kBuffers;
+        if (refill) {
           // the buffer still holds the gradients of tile gt - kBuffers
           if (!wait_for(&cnt.written[w], gt - kBuffers + 1, spin_limit)) {
             give_up();
             return;
           }
-          drain_buffer(buf);
+          take_buffer(out, buf);
         }
 #pragma unroll
         for (int k = 0; k < kBuffers; ++k) {
@@ -792,6 +834,7 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
         }
         // every lane's LDS writes precede the release by lane 0 of the same wave
         if (lane == 0) publish(my_loaded, gt + 1);
+        if (refill) store(out);
         // the next tile's inputs, fetched while this wave waits for its buffer
         if (m + 1 < g.ntiles) fetch(cur, g, m + 1);
         buf = buf + 1 == kBuffers ? 0 : buf + 1;
@@ -811,7 +854,9 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
         give_up();
         return;
       }
-      drain_buffer(buf);
+      Drained out;
+      take_buffer(out, buf);
+      store(out);
       buf = buf + 1 == kBuffers ? 0 : buf + 1;
     }
     if (!zeroed) zero_outside(wave - nsweep, nwaves - nsweep);
@@ -867,9 +912,11 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
       pull_row(d2q, gy_row);
 
       bool alive = true;
-      auto chunk = [&](auto up_c, auto down_c, int c4, int e0) __attribute__((always_inline)) {
+      // (kPlain: all 32 steps exist and none is the origin's, see the forward kernel)
+      auto chunk = [&](auto up_c, auto down_c, auto plain_c, int c4, int e0) __attribute__((always_inline)) {
         constexpr bool kUp = decltype(up_c)::value;
         constexpr bool kDown = decltype(down_c)::value;
+        constexpr bool kPlain = decltype(plain_c)::value;
         R handed = 0;
         if (kUp) {
           const int need = min(e0 + kChunk - shift, cols);
@@ -912,11 +959,13 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
           to_below = down[k];
           to_left = left[k];
         }
-        const int kf = fin_step - e0;  // wave-uniform
-        if ((unsigned)kf < (unsigned)kChunk) {
+        if (!kPlain) {
+          const int kf = fin_step - e0;  // wave-uniform
+          if ((unsigned)kf < (unsigned)kChunk) {
 #pragma unroll
-          for (int k = 0; k < kChunk; ++k)
-            if (k == kf) g_origin = cell[k];
+            for (int k = 0; k < kChunk; ++k)
+              if (k == kf) g_origin = cell[k];
+          }
         }
         // seam: the last lane's reversed columns e0 - 63 ... (the pads take what falls
         // outside)
@@ -931,24 +980,33 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
         push_chunk(gx_row + c4 * kChunk, down);
         push_chunk(gy_row + c4 * kChunk, left);
       };
-      auto tile = [&](auto up_c, auto down_c) __attribute__((always_inline)) {
+      auto tile = [&](auto up_c, auto down_c, auto plain_c) __attribute__((always_inline)) {
 #pragma unroll
         for (int c4 = 0; c4 < kTileSteps / kChunk; ++c4) {
           const int e0 = m * kTileSteps + c4 * kChunk;
           // the window's edges need no care here: d1 = d2 = 0 outside it
-          if (e0 < g.nsteps && (!decltype(up_c)::value || alive)) chunk(up_c, down_c, c4, e0);
+          if ((decltype(plain_c)::value || e0 < g.nsteps) && (!decltype(up_c)::value || alive))
+            chunk(up_c, down_c, plain_c, c4, e0);
         }
+      };
+      auto tile_of = [&](auto up_c, auto down_c) __attribute__((always_inline)) {
+        const bool plain = (m + 1) * kTileSteps <= g.nsteps &&
+                           (unsigned)(fin_step - m * kTileSteps) >= (unsigned)kTileSteps;
+        if (plain)
+          tile(up_c, down_c, std::true_type{});
+        else
+          tile(up_c, down_c, std::false_type{});
       };
       if (has_up) {
         if (has_down)
-          tile(std::true_type{}, std::true_type{});
+          tile_of(std::true_type{}, std::true_type{});
         else
-          tile(std::true_type{}, std::false_type{});
+          tile_of(std::true_type{}, std::false_type{});
       } else {
         if (has_down)
-          tile(std::false_type{}, std::true_type{});
+          tile_of(std::false_type{}, std::true_type{});
         else
-          tile(std::false_type{}, std::false_type{});
+          tile_of(std::false_type{}, std::false_type{});
       }
       if (!alive) {
         give_up();
