@@ -49,14 +49,14 @@ constexpr int kSeamPad = kChunk;        // slack on either side of a seam row, s
 constexpr int kSeamPadLeft = kSeamPad + 3;
 static_assert((kSeamPadLeft - (kWave - 1)) % 4 == 0, "seam chunks are not 16-byte aligned");
 constexpr int kSeamSlack = kSeamPadLeft + kSeamPad;
-constexpr int kFwdStagers = 2;         // staging waves per sweep wave
+constexpr int kFwdStagers = 3;         // staging waves per sweep wave
 constexpr int kBwdStagers = 3;
-// With at most two sweep waves the backward kernel runs more staging waves per sweep wave:
-// they evaluate d1 / d2 and are what the sweep would otherwise wait for (c2 shape: 22.9 us
-// with 3, 20.6 with 4, 19.3 - 19.6 with 5 to 7).  The forward kernel's staging waves only
-// copy, and more of them slow the sweep waves down (21.4 us with 2, 22.2 with 5, 23.0 with
-// 7 per sweep wave).
-constexpr int kBwdStagersFew = 6;
+// With at most two sweep waves a workgroup has room for more staging waves per sweep wave.
+// The backward kernel's evaluate d1 / d2 and are what its sweep waves wait for (c2 shape:
+// 17.2 us with 6, 16.9 with 7: 16 waves, the most a workgroup holds); the forward kernel's
+// only copy (18.45 us with 2, 18.05 with 3, 17.9 with 4).
+constexpr int kFwdStagersFew = 4;
+constexpr int kBwdStagersFew = 7;
 constexpr int kSpinLimit = 1 << 22;   // polls before a wait gives up (seconds, not microseconds)
 // Set by frnnt_set_spin_limit(): lets a test force the give-up path from the host.
 int g_spin_limit = kSpinLimit;
@@ -100,6 +100,15 @@ __device__ __forceinline__ int peek(const int *counter) {
   const int v = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   asm volatile("" ::: "memory");
   return v;
+}
+// Waits until this wave's LDS reads have arrived.  On the rare path that re-reads the seam
+// it keeps the common path's wait at "the read issued a chunk ago", which the LDS writes
+// issued since then do not hold up (after a join the compiler takes the stricter wait).
+__device__ __forceinline__ void lds_reads_done() {
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0) only
+}
+__device__ __forceinline__ void count_in(int *counter) {
+  __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 __device__ __forceinline__ void publish(int *counter, int value) {
   __hip_atomic_store(counter, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -205,11 +214,35 @@ __device__ __forceinline__ void push_chunk(R *dst, const R (&src)[kChunk]) {
   }
 }
 
+// The first (kHalf = 0) or second half of a chunk into its place in the tile row.  An LDS
+// write takes its data out of the registers over some 30 cycles after it has been issued,
+// and an instruction that overwrites one of them waits for that; so a sweep wave writes
+// the first half of a chunk as soon as it is complete, in the middle of the chunk, and
+// the second half at its end: each half then has four steps' time before the next chunk
+// comes to its registers.
+template <int kHalf, typename R>
+__device__ __forceinline__ void push_half(R *dst, const R (&src)[kChunk]) {
+  constexpr int kPer = 16 / (int)sizeof(R);
+  typedef R Piece __attribute__((ext_vector_type(kPer)));
+  Piece *d = reinterpret_cast<Piece *>(dst);
+#pragma unroll
+  for (int i = kHalf * (kChunk / 2 / kPer); i < (kHalf + 1) * (kChunk / 2 / kPer); ++i) {
+    Piece v;
+#pragma unroll
+    for (int e = 0; e < kPer; ++e) v[e] = src[i * kPer + e];
+    d[i] = v;
+  }
+}
+
 struct Counters {
   int failed;                             // set by a wave whose bounded wait ran out
   int ready[kMaxSweep];                   // seam columns published by sweep wave w
   int written[kMaxSweep];                 // tiles whose results sweep wave w has left in LDS
-  int loaded[16];                         // tiles staged for sweep wave w by its stager l (index w * stagers + l)
+  // per sweep wave w and tile buffer k (index w * buffers + k): how many times a staging
+  // wave has finished staging a tile into that buffer, all of w's staging waves and all
+  // tiles together -- the buffer's n-th tile is complete at n * stagers.  One counter for
+  // all staging waves: a sweep wave pays for every test it makes.
+  int loaded[16];
 };
 
 // Geometry of what sweep wave `w` does in band `band`; identical on the sweep
@@ -224,6 +257,24 @@ __device__ __forceinline__ Band band_of(int band, int w, int nsweep, int NS, int
   g.nsteps = NT + g.nrows;
   g.ntiles = (g.nsteps + kTileSteps - 1) / kTileSteps;
   return g;
+}
+
+// The tiles [lo, hi) of a sweep wave's band that are plain: all 32 steps exist
+// ((m + 1) * 32 <= nsteps), the step that holds the wave's result (fin_step, if any) is not
+// among them and, for a wave with a seam above it, every seam column that the tile and the
+// first chunk after it look at exists (0 <= 32 m - shift, 32 (m + 1) + 7 - shift <= NT).
+struct PlainTiles {
+  int lo, hi;
+};
+__device__ __forceinline__ PlainTiles plain_tiles(const Band &g, int fin_step, bool up, int shift, int NT) {
+  PlainTiles t;
+  t.lo = (up && shift > 0) ? 1 : 0;
+  t.hi = g.nsteps / kTileSteps;
+  if (fin_step >= 0) t.hi = min(t.hi, fin_step / kTileSteps);
+  if (up) t.hi = min(t.hi, max(NT - (kChunk - 1) + shift, 0) / kTileSteps);
+  t.lo = min(t.lo, g.ntiles);
+  t.hi = max(min(t.hi, g.ntiles), t.lo);
+  return t;
 }
 
 // =============================== forward =====================================
@@ -282,7 +333,6 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
     const int w = (wave - nsweep) / kStagers, l = (wave - nsweep) % kStagers;
     R *base = tiles + (size_t)w * 2 * kBuffers * kTileElems;
     const int half = lane >> 5, q = lane & 31;
-    int *my_loaded = &cnt.loaded[w * kStagers + l];
     // rows of a tile this wave stages: r(u) = 2*l + half + 2*kStagers*u
     constexpr int kRows = (kWave + 2 * kStagers - 1) / (2 * kStagers);
     struct Staged {
@@ -400,7 +450,7 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
           ydst[u * kStep * kTilePitch] = y;
         }
         // every lane's LDS writes precede the release by lane 0 of the same wave
-        if (lane == 0) publish(my_loaded, gt + 1);
+        if (lane == 0) count_in(&cnt.loaded[w * kBuffers + buf]);
         if (refill) store(out);
         // the next tile's inputs, fetched while this wave waits for its buffer
         if (m + 1 < g.ntiles) fetch(cur, g, m + 1);
@@ -430,7 +480,7 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
   R *my_seam = seam + (size_t)w * seam_pitch + kSeamPadLeft;
   const R *up_seam = seam + (size_t)prev * seam_pitch + kSeamPadLeft;
   R *base = tiles + (size_t)w * 2 * kBuffers * kTileElems;
-  int tile_base = 0, buf = 0;  // buf = tile number modulo kBuffers
+  int tile_base = 0, buf = 0, rounds = 0;  // tile number modulo kBuffers, and divided by it
   for (int band = 0; band * band_rows <= NS; ++band) {
     const Band g = band_of(band, w, nsweep, NS, NT);
     if (g.row0 > NS) break;
@@ -444,63 +494,68 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
 
     R own = (i == 0) ? (R)0 : ninf, own2 = ninf;
     R fin = ninf;
+    const R *seam_at = up_seam + (lane - shift);  // seam_at[e]: what lane 0 needs at step e + lane
     const bool has_down = g.nrows == kWave;
     // counters and seam values are read one chunk (one tile) ahead of their use, so
     // that the LDS round trip is off the chain; a stale value only costs a re-read
     int seen_ready = 0;
     R seen_seam = ninf;
-    int seen_loaded[kStagers];
-#pragma unroll
-    for (int l = 0; l < kStagers; ++l) seen_loaded[l] = 0;
-    for (int m = 0; m < g.ntiles; ++m) {
+    int seen_loaded = 0;
+    // One tile, specialised at compile time on whether the wave receives a seam (kUp),
+    // feeds one (kDown), and on kPlain: a tile whose 32 steps all exist, do not hold the
+    // answer's step and, with a seam above, look at existing seam columns only.  A single
+    // wave pays for every instruction it issues, scalar tests and branches included, so
+    // plain tiles run without the tests; and every kind of tile has a loop of its own (see
+    // sweep_tiles): with all kinds in one loop body the compiler's code for the steps
+    // themselves took twice as long.
+    auto one_tile = [&](int m, auto up_c, auto down_c, auto plain_c) __attribute__((always_inline)) -> bool {
+      constexpr bool kUp = decltype(up_c)::value;
+      constexpr bool kDown = decltype(down_c)::value;
+      constexpr bool kPlain = decltype(plain_c)::value;
       const int gt = tile_base + m;
-#pragma unroll
-      for (int l = 0; l < kStagers; ++l)
-        if (__builtin_amdgcn_readfirstlane(seen_loaded[l]) < gt + 1 &&
-            !wait_for(&cnt.loaded[w * kStagers + l], gt + 1, spin_limit)) {
-          give_up();
-          return;
-        }
+      if (__builtin_amdgcn_readfirstlane(seen_loaded) < kStagers * (rounds + 1) &&
+          !wait_for(&cnt.loaded[w * kBuffers + buf], kStagers * (rounds + 1), spin_limit)) {
+        give_up();
+        return false;
+      }
       // this lane's 32 steps of inputs go to registers in one burst
       R xq[kTileSteps], yq[kTileSteps];
       R *x_row = base + buf * kTileElems + lane * kTilePitch;  // x in, p out
       pull_row(xq, x_row);
       pull_row(yq, x_row + kBuffers * kTileElems);
       buf = buf + 1 == kBuffers ? 0 : buf + 1;
+      rounds += buf == 0;
 
-      // One chunk of kChunk steps, specialised at compile time on whether the wave
-      // receives a seam (kUp) and feeds one (kDown).
-      bool alive = true;
-      // kPlain: a tile whose 32 steps all exist and do not hold the answer's step; a single
-      // wave pays for every instruction it issues, scalar tests and branches included, so
-      // such tiles run without the two tests per chunk.
-      auto chunk = [&](auto up_c, auto down_c, auto plain_c, int c4, int e0) __attribute__((always_inline)) {
-        constexpr bool kUp = decltype(up_c)::value;
-        constexpr bool kDown = decltype(down_c)::value;
-        constexpr bool kPlain = decltype(plain_c)::value;
+      bool failed = false;
+      // one chunk of kChunk steps
+      auto chunk = [&](int c4, int e0) __attribute__((always_inline)) {
         R handed = ninf;  // lane k: the seam value lane 0 needs at step e0 + k
         if (kUp) {
-          const int need = min(e0 + kChunk - shift, cols);
+          const int need = kPlain ? e0 + kChunk - shift : min(e0 + kChunk - shift, cols);
           handed = seen_seam;
-          if (need > 0 && __builtin_amdgcn_readfirstlane(seen_ready) < up_base + need) {
-            if (!wait_for(&cnt.ready[prev], up_base + need, spin_limit)) {
-              alive = false;
-              return;
-            }
+          if ((kPlain || need > 0) && __builtin_amdgcn_readfirstlane(seen_ready) < up_base + need) {
+            // (a wait that has run out is not tried again: the wave finishes its tile on
+            // whatever the seam holds and then gives up)
+            if (!failed && !wait_for(&cnt.ready[prev], up_base + need, spin_limit)) failed = true;
             const int col = e0 + lane - shift;
             handed = (lane < kChunk && col >= 0 && col <= NT) ? up_seam[col] : ninf;
+            lds_reads_done();
           }
           // next chunk's counter, then its seam values (LDS serves a wave in order)
           seen_ready = peek(&cnt.ready[prev]);
-          const int col = e0 + kChunk + lane - shift;
-          seen_seam = ninf;
-          if (lane < kChunk && col >= 0 && col <= NT)
-            seen_seam = up_seam[col];
+          if (kPlain) {
+            // every column this tile and the first chunk after it look at exists: no
+            // tests, and what lanes 8 .. 63 read never reaches lane 0
+            seen_seam = seam_at[e0 + kChunk];
+          } else {
+            const int col = e0 + kChunk + lane - shift;
+            seen_seam = ninf;
+            if (lane < kChunk && col >= 0 && col <= NT) seen_seam = up_seam[col];
+          }
+          // (the reads above are for the next chunk: they are issued here, before the steps)
+          __builtin_amdgcn_sched_barrier(0);
         }
-        if (c4 == kTileSteps / kChunk - 1) {
-#pragma unroll
-          for (int l = 0; l < kStagers; ++l) seen_loaded[l] = peek(&cnt.loaded[w * kStagers + l]);
-        }
+        if (c4 == kTileSteps / kChunk - 1) seen_loaded = peek(&cnt.loaded[w * kBuffers + buf]);
         R vals[kChunk];
 #pragma unroll
         for (int k = 0; k < kChunk; ++k) {
@@ -519,6 +574,11 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
           vals[k] = v;
           own2 = own;
           own = v;
+          if (k == kChunk / 2 - 1) {
+            // the chunk's p takes the place of its x in the tile: first half
+            push_half<0>(x_row + c4 * kChunk, vals);
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
         if (!kPlain) {
           const int kf = fin_step - e0;  // wave-uniform
@@ -536,42 +596,39 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
             publish_lds_writes(&cnt.ready[w], my_base + done);
           }
         }
-        // the chunk's p takes the place of its x in the tile
-        push_chunk(x_row + c4 * kChunk, vals);
+        push_half<1>(x_row + c4 * kChunk, vals);
       };
-      auto tile = [&](auto up_c, auto down_c, auto plain_c) __attribute__((always_inline)) {
 #pragma unroll
-        for (int c4 = 0; c4 < kTileSteps / kChunk; ++c4) {
-          const int e0 = m * kTileSteps + c4 * kChunk;
-          if ((decltype(plain_c)::value || e0 < g.nsteps) && (!decltype(up_c)::value || alive))
-            chunk(up_c, down_c, plain_c, c4, e0);
-        }
-      };
-      auto tile_of = [&](auto up_c, auto down_c) __attribute__((always_inline)) {
-        const bool plain = (m + 1) * kTileSteps <= g.nsteps &&
-                           (unsigned)(fin_step - m * kTileSteps) >= (unsigned)kTileSteps;
-        if (plain)
-          tile(up_c, down_c, std::true_type{});
-        else
-          tile(up_c, down_c, std::false_type{});
-      };
-      if (has_up) {
-        if (has_down)
-          tile_of(std::true_type{}, std::true_type{});
-        else
-          tile_of(std::true_type{}, std::false_type{});
-      } else {
-        if (has_down)
-          tile_of(std::false_type{}, std::true_type{});
-        else
-          tile_of(std::false_type{}, std::false_type{});
+      for (int c4 = 0; c4 < kTileSteps / kChunk; ++c4) {
+        const int e0 = m * kTileSteps + c4 * kChunk;
+        if (kPlain || e0 < g.nsteps) chunk(c4, e0);
       }
-      if (!alive) {
+      if (failed) {
         give_up();
-        return;
+        return false;
       }
       if (lane == 0) publish_lds_writes(&cnt.written[w], gt + 1);
-    }
+      return true;
+    };
+    // the band's tiles: those before the plain ones, the plain ones, the rest
+    auto sweep_tiles = [&](auto up_c, auto down_c) __attribute__((always_inline)) -> bool {
+      const PlainTiles plain = plain_tiles(g, fin_step, decltype(up_c)::value, shift, NT);
+      for (int m = 0; m < plain.lo; ++m)
+        if (!one_tile(m, up_c, down_c, std::false_type{})) return false;
+      for (int m = plain.lo; m < plain.hi; ++m)
+        if (!one_tile(m, up_c, down_c, std::true_type{})) return false;
+      for (int m = plain.hi; m < g.ntiles; ++m)
+        if (!one_tile(m, up_c, down_c, std::false_type{})) return false;
+      return true;
+    };
+    bool done;
+    if (has_up)
+      done = has_down ? sweep_tiles(std::true_type{}, std::true_type{})
+                      : sweep_tiles(std::true_type{}, std::false_type{});
+    else
+      done = has_down ? sweep_tiles(std::false_type{}, std::true_type{})
+                      : sweep_tiles(std::false_type{}, std::false_type{});
+    if (!done) return;
     if (lane == fin_lane) ans[b] = peek(&cnt.failed) ? std::numeric_limits<R>::quiet_NaN() : fin;
     tile_base += g.ntiles;
   }
@@ -694,7 +751,6 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
     const int w = (wave - nsweep) / kStagers, l = (wave - nsweep) % kStagers;
     R *base = tiles + (size_t)w * 2 * kBuffers * kTileElems;
     const int half = lane >> 5, q = lane & 31;
-    int *my_loaded = &cnt.loaded[w * kStagers + l];
     // rows of a tile this wave stages: r(u) = 2*l + half + 2*kStagers*u
     constexpr int kRows = (kWave + 2 * kStagers - 1) / (2 * kStagers);
     struct Staged {
@@ -833,7 +889,7 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
           d2dst[u * kStep * kTilePitch] = d2;
         }
         // every lane's LDS writes precede the release by lane 0 of the same wave
-        if (lane == 0) publish(my_loaded, gt + 1);
+        if (lane == 0) count_in(&cnt.loaded[w * kBuffers + buf]);
         if (refill) store(out);
         // the next tile's inputs, fetched while this wave waits for its buffer
         if (m + 1 < g.ntiles) fetch(cur, g, m + 1);
@@ -874,7 +930,7 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
   const R *up_seam = seam + (size_t)prev * seam_pitch + kSeamPadLeft;
   R *base = tiles + (size_t)w * 2 * kBuffers * kTileElems;
   const R seed = ans_grad ? ans_grad[b] : (R)1;
-  int tile_base = 0, buf = 0;  // buf = tile number modulo kBuffers
+  int tile_base = 0, buf = 0, rounds = 0;  // tile number modulo kBuffers, and divided by it
   for (int band = 0; band * band_rows <= NS; ++band) {
     const Band g = band_of(band, w, nsweep, NS, NT);
     if (g.row0 > NS) break;
@@ -889,57 +945,56 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
     // the seed enters as "handed left" into the first cell of the reversed sweep
     R to_below = 0, to_below2 = 0, to_left = (r == 0) ? seed : (R)0;
     R g_origin = 0;
+    const R *seam_at = up_seam + (lane - shift);  // seam_at[e]: what lane 0 needs at step e + lane
     const bool has_down = g.nrows == kWave;
     int seen_ready = 0;
     R seen_seam = 0;
-    int seen_loaded[kStagers];
-#pragma unroll
-    for (int l = 0; l < kStagers; ++l) seen_loaded[l] = 0;
-    for (int m = 0; m < g.ntiles; ++m) {
+    int seen_loaded = 0;
+    // one tile; the compile-time flags and the loops are those of the forward kernel
+    auto one_tile = [&](int m, auto up_c, auto down_c, auto plain_c) __attribute__((always_inline)) -> bool {
+      constexpr bool kUp = decltype(up_c)::value;
+      constexpr bool kDown = decltype(down_c)::value;
+      constexpr bool kPlain = decltype(plain_c)::value;
       const int gt = tile_base + m;
-#pragma unroll
-      for (int l = 0; l < kStagers; ++l)
-        if (__builtin_amdgcn_readfirstlane(seen_loaded[l]) < gt + 1 &&
-            !wait_for(&cnt.loaded[w * kStagers + l], gt + 1, spin_limit)) {
-          give_up();
-          return;
-        }
+      if (__builtin_amdgcn_readfirstlane(seen_loaded) < kStagers * (rounds + 1) &&
+          !wait_for(&cnt.loaded[w * kBuffers + buf], kStagers * (rounds + 1), spin_limit)) {
+        give_up();
+        return false;
+      }
       R d1q[kTileSteps], d2q[kTileSteps];
       R *gx_row = base + buf * kTileElems + lane * kTilePitch;               // d1 in, gx out
       R *gy_row = base + (kBuffers + buf) * kTileElems + lane * kTilePitch;  // d2 in, gy out
       buf = buf + 1 == kBuffers ? 0 : buf + 1;
+      rounds += buf == 0;
       pull_row(d1q, gx_row);
       pull_row(d2q, gy_row);
 
-      bool alive = true;
-      // (kPlain: all 32 steps exist and none is the origin's, see the forward kernel)
-      auto chunk = [&](auto up_c, auto down_c, auto plain_c, int c4, int e0) __attribute__((always_inline)) {
-        constexpr bool kUp = decltype(up_c)::value;
-        constexpr bool kDown = decltype(down_c)::value;
-        constexpr bool kPlain = decltype(plain_c)::value;
+      bool failed = false;
+      auto chunk = [&](int c4, int e0) __attribute__((always_inline)) {
         R handed = 0;
         if (kUp) {
-          const int need = min(e0 + kChunk - shift, cols);
+          const int need = kPlain ? e0 + kChunk - shift : min(e0 + kChunk - shift, cols);
           handed = seen_seam;
-          if (need > 0 && __builtin_amdgcn_readfirstlane(seen_ready) < up_base + need) {
-            if (!wait_for(&cnt.ready[prev], up_base + need, spin_limit)) {
-              alive = false;
-              return;
-            }
+          if ((kPlain || need > 0) && __builtin_amdgcn_readfirstlane(seen_ready) < up_base + need) {
+            // (a wait that has run out is not tried again, see the forward kernel)
+            if (!failed && !wait_for(&cnt.ready[prev], up_base + need, spin_limit)) failed = true;
             const int col = e0 + lane - shift;
             handed = (lane < kChunk && col >= 0 && col <= NT) ? up_seam[col] : (R)0;
+            lds_reads_done();
           }
           // next chunk's counter, then its seam values (LDS serves a wave in order)
           seen_ready = peek(&cnt.ready[prev]);
-          const int col = e0 + kChunk + lane - shift;
-          seen_seam = 0;
-          if (lane < kChunk && col >= 0 && col <= NT)
-            seen_seam = up_seam[col];
+          if (kPlain) {
+            seen_seam = seam_at[e0 + kChunk];  // every column exists; lanes 8 .. 63 do not matter
+          } else {
+            const int col = e0 + kChunk + lane - shift;
+            seen_seam = 0;
+            if (lane < kChunk && col >= 0 && col <= NT) seen_seam = up_seam[col];
+          }
+          // (the reads above are for the next chunk: they are issued here, before the steps)
+          __builtin_amdgcn_sched_barrier(0);
         }
-        if (c4 == kTileSteps / kChunk - 1) {
-#pragma unroll
-          for (int l = 0; l < kStagers; ++l) seen_loaded[l] = peek(&cnt.loaded[w * kStagers + l]);
-        }
+        if (c4 == kTileSteps / kChunk - 1) seen_loaded = peek(&cnt.loaded[w * kBuffers + buf]);
         R down[kChunk], left[kChunk], cell[kChunk];
 #pragma unroll
         for (int k = 0; k < kChunk; ++k) {
@@ -958,6 +1013,12 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
           to_below2 = to_below;
           to_below = down[k];
           to_left = left[k];
+          if (k == kChunk / 2 - 1) {
+            // the chunk's gradients take the place of its d1 / d2 in the tile: first half
+            push_half<0>(gx_row + c4 * kChunk, down);
+            push_half<0>(gy_row + c4 * kChunk, left);
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
         if (!kPlain) {
           const int kf = fin_step - e0;  // wave-uniform
@@ -976,44 +1037,40 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
             publish_lds_writes(&cnt.ready[w], my_base + done);
           }
         }
-        // the chunk's gradients take the place of its d1 / d2 in the tile
-        push_chunk(gx_row + c4 * kChunk, down);
-        push_chunk(gy_row + c4 * kChunk, left);
+        push_half<1>(gx_row + c4 * kChunk, down);
+        push_half<1>(gy_row + c4 * kChunk, left);
       };
-      auto tile = [&](auto up_c, auto down_c, auto plain_c) __attribute__((always_inline)) {
 #pragma unroll
-        for (int c4 = 0; c4 < kTileSteps / kChunk; ++c4) {
-          const int e0 = m * kTileSteps + c4 * kChunk;
-          // the window's edges need no care here: d1 = d2 = 0 outside it
-          if ((decltype(plain_c)::value || e0 < g.nsteps) && (!decltype(up_c)::value || alive))
-            chunk(up_c, down_c, plain_c, c4, e0);
-        }
-      };
-      auto tile_of = [&](auto up_c, auto down_c) __attribute__((always_inline)) {
-        const bool plain = (m + 1) * kTileSteps <= g.nsteps &&
-                           (unsigned)(fin_step - m * kTileSteps) >= (unsigned)kTileSteps;
-        if (plain)
-          tile(up_c, down_c, std::true_type{});
-        else
-          tile(up_c, down_c, std::false_type{});
-      };
-      if (has_up) {
-        if (has_down)
-          tile_of(std::true_type{}, std::true_type{});
-        else
-          tile_of(std::true_type{}, std::false_type{});
-      } else {
-        if (has_down)
-          tile_of(std::false_type{}, std::true_type{});
-        else
-          tile_of(std::false_type{}, std::false_type{});
+      for (int c4 = 0; c4 < kTileSteps / kChunk; ++c4) {
+        const int e0 = m * kTileSteps + c4 * kChunk;
+        // the window's edges need no care here: d1 = d2 = 0 outside it
+        if (kPlain || e0 < g.nsteps) chunk(c4, e0);
       }
-      if (!alive) {
+      if (failed) {
         give_up();
-        return;
+        return false;
       }
       if (lane == 0) publish_lds_writes(&cnt.written[w], gt + 1);
-    }
+      return true;
+    };
+    auto sweep_tiles = [&](auto up_c, auto down_c) __attribute__((always_inline)) -> bool {
+      const PlainTiles plain = plain_tiles(g, fin_step, decltype(up_c)::value, shift, NT);
+      for (int m = 0; m < plain.lo; ++m)
+        if (!one_tile(m, up_c, down_c, std::false_type{})) return false;
+      for (int m = plain.lo; m < plain.hi; ++m)
+        if (!one_tile(m, up_c, down_c, std::true_type{})) return false;
+      for (int m = plain.hi; m < g.ntiles; ++m)
+        if (!one_tile(m, up_c, down_c, std::false_type{})) return false;
+      return true;
+    };
+    bool done;
+    if (has_up)
+      done = has_down ? sweep_tiles(std::true_type{}, std::true_type{})
+                      : sweep_tiles(std::true_type{}, std::false_type{});
+    else
+      done = has_down ? sweep_tiles(std::false_type{}, std::true_type{})
+                      : sweep_tiles(std::false_type{}, std::false_type{});
+    if (!done) return;
     if (lane == fin_lane && overwrite_ans_grad && ans_grad)
       ans_grad[b] = peek(&cnt.failed) ? std::numeric_limits<R>::quiet_NaN() : g_origin;
     tile_base += g.ntiles;
@@ -1052,12 +1109,12 @@ int forward_impl(const R *px, const R *py, const int64_t *boundary, R *p, R *ans
   // With at most two sweep waves there is room, for floats, for a third tile buffer, which
   // gives a staging wave two tiles' time instead of one to empty and refill a buffer.
   constexpr int kFewBuffers = sizeof(R) == 4 ? 3 : 2;
-  static_assert(kMaxSweep * kFwdStagers <= 16, "Counters::loaded is too short");
+  static_assert(kMaxSweep * 2 <= 16 && 2 * kFewBuffers <= 16, "Counters::loaded is too short");
   const bool few = n <= 2 && lds_bytes(n, T, kFewBuffers, sizeof(R)) <= kLdsBudget;
-  const int stagers = kFwdStagers;
+  const int stagers = few ? kFwdStagersFew : kFwdStagers;
   const size_t lds = lds_bytes(n, T, few ? kFewBuffers : 2, sizeof(R));
-  auto kernel = few ? (modified ? mi_forward_kernel<R, true, 2, kFwdStagers, kFewBuffers>
-                                : mi_forward_kernel<R, false, 2, kFwdStagers, kFewBuffers>)
+  auto kernel = few ? (modified ? mi_forward_kernel<R, true, 2, kFwdStagersFew, kFewBuffers>
+                                : mi_forward_kernel<R, false, 2, kFwdStagersFew, kFewBuffers>)
                     : (modified ? mi_forward_kernel<R, true, kMaxSweep, kFwdStagers, 2>
                                 : mi_forward_kernel<R, false, kMaxSweep, kFwdStagers, 2>);
   if (!allow_lds(reinterpret_cast<const void *>(kernel), lds))
@@ -1091,7 +1148,7 @@ int backward_impl(const R *px, const R *py, const int64_t *boundary, const R *p,
   constexpr bool kFloat = sizeof(R) == 4;
   constexpr int kFew = kFloat ? kBwdStagersFew : kBwdStagers;
   constexpr int kFewBuffers = kFloat ? 3 : 2;
-  static_assert(2 * kFew <= 16 && kMaxSweep * kBwdStagers <= 16, "Counters::loaded is too short");
+  static_assert(kMaxSweep * 2 <= 16 && 2 * kFewBuffers <= 16, "Counters::loaded is too short");
   const bool few = n <= 2 && lds_bytes(n, T, kFewBuffers, sizeof(R)) <= kLdsBudget;
   const int stagers = few ? kFew : kBwdStagers;
   const size_t lds = lds_bytes(n, T, few ? kFewBuffers : 2, sizeof(R));
