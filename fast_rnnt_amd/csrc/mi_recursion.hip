@@ -234,6 +234,16 @@ __device__ __forceinline__ void push_half(R *dst, const R (&src)[kChunk]) {
   }
 }
 
+// Keeps the registers of a half chunk that has just been written to LDS from being given
+// to the next results at once (see push_half): called four steps later, it makes them
+// count as still in use until then.  Emits no instruction.
+template <typename R>
+__device__ __forceinline__ void still_in_use(const R (&v)[kChunk], int first) {
+  if constexpr (sizeof(R) == 4) {
+    asm volatile("" ::"v"(v[first]), "v"(v[first + 1]), "v"(v[first + 2]), "v"(v[first + 3]));
+  }
+}
+
 struct Counters {
   int failed;                             // set by a wave whose bounded wait ran out
   int ready[kMaxSweep];                   // seam columns published by sweep wave w
@@ -527,6 +537,9 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
       rounds += buf == 0;
 
       bool failed = false;
+      R last[kChunk];  // the chunk before
+#pragma unroll
+      for (int k = 0; k < kChunk; ++k) last[k] = 0;
       // one chunk of kChunk steps
       auto chunk = [&](int c4, int e0) __attribute__((always_inline)) {
         R handed = ninf;  // lane k: the seam value lane 0 needs at step e0 + k
@@ -577,9 +590,11 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
           if (k == kChunk / 2 - 1) {
             // the chunk's p takes the place of its x in the tile: first half
             push_half<0>(x_row + c4 * kChunk, vals);
+            still_in_use(last, kChunk / 2);
             __builtin_amdgcn_sched_barrier(0);
           }
         }
+        still_in_use(vals, 0);
         if (!kPlain) {
           const int kf = fin_step - e0;  // wave-uniform
           if ((unsigned)kf < (unsigned)kChunk) {
@@ -597,6 +612,8 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
           }
         }
         push_half<1>(x_row + c4 * kChunk, vals);
+#pragma unroll
+        for (int k = kChunk / 2; k < kChunk; ++k) last[k] = vals[k];
       };
 #pragma unroll
       for (int c4 = 0; c4 < kTileSteps / kChunk; ++c4) {
