@@ -505,7 +505,7 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
     R own = (i == 0) ? (R)0 : ninf, own2 = ninf;
     R fin = ninf;
     const R *seam_at = up_seam + (lane - shift);  // seam_at[e]: what lane 0 needs at step e + lane
-    const bool has_down = g.nrows == kWave;
+    const bool has_down = g.row0 + kWave <= NS;  // rows below this wave's: someone reads the seam
     // counters and seam values are read one chunk (one tile) ahead of their use, so
     // that the LDS round trip is off the chain; a stale value only costs a re-read
     int seen_ready = 0;
@@ -963,7 +963,7 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
     R to_below = 0, to_below2 = 0, to_left = (r == 0) ? seed : (R)0;
     R g_origin = 0;
     const R *seam_at = up_seam + (lane - shift);  // seam_at[e]: what lane 0 needs at step e + lane
-    const bool has_down = g.nrows == kWave;
+    const bool has_down = g.row0 + kWave <= NS;  // rows below this wave's: someone reads the seam
     int seen_ready = 0;
     R seen_seam = 0;
     int seen_loaded = 0;
