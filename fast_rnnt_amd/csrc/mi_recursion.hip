@@ -7,9 +7,11 @@
 // earlier (modified lattice) and arrives through a DPP wave shift, and the
 // neighbour in the same row is the lane's own previous result.
 //
-// A single wave issues about one instruction every 4.5 cycles and nothing overlaps
+// A single wave issues about one instruction every 4.5 cycles (a dependent one every 8, a
+// scalar test with its branch costs 18 cycles, 35 when taken) and nothing overlaps
 // within it, so a sweep wave's time is its instruction count: everything that is not
-// the dependent chain is kept off it.  *Staging waves* of the same workgroup fetch
+// the dependent chain is kept off it, and tiles that need no tests run without them,
+// each kind of tile in a loop of its own.  *Staging waves* of the same workgroup fetch
 // px/py (forward) or p/px (backward) with coalesced, range-checked row loads, turn
 // them into diagonal ("sheared") 64-row x 32-step tiles in LDS and -- for the
 // backward sweep -- also evaluate the exp() of the gradient split; the sweep wave
@@ -17,10 +19,11 @@
 // in the same LDS buffer with 16-byte writes.  The staging waves carry the results
 // to memory as coalesced row segments through range-checked buffer stores (a cell
 // outside the window gets an offset that the hardware drops instead of a branch)
-// before they refill the buffer.  There are two or three buffers per sweep wave;
+// once they have refilled the buffer.  There are two or three buffers per sweep wave;
 // sweep and staging waves meet only through monotone LDS counters (bounded
-// spinning), never at a barrier, and the sweep wave looks at a counter one chunk
-// (one tile) before it needs it.
+// spinning; one counter per buffer, which all staging waves of a sweep wave count up),
+// never at a barrier, and the sweep wave looks at a counter one chunk (one tile) before
+// it needs it.
 //
 // Rows beyond 64 go to further sweep waves; wave w+1 consumes the last row of
 // wave w through an LDS seam row guarded by a progress counter and simply runs a
