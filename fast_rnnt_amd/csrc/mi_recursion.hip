@@ -1131,12 +1131,15 @@ int forward_impl(const R *px, const R *py, const int64_t *boundary, R *p, R *ans
   constexpr int kFewBuffers = sizeof(R) == 4 ? 3 : 2;
   static_assert(kMaxSweep * 2 <= 16 && 2 * kFewBuffers <= 16, "Counters::loaded is too short");
   const bool few = n <= 2 && lds_bytes(n, T, kFewBuffers, sizeof(R)) <= kLdsBudget;
-  const int stagers = few ? kFwdStagersFew : kFwdStagers;
+  // (doubles keep two staging waves per sweep wave: with more waves in the workgroup a sweep
+  // wave's two tile rows of doubles no longer fit its share of the registers)
+  constexpr int kMany = sizeof(R) == 4 ? kFwdStagers : 2, kFew = sizeof(R) == 4 ? kFwdStagersFew : 2;
+  const int stagers = few ? kFew : kMany;
   const size_t lds = lds_bytes(n, T, few ? kFewBuffers : 2, sizeof(R));
-  auto kernel = few ? (modified ? mi_forward_kernel<R, true, 2, kFwdStagersFew, kFewBuffers>
-                                : mi_forward_kernel<R, false, 2, kFwdStagersFew, kFewBuffers>)
-                    : (modified ? mi_forward_kernel<R, true, kMaxSweep, kFwdStagers, 2>
-                                : mi_forward_kernel<R, false, kMaxSweep, kFwdStagers, 2>);
+  auto kernel = few ? (modified ? mi_forward_kernel<R, true, 2, kFew, kFewBuffers>
+                                : mi_forward_kernel<R, false, 2, kFew, kFewBuffers>)
+                    : (modified ? mi_forward_kernel<R, true, kMaxSweep, kMany, 2>
+                                : mi_forward_kernel<R, false, kMaxSweep, kMany, 2>);
   if (!allow_lds(reinterpret_cast<const void *>(kernel), lds))
     return check_launch("mi_forward: hipFuncSetAttribute");
   hipLaunchKernelGGL(kernel, dim3(B), dim3(n * (1 + stagers) * kWave), lds,
@@ -1163,7 +1166,7 @@ int backward_impl(const R *px, const R *py, const int64_t *boundary, const R *p,
     return fail(FRNNT_ELIMIT, "mi_backward: T=%d needs %zu bytes of LDS", T, lds_bytes(n, T, 2, sizeof(R)));
   // With at most two sweep waves there is room for more staging waves per sweep wave and,
   // for floats, for a third tile buffer, which gives a staging wave two tiles' time instead
-  // of one to empty and refill a buffer.  (A workgroup of 14 waves leaves each 128
+  // of one to empty and refill a buffer.  (A workgroup of 16 waves leaves each 128
   // registers, too few for a sweep wave's two tile rows of doubles.)
   constexpr bool kFloat = sizeof(R) == 4;
   constexpr int kFew = kFloat ? kBwdStagersFew : kBwdStagers;
