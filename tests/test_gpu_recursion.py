@@ -108,6 +108,32 @@ def test_random_lattices_match_oracle(gpu_device, dtype, modified):
         _compare(px, py, _windows(g, B, S, T, modified), w, gpu_device, f"windows{n}")
 
 
+@pytest.mark.parametrize("modified", [False, True])
+def test_tile_and_seam_borders(gpu_device, modified):
+    # The sweep waves treat a 32-step tile as "plain" (no tests inside) when all its steps
+    # exist, the result's step is not among them and every seam column it looks at exists;
+    # a wave feeds the seam only when rows lie below it.  Frame counts around the multiples
+    # of 32 and row counts around one, two and three waves of 64 rows put every one of
+    # those borders on either side.
+    g = torch.Generator().manual_seed(300 + int(modified))
+    n = 0
+    for S in (62, 63, 64, 65, 126, 127, 128, 129, 191, 192):
+        for T in (31, 32, 33, 63, 64, 65, 71, 72, 95, 96, 97, 100):
+            if modified and T < S:
+                continue
+            B = 2
+            px = -0.7 + 0.3 * torch.randn(B, S, T + (0 if modified else 1), generator=g)
+            py = -0.7 + 0.3 * torch.randn(B, S + 1, T, generator=g)
+            if not modified:
+                px[:, :, T] = -math.inf
+            # second utterance: a window that ends a few rows / frames early
+            bnd = torch.tensor([[0, 0, S, T], [0, 0, S - n % 3, T - n % 5]], dtype=torch.int64)
+            if not modified:
+                px[1, :, T - n % 5] = -math.inf
+            _compare(px, py, bnd, torch.ones(B), gpu_device, f"border{n}")
+            n += 1
+
+
 def test_large_magnitudes_and_neg_inf(gpu_device):
     # fast_rnnt/python/tests/mutual_information_test.py:113-130 ("big" inputs)
     g = torch.Generator().manual_seed(7)
