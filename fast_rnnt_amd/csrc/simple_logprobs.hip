@@ -185,20 +185,6 @@ __global__ void __launch_bounds__(256)
 }
 
 // ---- backward ------------------------------------------------------------------------
-// The factor that the gradient of the scores puts on px_grad[b] / py_grad[b]:
-// scale * values[b * stride], or 1 without values.  The kernels below multiply what they
-// read of the two arrays by it; a caller that has scaled them in place passes no values.
-// (v * 1 is v bit for bit, so the multiplication is unconditional.)
-template <typename R>
-struct ScoreGrad {
-  const R *values;
-  int stride;
-  R scale;
-  __device__ __forceinline__ R of(int b) const {
-    return values ? scale * values[(long)b * stride] : (R)1;
-  }
-};
-
 // 256-thread workgroups.  The first ceil(B*(S+1)/4) of them give each wave one
 // lattice row (b, s): D[b,s,:] and the two row sums.  The remaining ones take 64
 // frames of one utterance each and form the column sums, the four waves splitting
@@ -210,7 +196,7 @@ __global__ void __launch_bounds__(256)
                            const R *__restrict__ norm_raw, const int64_t *__restrict__ boundary,
                            const int64_t *__restrict__ window, R *__restrict__ dmat,
                            R *__restrict__ row_x, R *__restrict__ row_y, R *__restrict__ col_y,
-                           int B, int S, int T, int ldd, int rnnt_type, ScoreGrad<R> score_grad) {
+                           int B, int S, int T, int ldd, int rnnt_type) {
   __shared__ R partial[4][kWave];
   const int S1 = S + 1;
   const int T1 = rnnt_type == kRegular ? T + 1 : T;
@@ -231,7 +217,6 @@ __global__ void __launch_bounds__(256)
     const R *gy_row = gpy + row * T;
     const R *nr_row = norm_raw + row * T;
     R *d_row = dmat + row * ldd;
-    const R g = score_grad.of(b);
     R sx = 0, sy = 0;
     for (int t0 = 0; t0 < T; t0 += 4 * kWave) {
       R gx[4], gy[4], nr[4];
@@ -239,9 +224,9 @@ __global__ void __launch_bounds__(256)
       for (int u = 0; u < 4; ++u) {
         const int t = t0 + u * kWave + lane;
         const bool ok = t < T && row_in && t >= lim.t_begin && t < lim.t_end;
-        gx[u] = (ok && gx_row && t != t_mask) ? gx_row[t] * g : (R)0;
-        gy[u] = ok ? gy_row[t] * g : (R)0;
-        if (ok && gx_prev && t != t_mask) gy[u] += gx_prev[t] * g;
+        gx[u] = (ok && gx_row && t != t_mask) ? gx_row[t] : (R)0;
+        gy[u] = ok ? gy_row[t] : (R)0;
+        if (ok && gx_prev && t != t_mask) gy[u] += gx_prev[t];
         nr[u] = ok ? nr_row[t] : (R)0;
       }
 #pragma unroll
@@ -265,16 +250,15 @@ __global__ void __launch_bounds__(256)
     const int t_mask = (rnnt_type == kRegular && boundary) ? (int)boundary[4 * b + 3] : -1;
     const Limits lim = limits_of(window, b, S, T);
     const bool ok = t < T && t >= lim.t_begin && t < lim.t_end;
-    const R g = score_grad.of(b);
     R acc = 0;
     for (int s0 = wave; s0 < S1; s0 += 16) {
       R v[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int s = s0 + 4 * u;
-        v[u] = (ok && s < S1) ? gpy[((long)b * S1 + s) * T + t] * g : (R)0;
+        v[u] = (ok && s < S1) ? gpy[((long)b * S1 + s) * T + t] : (R)0;
         if (constrained && ok && s >= 1 && s < S1 && t != t_mask)
-          v[u] += gpx[((long)b * S + s - 1) * T1 + t] * g;
+          v[u] += gpx[((long)b * S + s - 1) * T1 + t];
       }
       acc += (v[0] + v[1]) + (v[2] + v[3]);
     }
@@ -382,17 +366,16 @@ template <typename R>
 __global__ void __launch_bounds__(256)
     simple_bwd_symbols_kernel(const R *__restrict__ gpx, const int64_t *__restrict__ symbols,
                               const int64_t *__restrict__ boundary, R *__restrict__ am_grad,
-                              int B, int S, int T, int C, int rnnt_type, ScoreGrad<R> score_grad) {
+                              int B, int S, int T, int C, int rnnt_type) {
   const long idx = (long)blockIdx.x * 256 + threadIdx.x;
   if (idx >= (long)B * T) return;
   const int b = (int)(idx / T), t = (int)(idx % T);
   const int T1 = rnnt_type == kRegular ? T + 1 : T;
   if (rnnt_type == kRegular && boundary && boundary[4 * b + 3] == t) return;
   R *row = am_grad + idx * C;
-  const R g = score_grad.of(b);
   for (int s = 0; s < S; ++s) {
     const int64_t sym = symbols[(long)b * S + s];
-    if (sym >= 0 && sym < C) row[sym] += gpx[((long)b * S + s) * T1 + t] * g;
+    if (sym >= 0 && sym < C) row[sym] += gpx[((long)b * S + s) * T1 + t];
   }
 }
 
@@ -1033,7 +1016,7 @@ __device__ __forceinline__ void simple_bwd_am_panel_body(
     const float *__restrict__ dmat, const float *__restrict__ gpx,
     const float *__restrict__ col_y, float *__restrict__ am_grad,
     const int64_t *__restrict__ window, int B, int S, int T, int C, int ldd, int term,
-    int rnnt_type, int rows_cap, ScoreGrad<float> score_grad) {
+    int rnnt_type, int rows_cap) {
   using namespace dgemm;
   extern __shared__ float am_lds[];
   int *sym_s = reinterpret_cast<int *>(am_lds);   // [rows_cap] symbols of the pass (-1: none)
@@ -1057,7 +1040,6 @@ __device__ __forceinline__ void simple_bwd_am_panel_body(
   const float *amb = am + (long)b * T * C;
   const float *db = dmat + (long)b * S1 * ldd;
   const float *gxb = gpx + (long)b * S * T1;
-  const float gx_factor = score_grad.of(b);
   // symbols are < C < 2^31: their low words (little endian) are enough to compare
   const int *sym_lo = reinterpret_cast<const int *>(symbols + (long)b * S);
   const int t_mask = (rnnt_type == kRegular && boundary) ? (int)boundary[4 * b + 3] : -1;
@@ -1158,7 +1140,7 @@ __device__ __forceinline__ void simple_bwd_am_panel_body(
     const bool hot_ok = hot_t < T && hot_t != t_mask;
     auto hot_value = [&](int i) {
       const int k = k0 + 2 * i + half;
-      return (hot_ok && k < S) ? gxb[(long)k * T1 + hot_t] * gx_factor : 0.f;
+      return (hot_ok && k < S) ? gxb[(long)k * T1 + hot_t] : 0.f;
     };
     int ahead[kAmHotAhead];
     float ahead_v[kAmHotAhead];
@@ -1302,10 +1284,10 @@ __global__ void __launch_bounds__(256, kPerCu)
                                const float *__restrict__ gpx, const float *__restrict__ col_y,
                                float *__restrict__ am_grad, const int64_t *__restrict__ window,
                                int B, int S, int T, int C, int ldd, int term, int rnnt_type,
-                               int rows_cap, ScoreGrad<float> score_grad) {
+                               int rows_cap) {
   simple_bwd_am_panel_body<kCap>((int)blockIdx.x, lm, am, symbols, boundary, lm_max, am_max, dmat,
                                  gpx, col_y, am_grad, window, B, S, T, C, ldd, term, rnnt_type,
-                                 rows_cap, score_grad);
+                                 rows_cap);
 }
 // Both gradient products in one launch: the first lm_blocks workgroups take tiles of
 // lm.grad, the rest tiles of am.grad.  The two only read what the prep kernel left, so
@@ -1326,14 +1308,14 @@ __global__ void __launch_bounds__(256, 2)
                             const float *__restrict__ col_y, float *__restrict__ lm_grad,
                             float *__restrict__ am_grad, const int64_t *__restrict__ window, int B,
                             int S, int T, int C, int ldd, int term, int rnnt_type, int rows_cap,
-                            int lm_blocks, ScoreGrad<float> score_grad) {
+                            int lm_blocks) {
   if ((int)blockIdx.x < lm_blocks)
     simple_bwd_lm_slab_body<kS, kK>((int)blockIdx.x, lm, am, symbols, lm_max, am_max, dmat, row_x,
                                     row_y, lm_grad, window, B, S, T, C, ldd, term);
   else
     simple_bwd_am_panel_body<kAmCap>((int)blockIdx.x - lm_blocks, lm, am, symbols, boundary, lm_max, am_max,
                              dmat, gpx, col_y, am_grad, window, B, S, T, C, ldd, term, rnnt_type,
-                             rows_cap, score_grad);
+                             rows_cap);
 }
 // lm.grad and am.grad together (float only)
 void launch_bwd_both(const float *lm, const float *am, const int64_t *symbols,
@@ -1341,7 +1323,7 @@ void launch_bwd_both(const float *lm, const float *am, const int64_t *symbols,
                      const float *dmat, const float *gpx, const float *row_x, const float *row_y,
                      const float *col_y, float *lm_grad, float *am_grad, const int64_t *window,
                      int B, int S, int T, int C, int ldd, int term, int rnnt_type,
-                     ScoreGrad<float> score_grad, hipStream_t stream) {
+                     hipStream_t stream) {
   const int S1 = S + 1;
   const bool rows96 = (S1 + 95) / 96 * 96 < (S1 + 127) / 128 * 128;
   const int rows = rows96 ? 96 : 128;
@@ -1357,13 +1339,12 @@ void launch_bwd_both(const float *lm, const float *am, const int64_t *symbols,
   (void)allow_lds(reinterpret_cast<const void *>(kernel), lds);
   hipLaunchKernelGGL(kernel, dim3(am_blocks + lm_blocks), dim3(256), lds, stream, lm, am, symbols,
                      boundary, lm_max, am_max, dmat, gpx, row_x, row_y, col_y, lm_grad, am_grad,
-                     window, B, S, T, C, ldd, term, rnnt_type, rows_cap, (int)lm_blocks, score_grad);
+                     window, B, S, T, C, ldd, term, rnnt_type, rows_cap, (int)lm_blocks);
 }
 void launch_bwd_both(const double *, const double *, const int64_t *, const int64_t *,
                      const double *, const double *, const double *, const double *,
                      const double *, const double *, const double *, double *, double *,
-                     const int64_t *, int, int, int, int, int, int, int, ScoreGrad<double>,
-                     hipStream_t) {}
+                     const int64_t *, int, int, int, int, int, int, int, hipStream_t) {}
 void launch_bwd_lm(const float *lm, const float *am, const int64_t *symbols, const float *lm_max,
                    const float *am_max, const float *dmat, const float *row_x, const float *row_y,
                    float *lm_grad, const int64_t *window, int B, int S, int T, int C, int ldd,
@@ -1392,7 +1373,7 @@ void launch_bwd_am(const float *lm, const float *am, const int64_t *symbols,
                    const int64_t *boundary, const float *lm_max, const float *am_max,
                    const float *dmat, const float *gpx, const float *col_y, float *am_grad,
                    const int64_t *window, int B, int S, int T, int C, int ldd, int term,
-                   int rnnt_type, ScoreGrad<float> score_grad, hipStream_t stream) {
+                   int rnnt_type, hipStream_t stream) {
   const int tiles = ((C + kAmC - 1) / kAmC) * ((T + kAmT - 1) / kAmT);
   // rows of k held in LDS per pass: all of them when they fit
   // Rows of k held in LDS per pass: at most 64, in passes of equal size.  The workgroup's
@@ -1408,13 +1389,13 @@ void launch_bwd_am(const float *lm, const float *am, const int64_t *symbols,
   (void)allow_lds(reinterpret_cast<const void *>(kernel), lds);
   hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(tiles, B)), dim3(256), lds, stream, lm, am,
                      symbols, boundary, lm_max, am_max, dmat, gpx, col_y, am_grad, window, B, S, T, C,
-                     ldd, term, rnnt_type, rows_cap, score_grad);
+                     ldd, term, rnnt_type, rows_cap);
 }
 void launch_bwd_am(const double *lm, const double *am, const int64_t *symbols,
                    const int64_t *boundary, const double *lm_max, const double *am_max,
                    const double *dmat, const double *gpx, const double *col_y, double *am_grad,
                    const int64_t *, int B, int S, int T, int C, int ldd, int term, int rnnt_type,
-                   ScoreGrad<double> score_grad, hipStream_t stream) {
+                   hipStream_t stream) {
   const dim3 grid((C + kTileN - 1) / kTileN, (T + kTileM - 1) / kTileM, B);
   hipLaunchKernelGGL(simple_bwd_am_kernel<double>, grid, dim3(kGemmThreads), 0, stream, lm, am,
                      lm_max, am_max, dmat, col_y, am_grad, S, T, C, ldd, term);
@@ -1422,7 +1403,7 @@ void launch_bwd_am(const double *lm, const double *am, const int64_t *symbols,
     const long n = (long)B * T;
     hipLaunchKernelGGL(simple_bwd_symbols_kernel<double>, dim3((unsigned)((n + 255) / 256)),
                        dim3(256), 0, stream, gpx, symbols, boundary, am_grad, B, S, T, C,
-                       rnnt_type, score_grad);
+                       rnnt_type);
   }
 }
 
@@ -1482,15 +1463,9 @@ int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
        (long)(S + 1) * (T + 3) * 4 >= (1L << 31)))
     return fail(FRNNT_ELIMIT, "simple_logprobs_bwd: one utterance's lm, am or lattice exceeds 2 GiB");
   hipStream_t stream = static_cast<hipStream_t>(stream_);
-  // what the kernels multiply px_grad / py_grad by as they read them: nothing when the two
-  // arrays are scaled in place first
-  ScoreGrad<R> on_read{nullptr, 0, (R)1};
-  if (score_grad && (score_grad_stride & ~(FRNNT_SCORE_GRAD_PER_UTTERANCE | FRNNT_SCORE_GRAD_ON_READ)))
-    return fail(FRNNT_EINVAL, "simple_logprobs_bwd: bad score_grad_stride");
-  if (score_grad && (score_grad_stride & FRNNT_SCORE_GRAD_ON_READ)) {
-    on_read = ScoreGrad<R>{score_grad, score_grad_stride & FRNNT_SCORE_GRAD_PER_UTTERANCE,
-                           (R)score_grad_scale};
-  } else if (score_grad) {
+  if (score_grad) {
+    if (score_grad_stride != 0 && score_grad_stride != 1)
+      return fail(FRNNT_EINVAL, "simple_logprobs_bwd: score_grad_stride must be 0 or 1");
     const int T1 = rnnt_type == kRegular ? T + 1 : T;
     const int per_x = S * T1, per_y = (S + 1) * T;
     const int x_blocks = (per_x + 1023) / 1024, y_blocks = (per_y + 1023) / 1024;
@@ -1505,13 +1480,13 @@ int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
   const long prep_blocks = ((long)B * (S + 1) + 3) / 4 + (long)B * ((T + kWave - 1) / kWave);
   hipLaunchKernelGGL(simple_bwd_prep_kernel<R>, dim3((unsigned)prep_blocks), dim3(256), 0, stream,
                      px_grad, py_grad, norm_raw, boundary, window, dmat, row_x, row_y, col_y, B, S, T,
-                     ldd, rnnt_type, on_read);
+                     ldd, rnnt_type);
   // (one launch for both products while they are short: at B (S+1) T C = 3.2e8 it saves
   // about 1 us of 37; at 3.9e9 the common LDS and register budget costs 8 %)
   if (std::is_same<R, float>::value && lm_grad && am_grad && T > 0 &&
       (double)B * (S + 1) * T * C < 1e9) {
     launch_bwd_both(lm, am, symbols, boundary, lm_max, am_max, dmat, px_grad, row_x, row_y, col_y,
-                    lm_grad, am_grad, window, B, S, T, C, ldd, term, rnnt_type, on_read, stream);
+                    lm_grad, am_grad, window, B, S, T, C, ldd, term, rnnt_type, stream);
     return check_launch("simple_logprobs_bwd");
   }
   if (lm_grad)
@@ -1519,7 +1494,7 @@ int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
                   ldd, term, stream);
   if (am_grad && T > 0)
     launch_bwd_am(lm, am, symbols, boundary, lm_max, am_max, dmat, px_grad, col_y, am_grad, window,
-                  B, S, T, C, ldd, term, rnnt_type, on_read, stream);
+                  B, S, T, C, ldd, term, rnnt_type, stream);
   return check_launch("simple_logprobs_bwd");
 }
 

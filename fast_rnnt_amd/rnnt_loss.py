@@ -356,7 +356,7 @@ class _SimpleLoss(torch.autograd.Function):
         if need_grad:
             ctx.save_for_backward(lm_c, am_c, sym_c, bnd_c, work, px_grad, py_grad)
             ctx.meta = (B, S, T, C, int(termination_symbol), kind, sfx, reduction,
-                        o_lmx, o_amx, o_nr, bool(want_grads))
+                        o_lmx, o_amx, o_nr)
         if px_grad is None:
             return loss, None, None
         ctx.mark_non_differentiable(px_grad, py_grad)
@@ -367,16 +367,12 @@ class _SimpleLoss(torch.autograd.Function):
         if g_loss is None:
             return (None,) * 9
         lm, am, sym, bnd, work, px_grad, py_grad = ctx.saved_tensors
-        B, S, T, C, term, kind, sfx, reduction, o_lmx, o_amx, o_nr, handed_out = ctx.meta
+        B, S, T, C, term, kind, sfx, reduction, o_lmx, o_amx, o_nr = ctx.meta
         opts = dict(dtype=am.dtype, device=am.device)
         with _on_device(am.device):
             # d loss / d scores[b] = scale * g_loss[b * stride]
             g = g_loss.contiguous()
             stride = 1 if reduction == 0 else 0
-            if not handed_out:
-                # nobody else holds px_grad / py_grad: no need to scale them in place, the
-                # kernels apply the factor as they read them (FRNNT_SCORE_GRAD_ON_READ)
-                stride |= 2
             scale = -1.0 / B if reduction == 1 else -1.0
             ldd = (T + 3) // 4 * 4
             # scratch in one allocation: dmat | row_x | row_y | col_y
@@ -386,8 +382,8 @@ class _SimpleLoss(torch.autograd.Function):
             sbase, wbase, item = scratch.data_ptr(), work.data_ptr(), work.element_size()
             lm_grad = torch.empty_like(lm) if ctx.needs_input_grad[0] else None
             am_grad = torch.empty_like(am) if ctx.needs_input_grad[1] else None
-            # px_grad / py_grad that were handed out are scaled in place by the scores'
-            # gradient, exactly as MutualInformationRecursionFunction.backward does to them
+            # px_grad / py_grad are scaled in place by the scores' gradient, exactly as
+            # MutualInformationRecursionFunction.backward does to the tensors it handed out
             _lib.call("frnnt_simple_logprobs_bwd_" + sfx, lm.data_ptr(), am.data_ptr(),
                       sym.data_ptr(), _lib.ptr(bnd), wbase + o_lmx * item, wbase + o_amx * item,
                       wbase + o_nr * item, g.data_ptr(), stride, scale, px_grad.data_ptr(),

@@ -142,16 +142,12 @@ int frnnt_simple_logprobs_fwd_f64(const double *lm, const double *am, const int6
  * elementwise pass plus two MFMA GEMMs.
  *   px_grad, py_grad: dL/dpx, dL/dpy (shapes of px, py)                    in
  *   score_grad or NULL: when given, px_grad[b] and py_grad[b] are first multiplied
- *     IN PLACE by score_grad_scale * score_grad[b * stride] -- the scaling step of the
- *     recursion's autograd backward (mutual_information.py:173-181), for callers that
- *     hold the occupation gradients and the gradient of the scores separately.
- *     score_grad_stride: FRNNT_SCORE_GRAD_PER_UTTERANCE (1) = one value per utterance,
- *     0 = one scalar for all (the gradient of a summed or averaged loss, with the sign
- *     and the 1/B of rnnt_loss.py:160-169 in score_grad_scale).  With
- *     FRNNT_SCORE_GRAD_ON_READ (2) added, px_grad and py_grad are left as they are and the
- *     kernels apply the same factor as they read them -- the same lm_grad / am_grad bit
- *     for bit, one pass over the two arrays less -- for callers that hand px_grad /
- *     py_grad to nobody else (the reference scales the tensors it has handed out).
+ *     IN PLACE by score_grad_scale * score_grad[b * score_grad_stride] -- the scaling
+ *     step of the recursion's autograd backward (mutual_information.py:173-181), for
+ *     callers that hold the occupation gradients and the gradient of the scores
+ *     separately.  score_grad_stride 1: one value per utterance; 0: one scalar for
+ *     all (the gradient of a summed or averaged loss, with the sign and the 1/B of
+ *     rnnt_loss.py:160-169 in score_grad_scale)
  *   dmat [B][S+1][T rounded up to a multiple of 4], row_x [B][S+1], row_y [B][S+1],
  *   col_y [B][T]                                                           scratch
  *   lm_grad [B][S+1][C], am_grad [B][T][C]: out; either may be NULL to skip it
@@ -160,8 +156,6 @@ int frnnt_simple_logprobs_fwd_f64(const double *lm, const double *am, const int6
  *   the sums stop at s_end / t_end, and am_grad rows of frames >= t_end are stored as
  *   exact zeros without being computed.  Required when the forward ran with window_only.
  */
-#define FRNNT_SCORE_GRAD_PER_UTTERANCE 1
-#define FRNNT_SCORE_GRAD_ON_READ 2
 int frnnt_simple_logprobs_bwd_f32(const float *lm, const float *am, const int64_t *symbols,
                                   const int64_t *boundary, const float *lm_max,
                                   const float *am_max, const float *norm_raw,

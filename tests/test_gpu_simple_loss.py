@@ -351,42 +351,6 @@ def test_gradient_products_together_and_apart(gpu_device, shape, ragged):
     assert (lm_both - lm_only).abs().max().item() <= 1e-5 * max(1.0, lm_only.abs().max().item())
 
 
-@pytest.mark.parametrize("kind", KINDS)
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
-@pytest.mark.parametrize("reduction", ["none", "mean"])
-def test_scores_gradient_in_place_or_as_it_is_read(gpu_device, dtype, kind, reduction):
-    # With return_grad=True the occupation gradients were handed out and backward scales
-    # them in place by the gradient of the scores, as the reference does to its tensors;
-    # without, they stay as they are and the kernels apply the factor as they read them
-    # (FRNNT_SCORE_GRAD_ON_READ).  lm.grad and am.grad must agree bit for bit, also for
-    # shapes that take the separate launches and a second pass over the lattice rows.
-    for n, (B, S, T, C) in enumerate([(3, 5, 9, 8), (2, 60, 65, 33), (2, 100, 130, 520)]):
-        am, lm, sym, bnd = _case(900 + n, B, S, T, C, dtype, kind)
-        g = torch.Generator().manual_seed(17 + n)
-        weights = (torch.rand(B, generator=g, dtype=dtype) + 0.5).to(gpu_device)
-        _say(f"case {n}: B={B} S={S} T={T} C={C} {dtype} {kind} reduction={reduction}")
-        grads = []
-        for handed_out in (True, False):
-            lm_d = lm.to(gpu_device).requires_grad_(True)
-            am_d = am.to(gpu_device).requires_grad_(True)
-            out = fast_rnnt_amd.rnnt_loss_simple(lm_d, am_d, sym.to(gpu_device), C - 1,
-                                                 bnd.to(gpu_device),
-                                                 rnnt_type=kind, reduction=reduction,
-                                                 return_grad=handed_out)
-            loss, occupation = out if handed_out else (out, None)
-            before = [t.clone() for t in occupation] if handed_out else None
-            ((loss * weights).sum() if reduction == "none" else loss * 3.0).backward()
-            if handed_out:
-                # (the in-place scaling, as in the reference: -weights per utterance or -3 / B)
-                factor = -weights if reduction == "none" else torch.full((B,), -3.0 / B, dtype=dtype,
-                                                                          device=gpu_device)
-                for was, now in zip(before, occupation):
-                    assert torch.equal(now, was * factor.view(B, 1, 1))
-            grads.append((lm_d.grad.clone(), am_d.grad.clone()))
-        assert torch.equal(grads[0][0], grads[1][0])
-        assert torch.equal(grads[0][1], grads[1][1])
-
-
 def test_graph_replay_matches_eager(gpu_device):
     """rnnt_loss_simple + backward captured once in a HIP graph and replayed on new input
     values (copied into the captured tensors), with eager steps and synchronisations between
