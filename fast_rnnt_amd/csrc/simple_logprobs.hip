@@ -50,6 +50,55 @@ __device__ __forceinline__ Limits limits_of(const int64_t *window, int b, int S,
   return w;
 }
 
+// Which XCD works on which utterance in the gradient products.  Workgroup i runs on XCD
+// i % 8 and all tiles of an utterance stay on one XCD (xcd_grid.hip.h), so a launch of
+// many tiles lasts as long as its fullest XCD; with utterance b on XCD b % 8 that is left to
+// the order of the batch (ragged batches of 16 and 32 utterances: the fullest XCD 32 % and
+// 19 % above the average).  The prep kernel therefore ranks the utterances by the cells of
+// their windows (rank 0 = most) and the products deal them out by rank: rank r goes to XCD
+// r % 8 in even rounds of eight and to 7 - r % 8 in odd ones, so that every XCD takes its
+// larger utterances first (the same batches: 10 % and 1 % above the average; both products of
+// the larger one 223 -> 210 us).  The utterance of rank r is kept, as an int, in
+// row_x[r][S] -- the row sums of px_grad have no row S, nobody reads that entry as a number
+// -- so a workgroup finds its utterance with one scalar load.  Batches of more than 64 and
+// calls without a window rank by index.
+template <typename R>
+__device__ __forceinline__ int *rank_slot(R *row_x, int r, int S) {
+  return reinterpret_cast<int *>(row_x + (long)r * (S + 1) + S);
+}
+// one wave: ranks the batch and leaves the utterance of every rank in its slot
+template <typename R>
+__device__ __forceinline__ void rank_utterances(R *row_x, const int64_t *window, int B, int S, int T,
+                                                int lane) {
+  if (!window || B > kWave) {
+    for (int i = lane; i < B; i += kWave) *rank_slot(row_x, i, S) = i;
+    return;
+  }
+  unsigned key = 0;  // lanes without an utterance rank behind every utterance
+  if (lane < B) {
+    const Limits w = limits_of(window, lane, S, T);
+    const long cells = (long)max(w.s_end - w.s_begin + 1, 0) * max(w.t_end - w.t_begin, 0);
+    // (distinct keys: equal sizes rank by index)
+    key = ((unsigned)min(cells, 1L << 24) << 6 | (unsigned)(kWave - 1 - lane)) + 1u;
+  }
+  int rank = 0;
+  for (int j = 0; j < B; ++j) rank += (unsigned)__builtin_amdgcn_readlane((int)key, j) > key ? 1 : 0;
+  if (lane < B) *rank_slot(row_x, rank, S) = lane;
+}
+// (utterance, tile, window) of workgroup `id` of a grid of xcd_grid(tiles, B) workgroups
+__device__ __forceinline__ bool place_block(int id, int tiles, int B, const float *row_x,
+                                            const int64_t *window, int S, int T, int &b, int &tile,
+                                            Limits &lim) {
+  using dgemm::kXcds;
+  const int xcd = id % kXcds, slot = id / kXcds, round = slot / tiles;
+  tile = slot % tiles;
+  const int rank = round * kXcds + ((round & 1) ? kXcds - 1 - xcd : xcd);
+  if (rank >= B) return false;
+  b = *reinterpret_cast<const int *>(row_x + (long)rank * (S + 1) + S);
+  lim = limits_of(window, b, S, T);
+  return true;
+}
+
 template <typename R>
 __device__ __forceinline__ R wave_max(R v) {
 #pragma unroll
@@ -189,7 +238,8 @@ __global__ void __launch_bounds__(256)
 // lattice row (b, s): D[b,s,:] and the two row sums.  The remaining ones take 64
 // frames of one utterance each and form the column sums, the four waves splitting
 // the lattice rows.  Loads are issued in batches of four before anything is
-// stored, so a row costs one memory round trip, not one per 64 frames.
+// stored, so a row costs one memory round trip, not one per 64 frames.  The last
+// workgroup ranks the utterances for the gradient products (rank_utterances).
 template <typename R>
 __global__ void __launch_bounds__(256)
     simple_bwd_prep_kernel(const R *__restrict__ gpx, const R *__restrict__ gpy,
@@ -240,9 +290,11 @@ __global__ void __launch_bounds__(256)
     sx = wave_sum(sx);
     sy = wave_sum(sy);
     if (lane == 0) {
-      row_x[row] = sx;
+      if (s < S) row_x[row] = sx;  // (entry S of a row belongs to rank_utterances)
       row_y[row] = sy;
     }
+  } else if (blockIdx.x == gridDim.x - 1) {
+    if (wave == 0) rank_utterances(row_x, window, B, S, T, lane);
   } else {
     const int tiles = (T + kWave - 1) / kWave;
     const long cb = blockIdx.x - row_blocks;
@@ -807,7 +859,8 @@ __device__ __forceinline__ void simple_bwd_lm_slab_body(
   const int S1 = S + 1;
   const int c_tiles = (C + kLmC - 1) / kLmC, s_tiles = (S1 + kLmS - 1) / kLmS;
   int b, tile;
-  if (!decode_block(block_id, c_tiles * s_tiles, B, b, tile)) return;
+  Limits lim;
+  if (!place_block(block_id, c_tiles * s_tiles, B, row_x, window, S, T, b, tile, lim)) return;
   const int s_tile = (tile / c_tiles) * kLmS, c_tile = (tile % c_tiles) * kLmC;
   const float *lmb = lm + (long)b * S1 * C;
   const float *amb = am + (long)b * T * C;
@@ -820,7 +873,6 @@ __device__ __forceinline__ void simple_bwd_lm_slab_body(
   // With a window, D vanishes at frames >= t_end and on rows > s_end: the sum over frames
   // stops at t_end (the row maxima of later frames may not even be defined) and 32-row
   // tiles past s_end are left at 0.
-  const Limits lim = limits_of(window, b, S, T);
   const int t_lim = __builtin_amdgcn_readfirstlane(lim.t_end);
   const int s_lim = __builtin_amdgcn_readfirstlane(min(S1, lim.s_end + 1));
 
@@ -1014,9 +1066,9 @@ __device__ __forceinline__ void simple_bwd_am_panel_body(
     const int64_t *__restrict__ symbols, const int64_t *__restrict__ boundary,
     const float *__restrict__ lm_max, const float *__restrict__ am_max,
     const float *__restrict__ dmat, const float *__restrict__ gpx,
-    const float *__restrict__ col_y, float *__restrict__ am_grad,
-    const int64_t *__restrict__ window, int B, int S, int T, int C, int ldd, int term,
-    int rnnt_type, int rows_cap) {
+    const float *__restrict__ row_x, const float *__restrict__ col_y,
+    float *__restrict__ am_grad, const int64_t *__restrict__ window, int B, int S, int T, int C,
+    int ldd, int term, int rnnt_type, int rows_cap) {
   using namespace dgemm;
   extern __shared__ float am_lds[];
   int *sym_s = reinterpret_cast<int *>(am_lds);   // [rows_cap] symbols of the pass (-1: none)
@@ -1031,7 +1083,8 @@ __device__ __forceinline__ void simple_bwd_am_panel_body(
   const int T1 = rnnt_type == kRegular ? T + 1 : T;
   const int c_tiles = (C + kAmC - 1) / kAmC, t_tiles = (T + kAmT - 1) / kAmT;
   int b, tile;
-  if (!decode_block(block_id, c_tiles * t_tiles, B, b, tile)) return;
+  Limits lim;
+  if (!place_block(block_id, c_tiles * t_tiles, B, row_x, window, S, T, b, tile, lim)) return;
   const int t_tile = (tile / c_tiles) * kAmT, c_tile = (tile % c_tiles) * kAmC;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, r32 = lane & 31;
@@ -1049,7 +1102,6 @@ __device__ __forceinline__ void simple_bwd_am_panel_body(
   // With a window, D vanishes on rows > s_end and at frames >= t_end, where the frames'
   // maxima may not even be defined: such frames get exact zeros, the sum over the lattice
   // rows stops at s_end, and a tile without a frame below t_end only stores zeros.
-  const Limits lim = limits_of(window, b, S, T);
   const int t_lim = lim.t_end, k_lim = min(S1, lim.s_end + 1);
   if (t_tile >= t_lim) {
 #pragma unroll
@@ -1281,13 +1333,13 @@ __global__ void __launch_bounds__(256, kPerCu)
                                const int64_t *__restrict__ boundary,
                                const float *__restrict__ lm_max,
                                const float *__restrict__ am_max, const float *__restrict__ dmat,
-                               const float *__restrict__ gpx, const float *__restrict__ col_y,
-                               float *__restrict__ am_grad, const int64_t *__restrict__ window,
-                               int B, int S, int T, int C, int ldd, int term, int rnnt_type,
-                               int rows_cap) {
+                               const float *__restrict__ gpx, const float *__restrict__ row_x,
+                               const float *__restrict__ col_y, float *__restrict__ am_grad,
+                               const int64_t *__restrict__ window, int B, int S, int T, int C,
+                               int ldd, int term, int rnnt_type, int rows_cap) {
   simple_bwd_am_panel_body<kCap>((int)blockIdx.x, lm, am, symbols, boundary, lm_max, am_max, dmat,
-                                 gpx, col_y, am_grad, window, B, S, T, C, ldd, term, rnnt_type,
-                                 rows_cap);
+                                 gpx, row_x, col_y, am_grad, window, B, S, T, C, ldd, term,
+                                 rnnt_type, rows_cap);
 }
 // Both gradient products in one launch: the first lm_blocks workgroups take tiles of
 // lm.grad, the rest tiles of am.grad.  The two only read what the prep kernel left, so
@@ -1313,9 +1365,9 @@ __global__ void __launch_bounds__(256, 2)
     simple_bwd_lm_slab_body<kS, kK>((int)blockIdx.x, lm, am, symbols, lm_max, am_max, dmat, row_x,
                                     row_y, lm_grad, window, B, S, T, C, ldd, term);
   else
-    simple_bwd_am_panel_body<kAmCap>((int)blockIdx.x - lm_blocks, lm, am, symbols, boundary, lm_max, am_max,
-                             dmat, gpx, col_y, am_grad, window, B, S, T, C, ldd, term, rnnt_type,
-                             rows_cap);
+    simple_bwd_am_panel_body<kAmCap>((int)blockIdx.x - lm_blocks, lm, am, symbols, boundary, lm_max,
+                                     am_max, dmat, gpx, row_x, col_y, am_grad, window, B, S, T, C,
+                                     ldd, term, rnnt_type, rows_cap);
 }
 // lm.grad and am.grad together (float only)
 void launch_bwd_both(const float *lm, const float *am, const int64_t *symbols,
@@ -1371,9 +1423,9 @@ void launch_bwd_lm(const double *lm, const double *am, const int64_t *symbols,
 }
 void launch_bwd_am(const float *lm, const float *am, const int64_t *symbols,
                    const int64_t *boundary, const float *lm_max, const float *am_max,
-                   const float *dmat, const float *gpx, const float *col_y, float *am_grad,
-                   const int64_t *window, int B, int S, int T, int C, int ldd, int term,
-                   int rnnt_type, hipStream_t stream) {
+                   const float *dmat, const float *gpx, const float *row_x, const float *col_y,
+                   float *am_grad, const int64_t *window, int B, int S, int T, int C, int ldd,
+                   int term, int rnnt_type, hipStream_t stream) {
   const int tiles = ((C + kAmC - 1) / kAmC) * ((T + kAmT - 1) / kAmT);
   // rows of k held in LDS per pass: all of them when they fit
   // Rows of k held in LDS per pass: at most 64, in passes of equal size.  The workgroup's
@@ -1388,14 +1440,14 @@ void launch_bwd_am(const float *lm, const float *am, const int64_t *symbols,
   auto kernel = simple_bwd_am_panel_kernel<kAmCap, 4>;
   (void)allow_lds(reinterpret_cast<const void *>(kernel), lds);
   hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(tiles, B)), dim3(256), lds, stream, lm, am,
-                     symbols, boundary, lm_max, am_max, dmat, gpx, col_y, am_grad, window, B, S, T, C,
-                     ldd, term, rnnt_type, rows_cap);
+                     symbols, boundary, lm_max, am_max, dmat, gpx, row_x, col_y, am_grad, window, B, S,
+                     T, C, ldd, term, rnnt_type, rows_cap);
 }
 void launch_bwd_am(const double *lm, const double *am, const int64_t *symbols,
                    const int64_t *boundary, const double *lm_max, const double *am_max,
-                   const double *dmat, const double *gpx, const double *col_y, double *am_grad,
-                   const int64_t *, int B, int S, int T, int C, int ldd, int term, int rnnt_type,
-                   hipStream_t stream) {
+                   const double *dmat, const double *gpx, const double *, const double *col_y,
+                   double *am_grad, const int64_t *, int B, int S, int T, int C, int ldd, int term,
+                   int rnnt_type, hipStream_t stream) {
   const dim3 grid((C + kTileN - 1) / kTileN, (T + kTileM - 1) / kTileM, B);
   hipLaunchKernelGGL(simple_bwd_am_kernel<double>, grid, dim3(kGemmThreads), 0, stream, lm, am,
                      lm_max, am_max, dmat, col_y, am_grad, S, T, C, ldd, term);
@@ -1477,7 +1529,7 @@ int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
   const int ldd = (T + 3) & ~3;  // leading dimension of dmat: 16-byte rows
   // (the double kernels ignore the window: they take the whole lattice as it is)
   const int64_t *window = (window_only && std::is_same<R, float>::value) ? boundary : nullptr;
-  const long prep_blocks = ((long)B * (S + 1) + 3) / 4 + (long)B * ((T + kWave - 1) / kWave);
+  const long prep_blocks = ((long)B * (S + 1) + 3) / 4 + (long)B * ((T + kWave - 1) / kWave) + 1;
   hipLaunchKernelGGL(simple_bwd_prep_kernel<R>, dim3((unsigned)prep_blocks), dim3(256), 0, stream,
                      px_grad, py_grad, norm_raw, boundary, window, dmat, row_x, row_y, col_y, B, S, T,
                      ldd, rnnt_type);
@@ -1493,7 +1545,7 @@ int bwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
     launch_bwd_lm(lm, am, symbols, lm_max, am_max, dmat, row_x, row_y, lm_grad, window, B, S, T, C,
                   ldd, term, stream);
   if (am_grad && T > 0)
-    launch_bwd_am(lm, am, symbols, boundary, lm_max, am_max, dmat, px_grad, col_y, am_grad, window,
+    launch_bwd_am(lm, am, symbols, boundary, lm_max, am_max, dmat, px_grad, row_x, col_y, am_grad, window,
                   B, S, T, C, ldd, term, rnnt_type, stream);
   return check_launch("simple_logprobs_bwd");
 }

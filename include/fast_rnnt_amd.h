@@ -150,6 +150,9 @@ int frnnt_simple_logprobs_fwd_f64(const double *lm, const double *am, const int6
  *     rnnt_loss.py:160-169 in score_grad_scale)
  *   dmat [B][S+1][T rounded up to a multiple of 4], row_x [B][S+1], row_y [B][S+1],
  *   col_y [B][T]                                                           scratch
+ *     (what the library keeps there is its own business: besides D and its row and column
+ *     sums, the last entry of every row of row_x holds, as an int, the order in which the
+ *     utterances are dealt out to the XCDs)
  *   lm_grad [B][S+1][C], am_grad [B][T][C]: out; either may be NULL to skip it
  *   window_only: 1 (with a boundary) = px_grad / py_grad vanish outside each utterance's
  *   boundary window, as the recursion's backward leaves them: nothing outside is read,

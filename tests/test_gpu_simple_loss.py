@@ -170,6 +170,36 @@ def test_loss_and_all_gradients(gpu_device, dtype, kind):
             assert _close(gx, wx, gtol) and _close(gy, wy, gtol)
 
 
+@pytest.mark.parametrize("B", [1, 7, 13, 23, 64, 70])
+def test_batch_sizes_around_the_ranking_of_utterances(gpu_device, B):
+    # The gradient products deal the utterances out to the XCDs by the size of their
+    # windows: batches that do not fill a round of eight, equal sizes (ties), one utterance
+    # much larger than the rest, a minimal window, and a batch too large to be ranked by one wave.
+    dev = gpu_device
+    S, T, C = 9, 21, 40
+    _say(f"ranking B={B}")
+    am, lm, sym, bnd = _case(300 + B, B, S, T, C, torch.float32, "regular")
+    bnd[:, 2] = torch.tensor([(3 * i) % S + 1 for i in range(B)])
+    bnd[:, 3] = torch.tensor([(5 * i) % (T - 2) + 2 for i in range(B)])
+    bnd[0, 2], bnd[0, 3] = S, T
+    if B > 3:
+        bnd[2] = bnd[1]                       # a tie
+        bnd[3, 2], bnd[3, 3] = 1, 1           # the smallest window the losses accept
+    a = am.clone().requires_grad_(True)
+    l = lm.clone().requires_grad_(True)
+    want = O.loss_simple(l, a, sym, 0, boundary=bnd, reduction="none")
+    weights = torch.linspace(0.5, 1.5, B)
+    (want * weights).sum().backward()
+    da = am.to(dev).requires_grad_(True)
+    dl = lm.to(dev).requires_grad_(True)
+    got = fast_rnnt_amd.rnnt_loss_simple(dl, da, sym.to(dev), 0, boundary=bnd.to(dev),
+                                         reduction="none")
+    (got * weights.to(dev)).sum().backward()
+    assert _close(got, want, 0.0, 1e-5)
+    assert _close(da.grad, a.grad, 1e-4, 1e-4), (da.grad.cpu() - a.grad).abs().max()
+    assert _close(dl.grad, l.grad, 1e-4, 1e-4), (dl.grad.cpu() - l.grad).abs().max()
+
+
 @pytest.mark.parametrize("kind", KINDS)
 def test_fused_loss_ignores_frames_past_the_window(gpu_device, kind):
     # rnnt_loss_simple works on each utterance's window only: NaN planted (on the GPU side)
