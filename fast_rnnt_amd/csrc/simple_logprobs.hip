@@ -51,7 +51,7 @@ __device__ __forceinline__ Limits limits_of(const int64_t *window, int b, int S,
 }
 
 // Which XCD works on which utterance in the gradient products.  Workgroup i runs on XCD
-// i % 8 and all tiles of an utterance stay on one XCD (xcd_grid.hip.h), so a launch of
+// i % 8 and all tiles of an utterance stay on one XCD (one L2 holds its operands), so a launch of
 // many tiles lasts as long as its fullest XCD; with utterance b on XCD b % 8 that is left to
 // the order of the batch (ragged batches of 16 and 32 utterances: the fullest XCD 32 % and
 // 19 % above the average).  The prep kernel therefore ranks the utterances by the cells of
@@ -85,15 +85,59 @@ __device__ __forceinline__ void rank_utterances(R *row_x, const int64_t *window,
   for (int j = 0; j < B; ++j) rank += (unsigned)__builtin_amdgcn_readlane((int)key, j) > key ? 1 : 0;
   if (lane < B) *rank_slot(row_x, rank, S) = lane;
 }
-// (utterance, tile, window) of workgroup `id` of a grid of xcd_grid(tiles, B) workgroups
-__device__ __forceinline__ bool place_block(int id, int tiles, int B, const float *row_x,
-                                            const int64_t *window, int S, int T, int &b, int &tile,
-                                            Limits &lim) {
+// With fewer than 32 utterances a unit of placement is a PART of an utterance: its tiles
+// of every 2^part_shift-th stretch of the vocabulary (such tiles share D but nothing of lm or
+// am), enough parts for eight units per XCD while a part keeps four tiles along the
+// vocabulary.  A batch of two then reaches all eight XCDs instead of two (B = 2, S = 100,
+// T = 400, C = 5000: both products 117 -> 36 us), and a batch of sixteen is dealt out in 64
+// units (fullest XCD 2 % above the average instead of 10 %: 212 -> 201 us).
+inline int part_shift_for(int B, int c_tiles) {
+  if (B >= 32) return 0;
+  int shift = 0;
+  while ((B << shift) < 64 && (8 << shift) <= c_tiles) ++shift;
+  return shift;
+}
+inline unsigned placed_grid(int c_tiles, int other_tiles, int B, int part_shift) {
+  const long units = (long)B << part_shift;
+  const int c_per = (c_tiles + (1 << part_shift) - 1) >> part_shift;
+  return (unsigned)(dgemm::kXcds * ((units + dgemm::kXcds - 1) / dgemm::kXcds) * c_per * other_tiles);
+}
+// The normalizer kernel is the first of its call (no ranks yet): utterance b stays on XCD
+// b % 8, and a batch of fewer than eight is cut into parts along the frames until it reaches
+// every XCD (the parts of an utterance share its lm rows, the small operand).
+inline int frame_part_shift_for(int B, int t_tiles) {
+  int shift = 0;
+  while ((B << shift) < dgemm::kXcds && (2 << shift) <= t_tiles) ++shift;
+  return shift;
+}
+__device__ __forceinline__ bool place_frames(int id, int t_tiles, int s_tiles, int part_shift, int B,
+                                             int &b, int &s_idx, int &t_idx) {
   using dgemm::kXcds;
-  const int xcd = id % kXcds, slot = id / kXcds, round = slot / tiles;
-  tile = slot % tiles;
-  const int rank = round * kXcds + ((round & 1) ? kXcds - 1 - xcd : xcd);
-  if (rank >= B) return false;
+  const int t_per = (t_tiles + (1 << part_shift) - 1) >> part_shift;
+  const int unit_tiles = t_per * s_tiles;
+  const int xcd = id % kXcds, slot = id / kXcds, round = slot / unit_tiles;
+  const int within = slot - round * unit_tiles;
+  const int unit = round * kXcds + xcd;
+  b = unit >> part_shift;
+  s_idx = within / t_per;
+  t_idx = (unit & ((1 << part_shift) - 1)) * t_per + (within - s_idx * t_per);
+  return b < B && t_idx < t_tiles;
+}
+// (utterance, tile, window) of workgroup `id` of a grid of placed_grid() workgroups; a tile is
+// other * c_tiles + (its index along the vocabulary)
+__device__ __forceinline__ bool place_block(int id, int c_tiles, int other_tiles, int part_shift,
+                                            int B, const float *row_x, const int64_t *window, int S,
+                                            int T, int &b, int &tile, Limits &lim) {
+  using dgemm::kXcds;
+  const int c_per = (c_tiles + (1 << part_shift) - 1) >> part_shift;
+  const int unit_tiles = c_per * other_tiles;
+  const int xcd = id % kXcds, slot = id / kXcds, round = slot / unit_tiles;
+  const int within = slot - round * unit_tiles;
+  const int unit = round * kXcds + ((round & 1) ? kXcds - 1 - xcd : xcd);
+  const int rank = unit >> part_shift, part = unit & ((1 << part_shift) - 1);
+  const int other = within / c_per, c_idx = part * c_per + (within - other * c_per);
+  if (rank >= B || c_idx >= c_tiles) return false;
+  tile = other * c_tiles + c_idx;
   b = *reinterpret_cast<const int *>(row_x + (long)rank * (S + 1) + S);
   lim = limits_of(window, b, S, T);
   return true;
@@ -511,7 +555,7 @@ __global__ void __launch_bounds__(kPanThreads)
                             float *__restrict__ lm_max, float *__restrict__ am_max,
                             float *__restrict__ px, float *__restrict__ py,
                             float *__restrict__ norm_raw, const int64_t *__restrict__ window,
-                            int B, int S, int T, int C, int term, int rnnt_type) {
+                            int B, int S, int T, int C, int term, int rnnt_type, int part_shift) {
   using Shape = PanelShape<kS, kK>;
   constexpr int kPanS = kS, kPanK = kK, kPanRows = Shape::kRows, kPanPitch = Shape::kPitch;
   constexpr int kPanSlab = Shape::kSlab, kPanItems = Shape::kItems;
@@ -527,9 +571,9 @@ __global__ void __launch_bounds__(kPanThreads)
   __shared__ float col_term[kPanT], col_max[kPanT];                  // am[t,term], am_max[t]
   const int S1 = S + 1;
   const int t_tiles = T > 0 ? (T + kPanT - 1) / kPanT : 1, s_tiles = (S1 + kPanS - 1) / kPanS;
-  int b, tile;
-  if (!decode_block(t_tiles * s_tiles, B, b, tile)) return;
-  const int s_tile = (tile / t_tiles) * kPanS, t_tile = (tile % t_tiles) * kPanT;
+  int b, s_idx, t_idx;
+  if (!place_frames((int)blockIdx.x, t_tiles, s_tiles, part_shift, B, b, s_idx, t_idx)) return;
+  const int s_tile = s_idx * kPanS, t_tile = t_idx * kPanT;
   const int T1 = rnnt_type == kRegular ? T + 1 : T;
   // With a window only rows <= s_end and frames <= t_end are looked at afterwards (frame
   // t_end itself only for the -inf that closes the regular lattice): a tile past t_end has
@@ -850,7 +894,7 @@ __device__ __forceinline__ void simple_bwd_lm_slab_body(
     const float *__restrict__ am_max, const float *__restrict__ dmat,
     const float *__restrict__ row_x, const float *__restrict__ row_y,
     float *__restrict__ lm_grad, const int64_t *__restrict__ window, int B, int S, int T, int C,
-    int ldd, int term) {
+    int ldd, int term, int part_shift) {
   using Shape = LmShape<kS, kK>;
   constexpr int kLmS = kS, kLmK = kK, kLmPitch = Shape::kPitch, kLmSlab = Shape::kSlab;
   constexpr int kLmItems = Shape::kItems;
@@ -860,7 +904,8 @@ __device__ __forceinline__ void simple_bwd_lm_slab_body(
   const int c_tiles = (C + kLmC - 1) / kLmC, s_tiles = (S1 + kLmS - 1) / kLmS;
   int b, tile;
   Limits lim;
-  if (!place_block(block_id, c_tiles * s_tiles, B, row_x, window, S, T, b, tile, lim)) return;
+  if (!place_block(block_id, c_tiles, s_tiles, part_shift, B, row_x, window, S, T, b, tile, lim))
+    return;
   const int s_tile = (tile / c_tiles) * kLmS, c_tile = (tile % c_tiles) * kLmC;
   const float *lmb = lm + (long)b * S1 * C;
   const float *amb = am + (long)b * T * C;
@@ -1068,7 +1113,7 @@ __device__ __forceinline__ void simple_bwd_am_panel_body(
     const float *__restrict__ dmat, const float *__restrict__ gpx,
     const float *__restrict__ row_x, const float *__restrict__ col_y,
     float *__restrict__ am_grad, const int64_t *__restrict__ window, int B, int S, int T, int C,
-    int ldd, int term, int rnnt_type, int rows_cap) {
+    int ldd, int term, int rnnt_type, int rows_cap, int part_shift) {
   using namespace dgemm;
   extern __shared__ float am_lds[];
   int *sym_s = reinterpret_cast<int *>(am_lds);   // [rows_cap] symbols of the pass (-1: none)
@@ -1084,7 +1129,8 @@ __device__ __forceinline__ void simple_bwd_am_panel_body(
   const int c_tiles = (C + kAmC - 1) / kAmC, t_tiles = (T + kAmT - 1) / kAmT;
   int b, tile;
   Limits lim;
-  if (!place_block(block_id, c_tiles * t_tiles, B, row_x, window, S, T, b, tile, lim)) return;
+  if (!place_block(block_id, c_tiles, t_tiles, part_shift, B, row_x, window, S, T, b, tile, lim))
+    return;
   const int t_tile = (tile / c_tiles) * kAmT, c_tile = (tile % c_tiles) * kAmC;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, r32 = lane & 31;
@@ -1285,9 +1331,14 @@ void launch_fwd_panel(const float *lm, const float *am, const int64_t *symbols,
   const int s_tiles = (S + 1 + kS - 1) / kS;
   auto kernel = simple_fwd_panel_kernel<kS, kK>;
   (void)allow_lds(reinterpret_cast<const void *>(kernel), Shape::kLdsBytes);
-  hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(t_tiles * s_tiles, B)), dim3(kPanThreads),
-                     Shape::kLdsBytes, stream, lm, am, symbols, boundary, lm_max, am_max, px, py,
-                     norm_raw, window, B, S, T, C, term, rnnt_type);
+  const int shift = frame_part_shift_for(B, t_tiles);
+  const int t_per = (t_tiles + (1 << shift) - 1) >> shift;
+  const long units = (long)B << shift;
+  const unsigned grid =
+      (unsigned)(dgemm::kXcds * ((units + dgemm::kXcds - 1) / dgemm::kXcds) * t_per * s_tiles);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(kPanThreads), Shape::kLdsBytes, stream, lm, am,
+                     symbols, boundary, lm_max, am_max, px, py, norm_raw, window, B, S, T, C, term,
+                     rnnt_type, shift);
 }
 void launch_fwd_gemm(const float *lm, const float *am, const int64_t *symbols,
                      const int64_t *boundary, float *lm_max, float *am_max, float *px,
@@ -1322,9 +1373,9 @@ __global__ void __launch_bounds__(kLmThreads, 2)
                               const float *__restrict__ am_max, const float *__restrict__ dmat,
                               const float *__restrict__ row_x, const float *__restrict__ row_y,
                               float *__restrict__ lm_grad, const int64_t *__restrict__ window,
-                              int B, int S, int T, int C, int ldd, int term) {
+                              int B, int S, int T, int C, int ldd, int term, int part_shift) {
   simple_bwd_lm_slab_body<kS, kK>((int)blockIdx.x, lm, am, symbols, lm_max, am_max, dmat, row_x,
-                                  row_y, lm_grad, window, B, S, T, C, ldd, term);
+                                  row_y, lm_grad, window, B, S, T, C, ldd, term, part_shift);
 }
 template <int kCap, int kPerCu>
 __global__ void __launch_bounds__(256, kPerCu)
@@ -1336,10 +1387,10 @@ __global__ void __launch_bounds__(256, kPerCu)
                                const float *__restrict__ gpx, const float *__restrict__ row_x,
                                const float *__restrict__ col_y, float *__restrict__ am_grad,
                                const int64_t *__restrict__ window, int B, int S, int T, int C,
-                               int ldd, int term, int rnnt_type, int rows_cap) {
+                               int ldd, int term, int rnnt_type, int rows_cap, int part_shift) {
   simple_bwd_am_panel_body<kCap>((int)blockIdx.x, lm, am, symbols, boundary, lm_max, am_max, dmat,
                                  gpx, row_x, col_y, am_grad, window, B, S, T, C, ldd, term,
-                                 rnnt_type, rows_cap);
+                                 rnnt_type, rows_cap, part_shift);
 }
 // Both gradient products in one launch: the first lm_blocks workgroups take tiles of
 // lm.grad, the rest tiles of am.grad.  The two only read what the prep kernel left, so
@@ -1360,14 +1411,14 @@ __global__ void __launch_bounds__(256, 2)
                             const float *__restrict__ col_y, float *__restrict__ lm_grad,
                             float *__restrict__ am_grad, const int64_t *__restrict__ window, int B,
                             int S, int T, int C, int ldd, int term, int rnnt_type, int rows_cap,
-                            int lm_blocks) {
+                            int lm_blocks, int lm_part_shift, int am_part_shift) {
   if ((int)blockIdx.x < lm_blocks)
     simple_bwd_lm_slab_body<kS, kK>((int)blockIdx.x, lm, am, symbols, lm_max, am_max, dmat, row_x,
-                                    row_y, lm_grad, window, B, S, T, C, ldd, term);
+                                    row_y, lm_grad, window, B, S, T, C, ldd, term, lm_part_shift);
   else
     simple_bwd_am_panel_body<kAmCap>((int)blockIdx.x - lm_blocks, lm, am, symbols, boundary, lm_max,
                                      am_max, dmat, gpx, row_x, col_y, am_grad, window, B, S, T, C,
-                                     ldd, term, rnnt_type, rows_cap);
+                                     ldd, term, rnnt_type, rows_cap, am_part_shift);
 }
 // lm.grad and am.grad together (float only)
 void launch_bwd_both(const float *lm, const float *am, const int64_t *symbols,
@@ -1379,19 +1430,21 @@ void launch_bwd_both(const float *lm, const float *am, const int64_t *symbols,
   const int S1 = S + 1;
   const bool rows96 = (S1 + 95) / 96 * 96 < (S1 + 127) / 128 * 128;
   const int rows = rows96 ? 96 : 128;
-  const int lm_tiles = ((C + kLmC - 1) / kLmC) * ((S1 + rows - 1) / rows);
-  const int am_tiles = ((C + kAmC - 1) / kAmC) * ((T + kAmT - 1) / kAmT);
+  const int lm_c = (C + kLmC - 1) / kLmC, am_c = (C + kAmC - 1) / kAmC;
+  const int lm_shift = part_shift_for(B, lm_c), am_shift = part_shift_for(B, am_c);
   const int rows_cap = am_rows_per_pass(S);
   // (frames in slabs of 16 here also for the 96-row form: its LDS is then 50 KB, not 67,
   // and three workgroups fit on a CU whichever product they work on: 33.4 us against 36.2)
   const size_t lm_lds = rows96 ? LmShape<96, 16>::kLdsBytes : LmShape<128, 16>::kLdsBytes;
   const size_t lds = std::max(lm_lds, am_panel_lds_bytes(rows_cap));
-  const unsigned am_blocks = dgemm::xcd_grid(am_tiles, B), lm_blocks = dgemm::xcd_grid(lm_tiles, B);
+  const unsigned am_blocks = placed_grid(am_c, (T + kAmT - 1) / kAmT, B, am_shift);
+  const unsigned lm_blocks = placed_grid(lm_c, (S1 + rows - 1) / rows, B, lm_shift);
   auto kernel = rows96 ? simple_bwd_am_lm_kernel<96, 16> : simple_bwd_am_lm_kernel<128, 16>;
   (void)allow_lds(reinterpret_cast<const void *>(kernel), lds);
   hipLaunchKernelGGL(kernel, dim3(am_blocks + lm_blocks), dim3(256), lds, stream, lm, am, symbols,
                      boundary, lm_max, am_max, dmat, gpx, row_x, row_y, col_y, lm_grad, am_grad,
-                     window, B, S, T, C, ldd, term, rnnt_type, rows_cap, (int)lm_blocks);
+                     window, B, S, T, C, ldd, term, rnnt_type, rows_cap, (int)lm_blocks, lm_shift,
+                     am_shift);
 }
 void launch_bwd_both(const double *, const double *, const int64_t *, const int64_t *,
                      const double *, const double *, const double *, const double *,
@@ -1405,13 +1458,13 @@ void launch_bwd_lm(const float *lm, const float *am, const int64_t *symbols, con
   const int S1 = S + 1;
   const bool rows96 = (S1 + 95) / 96 * 96 < (S1 + 127) / 128 * 128;
   const int rows = rows96 ? 96 : 128;
-  const int tiles = ((C + kLmC - 1) / kLmC) * ((S1 + rows - 1) / rows);
+  const int c_tiles = (C + kLmC - 1) / kLmC, shift = part_shift_for(B, c_tiles);
   auto kernel = rows96 ? simple_bwd_lm_slab_kernel<96, 32> : simple_bwd_lm_slab_kernel<128, 16>;
   const size_t lds = rows96 ? LmShape<96, 32>::kLdsBytes : LmShape<128, 16>::kLdsBytes;
   (void)allow_lds(reinterpret_cast<const void *>(kernel), lds);
-  hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(tiles, B)), dim3(kLmThreads), lds, stream, lm,
-                     am, symbols, lm_max, am_max, dmat, row_x, row_y, lm_grad, window, B, S, T, C,
-                     ldd, term);
+  hipLaunchKernelGGL(kernel, dim3(placed_grid(c_tiles, (S1 + rows - 1) / rows, B, shift)),
+                     dim3(kLmThreads), lds, stream, lm, am, symbols, lm_max, am_max, dmat, row_x,
+                     row_y, lm_grad, window, B, S, T, C, ldd, term, shift);
 }
 void launch_bwd_lm(const double *lm, const double *am, const int64_t *symbols,
                    const double *lm_max, const double *am_max, const double *dmat,
@@ -1426,7 +1479,7 @@ void launch_bwd_am(const float *lm, const float *am, const int64_t *symbols,
                    const float *dmat, const float *gpx, const float *row_x, const float *col_y,
                    float *am_grad, const int64_t *window, int B, int S, int T, int C, int ldd,
                    int term, int rnnt_type, hipStream_t stream) {
-  const int tiles = ((C + kAmC - 1) / kAmC) * ((T + kAmT - 1) / kAmT);
+  const int c_tiles = (C + kAmC - 1) / kAmC, shift = part_shift_for(B, c_tiles);
   // rows of k held in LDS per pass: all of them when they fit
   // Rows of k held in LDS per pass: at most 64, in passes of equal size.  The workgroup's
   // phases (panels in, exp, products, results out) do not overlap inside it, so the compute
@@ -1439,9 +1492,9 @@ void launch_bwd_am(const float *lm, const float *am, const int64_t *symbols,
   // (the 16-byte accesses need no alignment)
   auto kernel = simple_bwd_am_panel_kernel<kAmCap, 4>;
   (void)allow_lds(reinterpret_cast<const void *>(kernel), lds);
-  hipLaunchKernelGGL(kernel, dim3(dgemm::xcd_grid(tiles, B)), dim3(256), lds, stream, lm, am,
-                     symbols, boundary, lm_max, am_max, dmat, gpx, row_x, col_y, am_grad, window, B, S,
-                     T, C, ldd, term, rnnt_type, rows_cap);
+  hipLaunchKernelGGL(kernel, dim3(placed_grid(c_tiles, (T + kAmT - 1) / kAmT, B, shift)), dim3(256),
+                     lds, stream, lm, am, symbols, boundary, lm_max, am_max, dmat, gpx, row_x, col_y,
+                     am_grad, window, B, S, T, C, ldd, term, rnnt_type, rows_cap, shift);
 }
 void launch_bwd_am(const double *lm, const double *am, const int64_t *symbols,
                    const int64_t *boundary, const double *lm_max, const double *am_max,

@@ -170,14 +170,17 @@ def test_loss_and_all_gradients(gpu_device, dtype, kind):
             assert _close(gx, wx, gtol) and _close(gy, wy, gtol)
 
 
-@pytest.mark.parametrize("B", [1, 7, 13, 23, 64, 70])
-def test_batch_sizes_around_the_ranking_of_utterances(gpu_device, B):
+@pytest.mark.parametrize("B,C", [(1, 40), (1, 1100), (3, 2100), (7, 600), (13, 40), (23, 300),
+                                 (64, 40), (70, 40)])
+def test_batch_sizes_around_the_ranking_of_utterances(gpu_device, B, C):
     # The gradient products deal the utterances out to the XCDs by the size of their
     # windows: batches that do not fill a round of eight, equal sizes (ties), one utterance
     # much larger than the rest, a minimal window, and a batch too large to be ranked by one wave.
+    # Small batches with a large vocabulary are dealt out in parts of utterances (vocabulary
+    # sizes whose tile counts do and do not divide by the number of parts).
     dev = gpu_device
-    S, T, C = 9, 21, 40
-    _say(f"ranking B={B}")
+    S, T = 9, 21
+    _say(f"ranking B={B} C={C}")
     am, lm, sym, bnd = _case(300 + B, B, S, T, C, torch.float32, "regular")
     bnd[:, 2] = torch.tensor([(3 * i) % S + 1 for i in range(B)])
     bnd[:, 3] = torch.tensor([(5 * i) % (T - 2) + 2 for i in range(B)])
