@@ -22,5 +22,7 @@ from .rnnt_loss import rnnt_loss_pruned
 from .rnnt_loss import rnnt_loss_simple
 from .rnnt_loss import rnnt_loss_smoothed
 
-# beyond the reference's export list: the joiner's input without the gathered copy
+# beyond the reference's export list: the joiner's input without the gathered copy, and
+# where the rows of a boundary tensor are asserted (on the device, raised later, by default)
 from .rnnt_loss import pruned_joiner_input
+from .mutual_information import check_boundaries, set_boundary_checks

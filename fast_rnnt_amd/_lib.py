@@ -1,8 +1,11 @@
-"""ctypes binding of libfast_rnnt_amd.so (the gfx950 C-ABI library).
+"""The two native pieces of this package: libfast_rnnt_amd.so (the gfx950 C-ABI
+library, bound here with ctypes for the operators that are not on the per-step hot
+path and for tests of the raw ABI) and the compiled torch operator module
+``fast_rnnt_amd._C`` that sits on top of it (:func:`ops`).
 
-The library is built in-tree by ``make -C fast_rnnt_amd/csrc`` (or
-``__graft_entry__.build()``).  There is no fallback: if it is missing, loading
-raises, and every operator of this package needs it.
+Both are built in-tree by ``make -C fast_rnnt_amd/csrc`` (or
+``__graft_entry__.build()``).  There is no fallback: if one is missing, loading
+raises, and every operator of this package needs them.
 """
 import ctypes
 import os
@@ -28,6 +31,8 @@ _SIGNATURES = {
     "frnnt_set_spin_limit": ([_I], None),
     "frnnt_mi_forward_f32": ([_P, _P, _P, _P, _P, _I, _I, _I, _I, _P], _I),
     "frnnt_mi_forward_f64": ([_P, _P, _P, _P, _P, _I, _I, _I, _I, _P], _I),
+    "frnnt_mi_forward_checked_f32": ([_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P], _I),
+    "frnnt_mi_forward_checked_f64": ([_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P], _I),
     "frnnt_mi_backward_f32": ([_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P], _I),
     "frnnt_mi_backward_f64": ([_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P], _I),
     "frnnt_simple_logprobs_fwd_f32": ([_P] * 9 + [_I] * 7 + [_P], _I),
@@ -39,10 +44,10 @@ _SIGNATURES = {
     "frnnt_smoothed_logprobs_fwd_f64": ([_P] * 14 + [_I] * 6 + [_D, _D, _P], _I),
     "frnnt_smoothed_logprobs_bwd_f32": ([_P] * 21 + [_I] * 6 + [_D, _D, _P], _I),
     "frnnt_smoothed_logprobs_bwd_f64": ([_P] * 21 + [_I] * 6 + [_D, _D, _P], _I),
-    "frnnt_simple_loss_fwd_f32": ([_P] * 14 + [_I] * 7 + [_P], _I),
-    "frnnt_simple_loss_fwd_f64": ([_P] * 14 + [_I] * 7 + [_P], _I),
-    "frnnt_mi_loss_fwd_f32": ([_P] * 8 + [_I] * 5 + [_P], _I),
-    "frnnt_mi_loss_fwd_f64": ([_P] * 8 + [_I] * 5 + [_P], _I),
+    "frnnt_simple_loss_fwd_f32": ([_P] * 14 + [_I] * 8 + [_P, _P], _I),
+    "frnnt_simple_loss_fwd_f64": ([_P] * 14 + [_I] * 8 + [_P, _P], _I),
+    "frnnt_mi_loss_fwd_f32": ([_P] * 8 + [_I] * 6 + [_P, _P], _I),
+    "frnnt_mi_loss_fwd_f64": ([_P] * 8 + [_I] * 6 + [_P, _P], _I),
     "frnnt_mi_scale_grads_f32": ([_P] * 3 + [_I, _D] + [_I] * 4 + [_P], _I),
     "frnnt_mi_scale_grads_f64": ([_P] * 3 + [_I, _D] + [_I] * 4 + [_P], _I),
     "frnnt_loss_reduce_f32": ([_P, _P, _I, _I, _P], _I),
@@ -95,6 +100,28 @@ def load():
             fn.restype = restype
         _lib = lib
     return _lib
+
+
+_ops = None
+
+
+def ops():
+    """The compiled torch operator module ``fast_rnnt_amd._C`` (csrc/torch_ops.cpp): the
+    reference's three operator functions and the loss nodes, also registered as
+    ``torch.ops.fast_rnnt_amd.*``.  Built in-tree beside the library by
+    ``make -C fast_rnnt_amd/csrc``; raises RuntimeError if it is missing."""
+    global _ops
+    if _ops is None:
+        load()  # the module links against the library: fail with the build hint first
+        try:
+            from . import _C
+        except ImportError as e:
+            raise RuntimeError(
+                f"fast_rnnt_amd/_C*.so cannot be imported ({e}): build it with "
+                "`make -C fast_rnnt_amd/csrc` (g++ against the installed torch). "
+                "fast_rnnt_amd has no CPU or eager fallback.") from e
+        _ops = _C
+    return _ops
 
 
 def call(name, *args):

@@ -68,6 +68,10 @@ struct Window {
   int s0, t0, ns, nt;  // origin and extent (ns = s_end - s_begin, ...)
   bool ok;
 };
+// `checks` bits and `status[0]` codes of the forward kernel (FRNNT_CHECK_* / FRNNT_STATUS_*
+// of the public header)
+constexpr int kCheckSymbols = 1, kCheckFrames = 2;
+constexpr int kStatusWindow = 1, kStatusNoSymbols = 2, kStatusFewFrames = 3;
 
 __device__ __forceinline__ Window load_window(const int64_t *boundary, int b, int S, int T) {
   Window w{0, 0, S, T, true};
@@ -302,7 +306,8 @@ template <typename R, bool kModified, int kSweepCap, int kStagers, int kBuffers>
 __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
     mi_forward_kernel(const R *__restrict__ px, const R *__restrict__ py,
                       const int64_t *__restrict__ boundary, R *__restrict__ p,
-                      R *__restrict__ ans, int S, int T, int spin_limit) {
+                      R *__restrict__ ans, int S, int T, int spin_limit, int checks,
+                      int *__restrict__ status) {
   extern __shared__ __align__(16) unsigned char dyn_lds[];
   __shared__ Counters cnt;
 
@@ -316,8 +321,23 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
   const R ninf = Num<R>::neg_inf();
 
   const Window win = load_window(boundary, b, S, T);
-  if (!win.ok) {
-    if (threadIdx.x == 0) ans[b] = std::numeric_limits<R>::quiet_NaN();
+  // What the loss functions assert of a boundary row before they call the recursion
+  // (rnnt_loss.py:25-42), for callers that do not want to wait for a host copy of the rows:
+  // a row that fails is treated like one whose window is out of range, and `status` -- memory
+  // the host can read, e.g. pinned host memory -- names the failed test and the row.
+  int bad = win.ok ? 0 : kStatusWindow;
+  if (checks != 0 && boundary != nullptr && win.ok) {
+    if ((checks & kCheckSymbols) && win.s0 + win.ns < 1) bad = kStatusNoSymbols;
+    else if ((checks & kCheckFrames) && win.t0 + win.nt < win.s0 + win.ns) bad = kStatusFewFrames;
+  }
+  if (bad != 0) {
+    if (threadIdx.x == 0) {
+      ans[b] = std::numeric_limits<R>::quiet_NaN();
+      if (status) {
+        status[1] = b;
+        status[0] = bad;
+      }
+    }
     return;
   }
   if (threadIdx.x < (int)(sizeof(Counters) / sizeof(int)))
@@ -1117,7 +1137,7 @@ size_t lds_bytes(int nsweep, int T, int buffers, size_t elem) {
 
 template <typename R>
 int forward_impl(const R *px, const R *py, const int64_t *boundary, R *p, R *ans, int B, int S,
-                 int T, int modified, void *stream) {
+                 int T, int modified, void *stream, int checks = 0, int *status = nullptr) {
   if (B < 0 || S < 0 || T < 0) return fail(FRNNT_EINVAL, "mi_forward: negative size");
   if (B == 0) return FRNNT_OK;
   if (!px || !py || !p || !ans) return fail(FRNNT_EINVAL, "mi_forward: null pointer");
@@ -1143,7 +1163,8 @@ int forward_impl(const R *px, const R *py, const int64_t *boundary, R *p, R *ans
   if (!allow_lds(reinterpret_cast<const void *>(kernel), lds))
     return check_launch("mi_forward: hipFuncSetAttribute");
   hipLaunchKernelGGL(kernel, dim3(B), dim3(n * (1 + stagers) * kWave), lds,
-                     static_cast<hipStream_t>(stream), px, py, boundary, p, ans, S, T, g_spin_limit);
+                     static_cast<hipStream_t>(stream), px, py, boundary, p, ans, S, T, g_spin_limit,
+                     checks, status);
   return check_launch("mi_forward");
 }
 
@@ -1217,6 +1238,18 @@ int frnnt_mi_forward_f32(const float *px, const float *py, const int64_t *bounda
 int frnnt_mi_forward_f64(const double *px, const double *py, const int64_t *boundary, double *p,
                          double *ans, int B, int S, int T, int modified, void *stream) {
   return frnnt::forward_impl<double>(px, py, boundary, p, ans, B, S, T, modified, stream);
+}
+int frnnt_mi_forward_checked_f32(const float *px, const float *py, const int64_t *boundary,
+                                 float *p, float *ans, int B, int S, int T, int modified,
+                                 int checks, int32_t *status, void *stream) {
+  return frnnt::forward_impl<float>(px, py, boundary, p, ans, B, S, T, modified, stream, checks,
+                                    status);
+}
+int frnnt_mi_forward_checked_f64(const double *px, const double *py, const int64_t *boundary,
+                                 double *p, double *ans, int B, int S, int T, int modified,
+                                 int checks, int32_t *status, void *stream) {
+  return frnnt::forward_impl<double>(px, py, boundary, p, ans, B, S, T, modified, stream, checks,
+                                     status);
 }
 int frnnt_mi_backward_f32(const float *px, const float *py, const int64_t *boundary,
                           const float *p, float *ans_grad, float *px_grad, float *py_grad, int B,

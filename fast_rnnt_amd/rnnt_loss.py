@@ -20,21 +20,25 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from .mutual_information import (_assert_boundary, boundary_rows,
+from .mutual_information import (_assert_boundary, boundary_rows,  # noqa: F401
                                  mutual_information_recursion)
 
 _RNNT_TYPES = {"regular": 0, "modified": 1, "constrained": 2}
 
 
 def validate_st_lengths(S: int, T: int, is_rnnt_type_regular: bool,
-                        boundary: Optional[Tensor] = None):
+                        boundary: Optional[Tensor] = None, on_device: bool = False):
     """fast_rnnt/python/fast_rnnt/rnnt_loss.py:25-42 (same assertions; the boundary
     rows are looked at on the host copy shared with the recursion's own check, so a
-    loss call waits for the device at most once)."""
+    loss call waits for the device at most once).  ``on_device``: the caller hands the
+    row tests to the recursion's forward kernel (:func:`_device_checks`), so nothing
+    waits for a host copy of the rows here."""
     if boundary is None:
         assert S >= 1, S
         assert is_rnnt_type_regular or T >= S, \
             f"Modified transducer requires T >= S, but got T={T} and S={S}"
+    elif on_device:
+        return
     else:
         rows = boundary_rows(boundary)
         assert all(r[2] >= 1 for r in rows), boundary[:, 2]
@@ -197,62 +201,21 @@ def _apply_delay_penalty(px: Tensor, boundary: Optional[Tensor], rnnt_type: str,
 _REDUCTIONS = {"none": 0, "mean": 1, "sum": 2}
 
 
-class _RecursionLoss(torch.autograd.Function):
-    """The tail the loss functions share, behind one autograd node: the lattice recursion, --
-    as its autograd wrapper does whenever gradients will be wanted
-    (mutual_information.py:159-168) -- its backward with a gradient of ones, and the
-    reduction of the scores to the loss (rnnt_loss.py:326-340).  backward() scales the
-    occupation gradients in place by the loss's gradient, sign and 1/B of the reduction
-    included, exactly as MutualInformationRecursionFunction.backward does to the tensors
-    it handed out (mutual_information.py:173-181), and passes them on as the gradients of
-    px / py.  Same arithmetic as mutual_information_recursion followed by the torch
-    reduction; one library call each way instead of a dozen small kernels."""
-
-    @staticmethod
-    def forward(ctx, px, py, boundary, want_grads, reduction):
-        B, S, T1 = px.shape
-        T = py.shape[2]
-        sfx = _lib.suffix(px.dtype)
-        bnd_c = boundary.contiguous() if boundary is not None else None
-        opts = dict(dtype=px.dtype, device=px.device)
-        need_grad = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
-        ctx.set_materialize_grads(False)
-        with _on_device(px.device):
-            p = torch.empty(B, S + 1, T + 1, **opts)
-            scores = torch.empty(B, **opts)
-            px_grad = py_grad = None
-            if want_grads or need_grad:
-                px_grad = torch.empty(B, S, T1, **opts)
-                py_grad = torch.empty(B, S + 1, T, **opts)
-            loss = torch.empty((B,) if reduction == 0 else (), **opts)
-            _lib.call("frnnt_mi_loss_fwd_" + sfx, px.data_ptr(), py.data_ptr(), _lib.ptr(bnd_c),
-                      p.data_ptr(), scores.data_ptr(), _lib.ptr(px_grad), _lib.ptr(py_grad),
-                      loss.data_ptr(), B, S, T, int(T1 == T), reduction, _lib.stream_of(px))
-        if need_grad:
-            ctx.save_for_backward(px_grad, py_grad)
-            ctx.meta = (B, S, T, int(T1 == T), sfx, reduction)
-        if px_grad is None:
-            return loss, None, None
-        ctx.mark_non_differentiable(px_grad, py_grad)
-        return loss, px_grad, py_grad
-
-    @staticmethod
-    def backward(ctx, g_loss, _gx, _gy):
-        if g_loss is None:
-            return (None,) * 5
-        px_grad, py_grad = ctx.saved_tensors
-        B, S, T, modified, sfx, reduction = ctx.meta
-        with _on_device(px_grad.device):
-            g = g_loss.contiguous()
-            stride = 1 if reduction == 0 else 0
-            scale = -1.0 / B if reduction == 1 else -1.0
-            _lib.call("frnnt_mi_scale_grads_" + sfx, px_grad.data_ptr(), py_grad.data_ptr(),
-                      g.data_ptr(), stride, scale, B, S, T, modified, _lib.stream_of(px_grad))
-        return px_grad, py_grad, None, None, None
+def _device_checks(rnnt_type: str, boundary: Optional[Tensor]) -> int:
+    """FRNNT_CHECK_* bits for the recursion's forward kernel when the boundary rows are to
+    be tested on the device (the default, see :func:`set_boundary_checks`): the two
+    assertions of validate_st_lengths (rnnt_loss.py:38-42); the window's range
+    (mutual_information.py:277-288) is always tested there.  0 = the rows have been
+    asserted on the host."""
+    if boundary is None or not _lib.ops().deferred_checks():
+        return 0
+    return 1 | (0 if rnnt_type == "regular" else 2)
 
 
 def _recursion_and_reduce(px, py, boundary, rnnt_type, delay_penalty, reduction, return_grad):
-    """Shared tail of the four losses (e.g. rnnt_loss.py:309-340)."""
+    """Shared tail of the four losses (e.g. rnnt_loss.py:309-340): one autograd node of the
+    operator module (recursion, its eager backward with a gradient of ones, the reduction;
+    its backward scales the occupation gradients in place, mutual_information.py:159-181)."""
     if delay_penalty > 0.0:
         _apply_delay_penalty(px, boundary, rnnt_type, delay_penalty)
     if reduction not in _REDUCTIONS:
@@ -265,11 +228,12 @@ def _recursion_and_reduce(px, py, boundary, rnnt_type, delay_penalty, reduction,
     assert px.shape[-1] in [T, T + 1]
     assert py.shape == (B, S + 1, T)
     assert px.dtype == py.dtype
+    checks = _device_checks(rnnt_type, boundary)
     if boundary is not None:
-        _assert_boundary(boundary, B, S, T)
+        _assert_boundary(boundary, B, S, T, on_device=checks != 0)
     _require_gpu(px, py)
-    loss, px_grad, py_grad = _RecursionLoss.apply(px.contiguous(), py.contiguous(), boundary,
-                                                  bool(return_grad), _REDUCTIONS[reduction])
+    loss, px_grad, py_grad = _lib.ops().recursion_loss(
+        px, py, boundary, bool(return_grad), _REDUCTIONS[reduction], checks)
     return (loss, (px_grad, py_grad)) if return_grad else loss
 
 
@@ -288,110 +252,6 @@ def _carve(sizes):
         offsets.append(total)
         total += (n + 3) & ~3
     return offsets, total
-
-
-class _SimpleLoss(torch.autograd.Function):
-    """rnnt_loss_simple's whole device pipeline behind one autograd node:
-    px/py (row maxima + MFMA contraction), the lattice recursion forward, the
-    reduction of the scores to the loss, and -- as the recursion's autograd wrapper
-    does (mutual_information.py:159-168) -- the recursion's backward with a gradient
-    of ones, whose result both is handed out as (px_grad, py_grad) and is what
-    backward() scales in place and pushes through the two gradient GEMMs.  Same
-    arithmetic as get_rnnt_logprobs, mutual_information_recursion and the
-    reduction of rnnt_loss.py:330-340; it only saves host time (one library call,
-    one workspace allocation) and elementwise kernels."""
-
-    @staticmethod
-    def forward(ctx, lm, am, symbols, boundary, termination_symbol, rnnt_type, delay_penalty,
-                want_grads, reduction):
-        B, T, C = am.shape
-        S = lm.shape[1] - 1
-        kind = _RNNT_TYPES[rnnt_type]
-        sfx = _lib.suffix(am.dtype)
-        lm_c, am_c = lm.contiguous(), am.contiguous()
-        sym_c = symbols.contiguous()
-        bnd_c = boundary.contiguous() if boundary is not None else None
-        opts = dict(dtype=am.dtype, device=am.device)
-        T1 = T + 1 if kind == 0 else T
-        need_grad = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
-        # gradients of the non-differentiable outputs are not wanted as zero tensors
-        ctx.set_materialize_grads(False)
-        n_px, n_py = B * S * T1, B * (S + 1) * T
-        # internal buffers live in one allocation: px | py | lm_max | am_max | norm_raw | p | scores
-        (o_px, o_py, o_lmx, o_amx, o_nr, o_p, o_sc), total = _carve(
-            [n_px, n_py, B * (S + 1), B * T, n_py if need_grad else 0, B * (S + 1) * (T + 1), B])
-        with _on_device(am.device):
-            stream = _lib.stream_of(am)
-            work = torch.empty(total, **opts)
-            base, item = work.data_ptr(), work.element_size()
-            at = lambda off: base + off * item  # noqa: E731
-            px_grad = py_grad = None
-            if want_grads or need_grad:
-                px_grad = torch.empty(B, S, T1, **opts)
-                py_grad = torch.empty(B, S + 1, T, **opts)
-            loss = torch.empty((B,) if reduction == 0 else (), **opts)
-            if delay_penalty > 0.0:
-                # the penalty is applied to px between the two stages (rnnt_loss.py:311-326)
-                px = work[o_px:o_px + n_px].view(B, S, T1)
-                _lib.call("frnnt_simple_logprobs_fwd_" + sfx, lm_c.data_ptr(), am_c.data_ptr(),
-                          sym_c.data_ptr(), _lib.ptr(bnd_c), at(o_px), at(o_py), at(o_lmx),
-                          at(o_amx), at(o_nr) if need_grad else None, B, S, T, C,
-                          int(termination_symbol), kind, int(bnd_c is not None), stream)
-                _apply_delay_penalty(px, boundary, rnnt_type, delay_penalty)
-                modified = int(kind != 0)
-                _lib.call("frnnt_mi_forward_" + sfx, at(o_px), at(o_py), _lib.ptr(bnd_c), at(o_p),
-                          at(o_sc), B, S, T, modified, stream)
-                if px_grad is not None:
-                    _lib.call("frnnt_mi_backward_" + sfx, at(o_px), at(o_py), _lib.ptr(bnd_c),
-                              at(o_p), None, px_grad.data_ptr(), py_grad.data_ptr(), B, S, T,
-                              modified, 0, stream)
-                _lib.call("frnnt_loss_reduce_" + sfx, at(o_sc), loss.data_ptr(), B, reduction,
-                          stream)
-            else:
-                _lib.call("frnnt_simple_loss_fwd_" + sfx, lm_c.data_ptr(), am_c.data_ptr(),
-                          sym_c.data_ptr(), _lib.ptr(bnd_c), at(o_px), at(o_py), at(o_lmx),
-                          at(o_amx), at(o_nr) if need_grad else None, at(o_p), at(o_sc),
-                          _lib.ptr(px_grad), _lib.ptr(py_grad), loss.data_ptr(), B, S, T, C,
-                          int(termination_symbol), kind, reduction, stream)
-        if need_grad:
-            ctx.save_for_backward(lm_c, am_c, sym_c, bnd_c, work, px_grad, py_grad)
-            ctx.meta = (B, S, T, C, int(termination_symbol), kind, sfx, reduction,
-                        o_lmx, o_amx, o_nr)
-        if px_grad is None:
-            return loss, None, None
-        ctx.mark_non_differentiable(px_grad, py_grad)
-        return loss, px_grad, py_grad
-
-    @staticmethod
-    def backward(ctx, g_loss, _gx, _gy):
-        if g_loss is None:
-            return (None,) * 9
-        lm, am, sym, bnd, work, px_grad, py_grad = ctx.saved_tensors
-        B, S, T, C, term, kind, sfx, reduction, o_lmx, o_amx, o_nr = ctx.meta
-        opts = dict(dtype=am.dtype, device=am.device)
-        with _on_device(am.device):
-            # d loss / d scores[b] = scale * g_loss[b * stride]
-            g = g_loss.contiguous()
-            stride = 1 if reduction == 0 else 0
-            scale = -1.0 / B if reduction == 1 else -1.0
-            ldd = (T + 3) // 4 * 4
-            # scratch in one allocation: dmat | row_x | row_y | col_y
-            (o_d, o_rx, o_ry, o_cy), total = _carve(
-                [B * (S + 1) * ldd, B * (S + 1), B * (S + 1), B * T])
-            scratch = torch.empty(total, **opts)
-            sbase, wbase, item = scratch.data_ptr(), work.data_ptr(), work.element_size()
-            lm_grad = torch.empty_like(lm) if ctx.needs_input_grad[0] else None
-            am_grad = torch.empty_like(am) if ctx.needs_input_grad[1] else None
-            # px_grad / py_grad are scaled in place by the scores' gradient, exactly as
-            # MutualInformationRecursionFunction.backward does to the tensors it handed out
-            _lib.call("frnnt_simple_logprobs_bwd_" + sfx, lm.data_ptr(), am.data_ptr(),
-                      sym.data_ptr(), _lib.ptr(bnd), wbase + o_lmx * item, wbase + o_amx * item,
-                      wbase + o_nr * item, g.data_ptr(), stride, scale, px_grad.data_ptr(),
-                      py_grad.data_ptr(), sbase + o_d * item, sbase + o_rx * item,
-                      sbase + o_ry * item, sbase + o_cy * item, _lib.ptr(lm_grad),
-                      _lib.ptr(am_grad), B, S, T, C, term, kind, int(bnd is not None),
-                      _lib.stream_of(am))
-        return lm_grad, am_grad, None, None, None, None, None, None, None
 
 
 def rnnt_loss_simple(
@@ -413,20 +273,22 @@ def rnnt_loss_simple(
     (B, T, C) = am.shape
     S = lm.shape[1] - 1
     assert symbols.shape == (B, S), symbols.shape
-    validate_st_lengths(S, T, rnnt_type == "regular", boundary)
     assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
+    checks = _device_checks(rnnt_type, boundary)
+    validate_st_lengths(S, T, rnnt_type == "regular", boundary, on_device=checks != 0)
     _check_tensors([("am", am), ("lm", lm)], [("symbols", symbols), ("boundary", boundary)])
     if boundary is not None:
-        assert boundary.shape == (B, 4)
-        for s_begin, t_begin, s_end, t_end in boundary_rows(boundary):
-            assert 0 <= s_begin <= s_end <= S
-            assert 0 <= t_begin <= t_end <= T
+        _assert_boundary(boundary, B, S, T, on_device=checks != 0)
     if reduction not in ("none", "mean", "sum"):
         raise ValueError(f"reduction should be ('none' | 'mean' | 'sum'), given {reduction}")
     lm, am = _widen(lm, am)
-    loss, px_grad, py_grad = _SimpleLoss.apply(
-        lm, am, symbols, boundary, termination_symbol, rnnt_type, float(delay_penalty),
-        bool(return_grad), _REDUCTIONS[reduction])
+    # the whole device pipeline is one autograd node of the operator module: px / py (row
+    # maxima + MFMA contraction), the recursion, its backward with a gradient of ones, the
+    # reduction; its backward scales the occupation gradients in place and runs the two
+    # gradient products
+    loss, px_grad, py_grad = _lib.ops().simple_loss(
+        lm, am, symbols, boundary, int(termination_symbol), _RNNT_TYPES[rnnt_type],
+        float(delay_penalty), bool(return_grad), _REDUCTIONS[reduction], checks)
     return (loss, (px_grad, py_grad)) if return_grad else loss
 
 
@@ -489,11 +351,13 @@ def _joint_logprobs(logits, symbols, termination_symbol, boundary, rnnt_type, wi
     (B, T, S1, C) = logits.shape
     S = S1 - 1
     assert symbols.shape == (B, S), symbols.shape
-    validate_st_lengths(S, T, rnnt_type == "regular", boundary)
     assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
+    # (window_only: the caller is a loss function, whose recursion tests the rows itself)
+    on_device = bool(window_only) and _device_checks(rnnt_type, boundary) != 0
+    validate_st_lengths(S, T, rnnt_type == "regular", boundary, on_device=on_device)
     _check_tensors([("logits", logits)], [("symbols", symbols), ("boundary", boundary)])
     if window_only and boundary is not None:
-        _assert_boundary(boundary, B, S, T)
+        _assert_boundary(boundary, B, S, T, on_device=on_device)
     return _LatticeLogprobs.apply(logits, symbols, None, boundary, termination_symbol, rnnt_type,
                                   window_only)
 
@@ -722,12 +586,13 @@ def _pruned_logprobs(logits, symbols, ranges, termination_symbol, boundary, rnnt
     (B, T, s_range, C) = logits.shape
     assert ranges.shape == (B, T, s_range), f"{ranges.shape} == ({B}, {T}, {s_range})"
     (B, S) = symbols.shape
-    validate_st_lengths(S, T, rnnt_type == "regular", boundary)
     assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
+    on_device = bool(window_only) and _device_checks(rnnt_type, boundary) != 0
+    validate_st_lengths(S, T, rnnt_type == "regular", boundary, on_device=on_device)
     _check_tensors([("logits", logits)],
                    [("symbols", symbols), ("ranges", ranges), ("boundary", boundary)])
     if window_only and boundary is not None:
-        _assert_boundary(boundary, B, S, T)
+        _assert_boundary(boundary, B, S, T, on_device=on_device)
     return _LatticeLogprobs.apply(logits, symbols, ranges, boundary, termination_symbol,
                                   rnnt_type, window_only)
 
@@ -839,6 +704,13 @@ def get_rnnt_logprobs_smoothed(
     from the fused MFMA kernel; the lm-only / am-only models, the unigram over the
     whole batch and the interpolation come from frnnt_smoothed_logprobs_fwd/bwd.
     """
+    return _smoothed_logprobs(lm, am, symbols, termination_symbol, lm_only_scale,
+                              am_only_scale, boundary, rnnt_type, False)
+
+
+def _smoothed_logprobs(lm, am, symbols, termination_symbol, lm_only_scale, am_only_scale,
+                       boundary, rnnt_type, from_loss):
+    # from_loss: the recursion that follows tests the boundary rows on the device
     assert lm.ndim == 3, lm.ndim
     assert am.ndim == 3, am.ndim
     assert lm.shape[0] == am.shape[0], (lm.shape[0], am.shape[0])
@@ -846,8 +718,9 @@ def get_rnnt_logprobs_smoothed(
     (B, T, C) = am.shape
     S = lm.shape[1] - 1
     assert symbols.shape == (B, S), symbols.shape
-    validate_st_lengths(S, T, rnnt_type == "regular", boundary)
     assert rnnt_type in ["regular", "modified", "constrained"], rnnt_type
+    validate_st_lengths(S, T, rnnt_type == "regular", boundary,
+                        on_device=from_loss and _device_checks(rnnt_type, boundary) != 0)
     _check_tensors([("am", am), ("lm", lm)], [("symbols", symbols), ("boundary", boundary)])
 
     lm, am = _widen(lm, am)
@@ -880,9 +753,7 @@ def rnnt_loss_smoothed(
     delay_penalty: float = 0.0, reduction: Optional[str] = "mean", return_grad: bool = False,
 ) -> Union[Tuple[Tensor, Tuple[Tensor, Tensor]], Tensor]:
     """rnnt_loss_simple with lm-only / am-only smoothing (rnnt_loss.py:1372-1494)."""
-    px, py = get_rnnt_logprobs_smoothed(
-        lm=lm, am=am, symbols=symbols, termination_symbol=termination_symbol,
-        lm_only_scale=lm_only_scale, am_only_scale=am_only_scale, boundary=boundary,
-        rnnt_type=rnnt_type)
+    px, py = _smoothed_logprobs(lm, am, symbols, termination_symbol, lm_only_scale,
+                                am_only_scale, boundary, rnnt_type, True)
     return _recursion_and_reduce(px, py, boundary, rnnt_type, delay_penalty, reduction,
                                  return_grad)

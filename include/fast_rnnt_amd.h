@@ -78,6 +78,29 @@ int frnnt_mi_forward_f32(const float *px, const float *py, const int64_t *bounda
 int frnnt_mi_forward_f64(const double *px, const double *py, const int64_t *boundary,
                          double *p, double *ans, int B, int S, int T, int modified,
                          void *stream);
+/*
+ * frnnt_mi_forward_* that also REPORTS a bad boundary row, for callers that do not want to
+ * wait for a host copy of the rows before every call (the reference's Python layer checks
+ * them through boundary.tolist(), mutual_information.py:277-288, rnnt_loss.py:25-42, which
+ * waits for the device).  Every row is tested on the device anyway; a row that fails is
+ * skipped (ans[b] = NaN) and, when `status` is given, the kernel stores the failed test in
+ * status[0] and the row's index in status[1] (any one of the failing rows).  `status`: two
+ * int32 the host can read once the kernel has run, e.g. pinned host memory
+ * (hipHostMalloc), zeroed by the caller; it is only ever written on a failure.
+ *   checks: FRNNT_CHECK_* bits for the tests of validate_st_lengths on top of the window's
+ *           range (which is always tested).
+ */
+#define FRNNT_CHECK_SYMBOLS 1    /* s_end >= 1                                (rnnt_loss.py:38-39) */
+#define FRNNT_CHECK_FRAMES 2     /* t_end >= s_end, non-regular lattices      (rnnt_loss.py:40-42) */
+#define FRNNT_STATUS_WINDOW 1    /* not 0 <= s_begin <= s_end <= S, 0 <= t_begin <= t_end <= T */
+#define FRNNT_STATUS_NO_SYMBOLS 2
+#define FRNNT_STATUS_FEW_FRAMES 3
+int frnnt_mi_forward_checked_f32(const float *px, const float *py, const int64_t *boundary,
+                                 float *p, float *ans, int B, int S, int T, int modified,
+                                 int checks, int32_t *status, void *stream);
+int frnnt_mi_forward_checked_f64(const double *px, const double *py, const int64_t *boundary,
+                                 double *p, double *ans, int B, int S, int T, int modified,
+                                 int checks, int32_t *status, void *stream);
 
 /*
  * Lattice recursion, backward.  Replaces
@@ -254,34 +277,38 @@ int frnnt_smoothed_logprobs_bwd_f64(const double *lm, const double *am, const in
  * given -- frnnt_mi_backward with a gradient of ones (what the recursion's autograd
  * wrapper computes eagerly, mutual_information.py:159-168), then -- when loss is
  * given -- frnnt_loss_reduce.  Arguments as in those entry points; p [B][S+1][T+1]
- * and scores [B] are outputs as well.  It exists to save host time per call.
+ * and scores [B] are outputs as well; checks / status (may be 0 / NULL) as in
+ * frnnt_mi_forward_checked.  It exists to save host time per call.
  */
 int frnnt_simple_loss_fwd_f32(const float *lm, const float *am, const int64_t *symbols,
                               const int64_t *boundary, float *px, float *py, float *lm_max,
                               float *am_max, float *norm_raw, float *p, float *scores,
                               float *px_grad, float *py_grad, float *loss, int B, int S, int T,
                               int C, int termination_symbol, int rnnt_type, int reduction,
-                              void *stream);
+                              int checks, int32_t *status, void *stream);
 int frnnt_simple_loss_fwd_f64(const double *lm, const double *am, const int64_t *symbols,
                               const int64_t *boundary, double *px, double *py, double *lm_max,
                               double *am_max, double *norm_raw, double *p, double *scores,
                               double *px_grad, double *py_grad, double *loss, int B, int S, int T,
                               int C, int termination_symbol, int rnnt_type, int reduction,
-                              void *stream);
+                              int checks, int32_t *status, void *stream);
 
 /*
  * The tail every loss function shares (rnnt_loss.py:326-340, :535-547, :1119-1132, :1481-1494)
  * in one call: frnnt_mi_forward, then -- when px_grad / py_grad are given -- frnnt_mi_backward
  * with a gradient of ones (mutual_information.py:159-168), then -- when loss is given --
  * frnnt_loss_reduce (the backward kernel reduces the scores on its way: no extra launch).
- * p [B][S+1][T+1] and scores [B] are outputs as well.
+ * p [B][S+1][T+1] and scores [B] are outputs as well; checks / status (may be 0 / NULL) as
+ * in frnnt_mi_forward_checked.
  */
 int frnnt_mi_loss_fwd_f32(const float *px, const float *py, const int64_t *boundary, float *p,
                           float *scores, float *px_grad, float *py_grad, float *loss, int B, int S,
-                          int T, int modified, int reduction, void *stream);
+                          int T, int modified, int reduction, int checks, int32_t *status,
+                          void *stream);
 int frnnt_mi_loss_fwd_f64(const double *px, const double *py, const int64_t *boundary, double *p,
                           double *scores, double *px_grad, double *py_grad, double *loss, int B,
-                          int S, int T, int modified, int reduction, void *stream);
+                          int S, int T, int modified, int reduction, int checks, int32_t *status,
+                          void *stream);
 /*
  * The backward of that tail: px_grad[b] and py_grad[b] are multiplied IN PLACE by
  * score_grad_scale * score_grad[b * score_grad_stride] -- what the recursion's autograd

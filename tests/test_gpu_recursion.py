@@ -193,6 +193,9 @@ def test_invalid_window_is_skipped_not_read(gpu_device):
     gx, gy = _fast_rnnt.mutual_information_backward(px, py, bnd, p, torch.ones(2, device=gpu_device))
     assert math.isnan(ans[1].item()) and math.isfinite(ans[0].item())
     assert (gx[1] == 0).all() and (gy[1] == 0).all()
+    # the operator also reports the row to the host, which raises it when it next looks
+    with pytest.raises(AssertionError, match="boundary row 1"):
+        fast_rnnt_amd.check_boundaries()
 
 
 def test_autograd_front_end(gpu_device):
@@ -215,8 +218,19 @@ def test_autograd_front_end(gpu_device):
     assert torch.allclose(da.grad.cpu(), a.grad, atol=1e-4)
     assert torch.allclose(dc.grad.cpu(), c.grad, atol=1e-4)
     assert torch.allclose(gx.cpu(), wx, atol=1e-4)  # scaled in place by backward, like the reference
+    # a boundary row out of range: the kernel skips the row (nan) and the reference's
+    # AssertionError (mutual_information.py:277-288) is raised once the host looks
+    bad = torch.tensor([[0, 0, 7, 11]] * 3, device=gpu_device)
+    scores = fast_rnnt_amd.mutual_information_recursion(da, dc, bad)
     with pytest.raises(AssertionError):
-        fast_rnnt_amd.mutual_information_recursion(da, dc, torch.tensor([[0, 0, 7, 11]] * 3, device=gpu_device))
+        fast_rnnt_amd.check_boundaries()
+    assert torch.isnan(scores).all()
+    fast_rnnt_amd.set_boundary_checks("host")
+    try:
+        with pytest.raises(AssertionError):
+            fast_rnnt_amd.mutual_information_recursion(da, dc, bad)
+    finally:
+        fast_rnnt_amd.set_boundary_checks("device")
 
 
 def test_joint_recursion_splits_the_total(gpu_device):
