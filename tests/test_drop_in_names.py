@@ -54,3 +54,17 @@ def test_operator_module_signatures():
         _fast_rnnt.mutual_information_forward(px, py, None, p)
     with pytest.raises(RuntimeError, match="3-dimensional"):
         _fast_rnnt.mutual_information_forward(px[0], py, None, p)
+
+
+def test_k2_names():
+    # README.md:4 -- k2 ships the same functions; recipes written against `k2.*` can import
+    # this module under that name (never a top-level `k2`)
+    import importlib.util
+
+    import fast_rnnt_amd.k2_compat as k2
+    for name in REFERENCE_EXPORTS:
+        if name != "with_cuda":
+            assert getattr(k2, name) is getattr(fast_rnnt_amd, name), name
+    assert sorted(k2.__all__) == sorted(n for n in REFERENCE_EXPORTS if n != "with_cuda")
+    spec = importlib.util.find_spec("k2")
+    assert spec is None or "fast_rnnt" not in (spec.origin or "")
