@@ -69,6 +69,17 @@ __device__ __forceinline__ int64_t row_symbol(const int64_t *symbols, const int6
   return s == S ? (int64_t)term : symbols[(long)b * S + s];
 }
 
+// Lattice row that logits row `row` = (frame, j) is placed at: j without ranges, else
+// (ranges[frame][0] + j) mod (S + 1) -- the roll of rnnt_loss.py:968-984, the rule the assembly
+// and the gradient kernels follow, whatever the frame's other range entries hold (the
+// reference accepts ranges that are not consecutive and rolls by the first entry alone).
+__device__ __forceinline__ int64_t placed_row(const int64_t *ranges, long row, int Rr, int S) {
+  const int j = (int)(row % Rr);
+  if (!ranges) return j;
+  int64_t s = ((int64_t)j + ranges[row - j]) % (S + 1);
+  return s < 0 ? s + S + 1 : s;
+}
+
 // True when the logits row (b, t) x lattice row s lies outside utterance b's boundary
 // window [s_begin, s_end] x [t_begin, t_end): the recursion never looks at its px / py
 // and hands it a gradient of exact zeros.  Callers that go on to the recursion with the
@@ -92,7 +103,7 @@ __global__ void __launch_bounds__(256)
   if (row >= rows) return;
   if (window &&
       outside_window(window, (int)(row / ((long)Rr * T)), (int)((row / Rr) % T),
-                     ranges ? ranges[row] : row % Rr))
+                     placed_row(ranges, row, Rr, S)))
     return;
   const R *x = logits + row * C;
   R m = Num<R>::neg_inf();
@@ -148,7 +159,7 @@ __device__ __forceinline__ floatx4u as_floats(intx4 raw) {
 // which rows of the wave's group need work (bit r), wave-uniform
 template <int kRows>
 __device__ __forceinline__ unsigned live_rows(long first, long rows, const int64_t *ranges,
-                                              const int64_t *window, int T, int Rr) {
+                                              const int64_t *window, int T, int Rr, int S) {
   unsigned live = 0;
 #pragma unroll
   for (int r = 0; r < kRows; ++r) {
@@ -157,7 +168,7 @@ __device__ __forceinline__ unsigned live_rows(long first, long rows, const int64
     bool needed = true;
     if (window)
       needed = !outside_window(window, (int)(row / ((long)Rr * T)), (int)((row / Rr) % T),
-                               ranges ? ranges[row] : row % Rr);
+                               placed_row(ranges, row, Rr, S));
     live |= needed ? 1u << r : 0u;
   }
   return live;
@@ -173,7 +184,7 @@ __global__ void __launch_bounds__(256)
   const long first = ((long)blockIdx.x * 4 + wave) * kRows;
   const int lane = threadIdx.x & 63;
   if (first >= rows) return;
-  const unsigned live = live_rows<kRows>(first, rows, ranges, window, T, Rr);
+  const unsigned live = live_rows<kRows>(first, rows, ranges, window, T, Rr, S);
   if (live == 0) return;
   const long here = rows - first < kRows ? rows - first : kRows;
   const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
@@ -321,7 +332,7 @@ __global__ void __launch_bounds__(256)
   if (row >= rows) return;
   if (window &&
       outside_window(window, (int)(row / ((long)Rr * T)), (int)((row / Rr) % T),
-                     ranges ? ranges[row] : row % Rr)) {
+                     placed_row(ranges, row, Rr, S))) {
     for (int c = lane; c < C; c += kWave) glogits[row * C + c] = 0;
     return;
   }
@@ -375,7 +386,7 @@ __global__ void __launch_bounds__(256)
   const long first = ((long)blockIdx.x * 4 + wave) * kRows;
   const int lane = threadIdx.x & 63;
   if (first >= rows) return;
-  const unsigned live = live_rows<kRows>(first, rows, ranges, window, T, Rr);
+  const unsigned live = live_rows<kRows>(first, rows, ranges, window, T, Rr, S);
   const long here = rows - first < kRows ? rows - first : kRows;
   const __amdgpu_buffer_rsrc_t in_rs = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<float *>(logits + first * C), 0, (int)(here * C * 4), 0x00020000);
@@ -517,7 +528,7 @@ __global__ void __launch_bounds__(256)
   const long row = (long)blockIdx.x * 4 + wave;
   const int lane = threadIdx.x & 63;
   if (row >= rows) return;
-  if (live_rows<1>(row, rows, ranges, window, T, Rr) == 0) return;
+  if (live_rows<1>(row, rows, ranges, window, T, Rr, S) == 0) return;
   const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint16_t *>(logits + row * C), 0, C * 2, 0x00020000);
   constexpr int kAux = kStream ? 2 : 0;
@@ -576,7 +587,7 @@ __global__ void __launch_bounds__(256)
   const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (row >= rows) return;
-  if (live_rows<1>(row, rows, ranges, window, T, Rr) == 0) return;
+  if (live_rows<1>(row, rows, ranges, window, T, Rr, S) == 0) return;
   const uint16_t *x = logits + row * C;
   float m = -__builtin_huge_valf();
   for (int c = lane; c < C; c += kWave) {
@@ -646,7 +657,7 @@ __global__ void __launch_bounds__(256)
   const long row = (long)blockIdx.x * 4 + wave;
   const int lane = threadIdx.x & 63;
   if (row >= rows) return;
-  const bool live = live_rows<1>(row, rows, ranges, window, T, Rr) != 0;  // wave-uniform
+  const bool live = live_rows<1>(row, rows, ranges, window, T, Rr, S) != 0;  // wave-uniform
   const __amdgpu_buffer_rsrc_t in_rs = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint16_t *>(logits + row * C), 0, C * 2, 0x00020000);
   const __amdgpu_buffer_rsrc_t out_rs =
@@ -701,7 +712,7 @@ __global__ void __launch_bounds__(256)
   const int lane = threadIdx.x & 63;
   if (row >= rows) return;
   uint16_t *g = glogits + row * C;
-  if (live_rows<1>(row, rows, ranges, window, T, Rr) == 0) {
+  if (live_rows<1>(row, rows, ranges, window, T, Rr, S) == 0) {
     for (int c = lane; c < C; c += kWave) g[c] = 0;
     return;
   }

@@ -669,7 +669,15 @@ __global__ void __launch_bounds__((1 + kStagers) * kSweepCap *kWave)
       done = has_down ? sweep_tiles(std::false_type{}, std::true_type{})
                       : sweep_tiles(std::false_type{}, std::false_type{});
     if (!done) return;
-    if (lane == fin_lane) ans[b] = peek(&cnt.failed) ? std::numeric_limits<R>::quiet_NaN() : fin;
+    if (lane == fin_lane) {
+      ans[b] = peek(&cnt.failed) ? std::numeric_limits<R>::quiet_NaN() : fin;
+      // A staging wave may give up between that look and the store, and its NaN must not be
+      // covered by the score: once the store has left, look again.  A wave that gives up
+      // after this second look stores its NaN after it, and so after the score.
+      __threadfence();
+      if (__hip_atomic_load(&cnt.failed, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP))
+        ans[b] = std::numeric_limits<R>::quiet_NaN();
+    }
     tile_base += g.ntiles;
   }
 }

@@ -1687,6 +1687,20 @@ int frnnt_simple_logprobs_bwd_noalloc_f32(const float *lm, const float *am, cons
                 "library's own buffer holds %zu; use frnnt_simple_logprobs_bwd_f32 with a "
                 "caller-provided workspace",
                 B, S, T, need * sizeof(float), frnnt::kOwnScratchFloats * sizeof(float));
+  // the array is the current device's copy: the buffers must live on that device
+  if (px_grad) {
+    hipPointerAttribute_t where;
+    int current = -1;
+    if (hipPointerGetAttributes(&where, px_grad) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(FRNNT_EINVAL, "simple_logprobs_bwd_noalloc: px_grad is not a device pointer");
+    }
+    if (hipGetDevice(&current) != hipSuccess || where.device != current)
+      return fail(FRNNT_EINVAL,
+                  "simple_logprobs_bwd_noalloc: the buffers live on device %d but device %d is "
+                  "current; make the buffers' device current before the call",
+                  where.device, current);
+  }
   float *base = frnnt::own_scratch_address();
   if (!base) return fail(FRNNT_ELAUNCH, "simple_logprobs_bwd_noalloc: hipGetSymbolAddress failed");
   float *dmat = base, *row_x = dmat + n_dmat, *row_y = row_x + n_rows, *col_y = row_y + n_rows;

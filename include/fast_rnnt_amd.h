@@ -210,7 +210,9 @@ int frnnt_simple_logprobs_bwd_f64(const double *lm, const double *am, const int6
  * bytes (each part rounded up to 16) exceed 16 MiB.  All calls on one GPU share that
  * array: calls that overlap there (two streams, two threads) race, so issue them one
  * after the other on one stream.  The first call on a device looks the array's address
- * up (hipGetSymbolAddress); make that call outside a stream capture.
+ * up (hipGetSymbolAddress); make that call outside a stream capture.  The device that
+ * holds the buffers must be the calling thread's current device (as for every entry
+ * point; here it also selects the array): FRNNT_EINVAL when px_grad lives elsewhere.
  */
 int frnnt_simple_logprobs_bwd_noalloc_f32(const float *lm, const float *am, const int64_t *symbols,
                                           const int64_t *boundary, const float *lm_max,

@@ -398,6 +398,50 @@ def test_small_s_range_never_gives_inf(gpu_device):
         assert torch.isfinite(loss).all(), (S, loss)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_ranges_that_are_not_consecutive(gpu_device, dtype):
+    # The reference takes any `ranges`: row j of frame t scores the symbol of lattice row
+    # ranges[b,t,j] and is rolled to lattice row ranges[b,t,0] + j (rnnt_loss.py:955-984).  The
+    # loss (which skips logits rows outside the boundary window) must place and skip by that
+    # same rule: equal to the (px, py) builder followed by the recursion, and to the oracle.
+    dev = gpu_device
+    B, S, T, C, R = 3, 12, 20, 15, 4
+    g = torch.Generator().manual_seed(811)
+    logits = torch.randn(B, T, R, C, generator=g, dtype=dtype)
+    sym = torch.randint(1, C, (B, S), generator=g)
+    bnd = torch.tensor([[0, 0, S, T], [0, 0, 7, 13], [2, 3, 10, 18]])
+    # first entries that follow each window's diagonal (so that every lattice has paths) ...
+    t = torch.arange(T).reshape(1, T)
+    s0, t0, s1, t1 = (bnd[:, k].reshape(B, 1) for k in range(4))
+    along = s0 + ((t - t0).clamp(min=0) * (s1 - s0)) // (t1 - t0) - 1
+    first = along.clamp(min=0, max=S + 1 - R).reshape(B, T, 1)
+    ranges = first + torch.arange(R).reshape(1, 1, R)
+    # ... and later entries shuffled or repeated, within [0, S]
+    ranges[:, ::2, 1:] = ranges[:, ::2, 1:].flip(-1)
+    ranges[:, 1::3, 2] = ranges[:, 1::3, 1]
+    ranges[0, ::5, 3] = S
+    a = logits.clone().requires_grad_(True)
+    want = O.loss_pruned(a, sym, ranges, 0, boundary=bnd, reduction="none")
+    finite = torch.isfinite(want)
+    assert finite.all()
+    want[finite].sum().backward()
+
+    d1 = logits.to(dev).requires_grad_(True)
+    loss = fast_rnnt_amd.rnnt_loss_pruned(d1, sym.to(dev), ranges.to(dev), 0, boundary=bnd.to(dev),
+                                          reduction="none")
+    loss[finite.to(dev)].sum().backward()
+    d2 = logits.to(dev).requires_grad_(True)
+    px, py = fast_rnnt_amd.get_rnnt_logprobs_pruned(d2, sym.to(dev), ranges.to(dev), 0,
+                                                    boundary=bnd.to(dev))
+    scores = fast_rnnt_amd.mutual_information_recursion(px, py, bnd.to(dev))
+    (-scores)[finite.to(dev)].sum().backward()
+    tol = 1e-4 if dtype == torch.float32 else 1e-9
+    assert _close(loss, -scores, 0.0, 1e-6 if dtype == torch.float32 else 1e-12)
+    assert _close(loss, want, 0.0, 1e-5 if dtype == torch.float32 else 1e-10)
+    assert _close(d1.grad, d2.grad, tol * 0.1, tol * 0.1)
+    assert _close(d1.grad, a.grad, tol, tol)
+
+
 @pytest.mark.parametrize("kind", KINDS)
 def test_pruned_with_every_row_kept_equals_unpruned(gpu_device, kind):
     # ranges that keep all S + 1 rows of every frame: rnnt_loss_pruned must give what

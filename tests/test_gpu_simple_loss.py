@@ -239,6 +239,82 @@ def test_fused_loss_ignores_frames_past_the_window(gpu_device, kind):
         assert _close(dl.grad, l.grad, 1e-4, 1e-4)
 
 
+def _poison_the_allocator(dev, nbytes):
+    """Leaves NaN in the blocks that torch's caching allocator will hand out next: every
+    buffer the loss functions take with torch.empty / at::empty (px, py, the normalizers,
+    the row maxima, p, scratch) then starts as NaN wherever the kernels do not write."""
+    sizes = [nbytes, nbytes // 2, nbytes // 4, nbytes // 8, 1 << 20, 1 << 16, 1 << 12, 512]
+    blocks = [torch.full((max(n // 4, 1),), float("nan"), device=dev) for n in sizes for _ in (0, 1)]
+    torch.cuda.synchronize()
+    del blocks
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_nothing_undefined_is_read_outside_the_windows(gpu_device, dtype, kind):
+    # With a boundary the float32 kernels leave px, py, the normalizers and the frames' maxima
+    # undefined outside each utterance's window (the float64 ones compute everything): every
+    # later reader must keep to the window.  Windows that start past (0, 0), internal buffers
+    # that start as NaN, lm / am rows outside the windows that hold NaN and infinities: the
+    # losses stay finite and equal to the oracle's on clean input, the gradients are exact
+    # zeros outside the windows.
+    dev = gpu_device
+    B, S, T, C = 4, 37, 90, 41
+    am, lm, sym, _ = _case(500 + KINDS.index(kind), B, S, T, C, dtype, kind, with_boundary=False)
+    bnd = torch.tensor([[0, 0, S, T], [3, 7, 30, 80], [5, 0, 20, 41], [0, 11, 37, 75]])
+    if kind != "regular":
+        bnd[2, 3] = 60  # T_b - t_begin >= S_b - s_begin paths exist; T_b >= S_b is asserted
+    t_idx = torch.arange(T).reshape(1, T, 1)
+    s_idx = torch.arange(S + 1).reshape(1, S + 1, 1)
+    past_t = (t_idx >= bnd[:, 3].reshape(B, 1, 1)).expand(B, T, C)
+    past_s = (s_idx > bnd[:, 2].reshape(B, 1, 1)).expand(B, S + 1, C)
+    a = am.clone().requires_grad_(True)
+    l = lm.clone().requires_grad_(True)
+    want, (wx, wy) = O.loss_simple(l, a, sym, 0, boundary=bnd, rnnt_type=kind, reduction="none",
+                                   return_grad=True)
+    wx0, wy0 = wx.clone(), wy.clone()
+    want.sum().backward()
+    assert torch.isfinite(want).all()
+
+    bad_am = am.clone()
+    bad_am[past_t] = float("nan")
+    bad_lm = lm.clone()
+    bad_lm[past_s] = float("inf")
+    if dtype == torch.float64:
+        # (the float64 kernels take the whole lattice: they get clean input and only the
+        # poisoned buffers)
+        bad_am, bad_lm = am, lm
+    _poison_the_allocator(dev, 4 * B * (S + 1) * (T + 1) * 8)
+    da = bad_am.to(dev).requires_grad_(True)
+    dl = bad_lm.to(dev).requires_grad_(True)
+    _poison_the_allocator(dev, 4 * B * (S + 1) * (T + 1) * 8)
+    got, (gx, gy) = fast_rnnt_amd.rnnt_loss_simple(dl, da, sym.to(dev), 0, boundary=bnd.to(dev),
+                                                   rnnt_type=kind, reduction="none",
+                                                   return_grad=True)
+    gx0, gy0 = gx.clone(), gy.clone()
+    _poison_the_allocator(dev, 4 * B * (S + 1) * (T + 1) * 8)
+    got.sum().backward()
+    tol = 1e-4 if dtype == torch.float32 else 1e-9
+    assert torch.isfinite(got).all() and _close(got, want, 0.0, 1e-5 if dtype == torch.float32 else 1e-10)
+    assert _close(gx0, wx0, tol) and _close(gy0, wy0, tol)
+    # the occupation gradients outside the windows: exact zeros, as the recursion writes them
+    inside_x = torch.zeros_like(wx0, dtype=torch.bool)
+    inside_y = torch.zeros_like(wy0, dtype=torch.bool)
+    for b, (s0, t0, s1, t1) in enumerate(bnd.tolist()):
+        inside_x[b, s0:s1, t0:t1 + 1] = True
+        inside_y[b, s0:s1 + 1, t0:t1] = True
+    assert bool((gx0.cpu()[~inside_x[:, :, :gx0.shape[2]]] == 0).all())
+    assert bool((gy0.cpu()[~inside_y] == 0).all())
+    ga, gl = da.grad.cpu(), dl.grad.cpu()
+    if dtype == torch.float32:
+        assert bool((ga[past_t] == 0).all())
+        assert _close(ga[~past_t], a.grad[~past_t], tol, tol)
+        assert _close(gl[~past_s], l.grad[~past_s], tol, tol)
+    else:
+        assert _close(ga, a.grad, tol, tol) and _close(gl, l.grad, tol, tol)
+    assert torch.isfinite(ga).all()
+
+
 def test_delay_penalty_and_only_one_input_needs_grad(gpu_device):
     dev = gpu_device
     am, lm, sym, bnd = _case(77, 3, 9, 30, 21, torch.float32, "regular")
