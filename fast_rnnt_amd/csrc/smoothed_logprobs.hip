@@ -236,6 +236,92 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// The same interpolation, a workgroup per (utterance, 8 frames).  The elementwise form above
+// reads am[b, t, sym[b, s]] with t along the lanes: a different 4 C-byte row -- a whole cache
+// line -- for every cell (B = 32, S = 80, T = 250, C = 500: 77 MB fetched for 5 MB written).
+// Here the tile's am values are gathered once with s along the lanes (the lanes of a frame
+// share its row's lines) into LDS, the per-row terms of lm and the per-frame normalizers are
+// staged beside them, and px / py leave with t along the lanes.  Same operations in the same
+// order as the elementwise form: bit-identical results.
+constexpr int kCombineFrames = 8;
+template <typename R>
+size_t combine_tile_lds_bytes(int S) {
+  const int S1 = S + 1, pitch = S1 | 1;
+  return ((size_t)kCombineFrames * pitch + 3 * (size_t)S1 + kCombineFrames) * sizeof(R);
+}
+template <typename R>
+__global__ void __launch_bounds__(256)
+    smoothed_combine_tile_kernel(const R *__restrict__ lm, const R *__restrict__ am,
+                                 const int64_t *__restrict__ symbols,
+                                 const int64_t *__restrict__ boundary, const R *__restrict__ pxj,
+                                 const R *__restrict__ pyj, const R *__restrict__ lm_max,
+                                 const R *__restrict__ lm_sum, const R *__restrict__ am_max,
+                                 const R *__restrict__ am_z, const R *__restrict__ unigram,
+                                 R *__restrict__ px, R *__restrict__ py, int S, int T, int C,
+                                 int term, int regular, R k_joint, R k_lm, R k_am) {
+  extern __shared__ __align__(16) unsigned char combine_lds[];
+  const int S1 = S + 1, T1 = regular ? T + 1 : T, pitch = S1 | 1;
+  R *am_s = reinterpret_cast<R *>(combine_lds);  // [32][pitch]: am[t][sym[s]], column S: am[t][term]
+  R *lm_x = am_s + kCombineFrames * pitch;        // [S1] lm[s][sym[s]] - log-normalizer of row s
+  R *lm_y = lm_x + S1;                            // [S1] lm[s][term] - log-normalizer of row s
+  R *lu_s = lm_y + S1;                            // [S1] log(unigram[sym[s]]), entry S: log(unigram[term])
+  R *an_s = lu_s + S1;                            // [32] log-normalizer of the am-only model per frame
+  const int b = blockIdx.y, t0 = blockIdx.x * kCombineFrames;
+  const int tid = threadIdx.x;
+  const R nan = std::numeric_limits<R>::quiet_NaN();
+  const R ninf = Num<R>::neg_inf();
+  for (int s = tid; s < S1; s += 256) {
+    const long lrow = (long)b * S1 + s;
+    const R ln = log(lm_sum[lrow]) + lm_max[lrow];
+    lm_y[s] = lm[lrow * C + term] - ln;
+    if (s < S) {
+      const int64_t sym = symbols[(long)b * S + s];
+      const bool in = sym >= 0 && sym < C;
+      lm_x[s] = (in ? lm[lrow * C + sym] : nan) - ln;
+      lu_s[s] = in ? log(unigram[sym]) : nan;
+    } else {
+      lu_s[s] = log(unigram[term]);
+    }
+  }
+  if (tid < kCombineFrames) {
+    const int t = t0 + tid;
+    if (t < T) {
+      const long arow = (long)b * T + t;
+      an_s[tid] = log(am_z[arow]) + am_max[arow];
+    }
+  }
+  for (int i = tid; i < kCombineFrames * S1; i += 256) {
+    const int tl = i / S1, s = i - tl * S1, t = t0 + tl;
+    if (t >= T) continue;
+    int64_t col = term;
+    if (s < S) col = symbols[(long)b * S + s];
+    am_s[tl * pitch + s] = (col >= 0 && col < C) ? am[((long)b * T + t) * C + col] : nan;
+  }
+  __syncthreads();
+  const int t_mask = (boundary && regular) ? (int)boundary[4 * b + 3] : -1;
+  const R *pxjb = pxj + (long)b * S * T1;
+  R *pxb = px + (long)b * S * T1;
+  for (int i = tid; i < kCombineFrames * S; i += 256) {
+    const int s = i / kCombineFrames, tl = i % kCombineFrames, t = t0 + tl;
+    if (t >= T1) continue;
+    R am_only = ninf;
+    if (t < T) am_only = (am_s[tl * pitch + s] + lu_s[s]) - an_s[tl];
+    R v = pxjb[(long)s * T1 + t] * k_joint + lm_x[s] * k_lm + am_only * k_am;
+    // nothing can be emitted after an utterance's last frame (fix_for_boundary,
+    // rnnt_loss.py:45-63, applied by the reference after the interpolation)
+    if (t == t_mask) v = ninf;
+    pxb[(long)s * T1 + t] = v;
+  }
+  const R *pyjb = pyj + (long)b * S1 * T;
+  R *pyb = py + (long)b * S1 * T;
+  for (int i = tid; i < kCombineFrames * S1; i += 256) {
+    const int s = i / kCombineFrames, tl = i % kCombineFrames, t = t0 + tl;
+    if (t >= T) continue;
+    const R am_only = (am_s[tl * pitch + S] + lu_s[S]) - an_s[tl];
+    pyb[(long)s * T + t] = pyjb[(long)s * T + t] * k_joint + lm_y[s] * k_lm + am_only * k_am;
+  }
+}
+
 // ---- backward -----------------------------------------------------------------------
 
 // Row sums rx, ry (one wave per lattice row; rx over all T1 columns) and column sums
@@ -549,7 +635,17 @@ int fwd_impl(const R *lm, const R *am, const int64_t *symbols, const int64_t *bo
   const long total = (long)B * S * T1 + (long)B * (S + 1) * T;
   const R k_lm = (R)lm_only_scale, k_am = (R)am_only_scale;
   const R k_joint = (R)(1.0 - lm_only_scale - am_only_scale);
-  if (total > 0)
+  // (the tile form needs 8 x (S + 1) values in LDS; lattices too tall for that keep the
+  // elementwise form)
+  const size_t tile_lds = combine_tile_lds_bytes<R>(S);
+  if (total > 0 && tile_lds <= (size_t)96 * 1024 &&
+      allow_lds(reinterpret_cast<const void *>(smoothed_combine_tile_kernel<R>), tile_lds))
+    hipLaunchKernelGGL(smoothed_combine_tile_kernel<R>,
+                       dim3((unsigned)((T1 + kCombineFrames - 1) / kCombineFrames), (unsigned)B),
+                       dim3(256), tile_lds, stream, lm, am, symbols, boundary, pxj, pyj, lm_max,
+                       lm_sum, am_max, am_z, unigram, px, py, S, T, C, term, regular, k_joint, k_lm,
+                       k_am);
+  else if (total > 0)
     hipLaunchKernelGGL(smoothed_combine_kernel<R>, dim3((unsigned)((total + 255) / 256)),
                        dim3(256), 0, stream, lm, am, symbols, boundary, pxj, pyj, lm_max, lm_sum, am_max,
                        am_z, unigram, px, py, B, S, T, C, term, regular, k_joint, k_lm, k_am);
