@@ -535,7 +535,10 @@ constexpr int kPanThreads = kPanWaves * kWave;
 template <int kS, int kK>
 struct PanelShape {
   static constexpr int kRows = kS + kPanT;        // rows of a slab: lm rows, then am rows
-  static constexpr int kPitch = kK + 1;
+  // Row pitch in LDS: kK + 4.  Rows start 16-byte aligned, so a lane's four values of a row
+  // go in as one 16-byte write, and a lane reads its row's eight k of a slab half as two
+  // 16-byte reads: eight lanes' reads (rows r .. r + 7, 20 floats apart) fall on all 32 banks.
+  static constexpr int kPitch = kK + 4;
   static constexpr int kSlab = kRows * kPitch;    // floats per slab
   static constexpr int kRowLanes = kK / 4;        // lanes that share a row of a slab
   static constexpr int kRowsPerLoad = kWave / kRowLanes;
@@ -561,7 +564,7 @@ __global__ void __launch_bounds__(kPanThreads)
   constexpr int kPanSlab = Shape::kSlab, kPanItems = Shape::kItems;
   constexpr int kRowLanes = Shape::kRowLanes, kRowsPerLoad = Shape::kRowsPerLoad;
   using namespace dgemm;
-  extern __shared__ float pan_lds[];
+  extern __shared__ __align__(16) float pan_lds[];
   __shared__ float wave_max[kPanWaves][kPanRows];    // row maxima over each wave's share of k
   __shared__ float wave_shift[kPanWaves][kPanRows];  // the waves' final shifts, as -shift log2(e)
   __shared__ float factor[kPanWaves][kPanRows];      // scale factors for a wave's partial sums
@@ -742,22 +745,32 @@ __global__ void __launch_bounds__(kPanThreads)
     if (__any(above)) raise_shifts(first);
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
-      float *d = mine + (sub + kRowsPerLoad * j) * kPanPitch + kq;
+      floatx4 e;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) d[i] = exp_shifted(slab[j][i], shift2[j]);
+      for (int i = 0; i < 4; ++i) e[i] = exp_shifted(slab[j][i], shift2[j]);
+      *reinterpret_cast<floatx4 *>(mine + (sub + kRowsPerLoad * j) * kPanPitch + kq) = e;
     }
     if (next_chunk < chunks) fetch(slab, next_chunk * kPanK);
-    const float *ap = mine + r32 * kPanPitch + half;
-    const float *bp = mine + (kPanS + r32) * kPanPitch + half;
+    // MFMA i of the slab multiplies k = i (lanes 0..31) and k = i + kK / 2 (lanes 32..63): the
+    // order in which a slab's k are summed is free, and this one lets a lane take its row's
+    // share of the slab with 16-byte reads
+    static_assert(kPanK == 16, "two 16-byte reads per row and slab half");
+    const float *ap = mine + r32 * kPanPitch + 8 * half;
+    const float *bp = mine + (kPanS + r32) * kPanPitch + 8 * half;
+    const floatx4 b0 = *reinterpret_cast<const floatx4 *>(bp);
+    const floatx4 b1 = *reinterpret_cast<const floatx4 *>(bp + 4);
 #pragma unroll
-    for (int i = 0; i < kPanK / 2; ++i) {
-      const float bv = bp[2 * i];
+    for (int j = 0; j < kPanS / 32; ++j)
+      if (j < live_tiles) {
+        const floatx4 a0 = *reinterpret_cast<const floatx4 *>(ap + j * 32 * kPanPitch);
+        const floatx4 a1 = *reinterpret_cast<const floatx4 *>(ap + j * 32 * kPanPitch + 4);
 #pragma unroll
-      for (int j = 0; j < kPanS / 32; ++j)
-        if (j < live_tiles)
-          acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[j * 32 * kPanPitch + 2 * i], bv, acc[j],
-                                                        0, 0, 0);
-    }
+        for (int i = 0; i < 4; ++i)
+          acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i], b0[i], acc[j], 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b1[i], acc[j], 0, 0, 0);
+      }
   };
   for (int chunk = wave; chunk < chunks; chunk += kPanWaves)
     consume(slab, chunk + kPanWaves, chunk == wave);
@@ -876,7 +889,8 @@ constexpr int kLmThreads = kLmWaves * kWave;
 constexpr int kLmOutPitch = kLmC + 1;  // pitch of a wave's partial sums in LDS
 template <int kS, int kK>
 struct LmShape {
-  static constexpr int kPitch = kK + 1;
+  // (row pitch of the D slab: 16-byte aligned rows, as in PanelShape)
+  static constexpr int kPitch = kK + 4;
   static constexpr int kSlab = kS * kPitch + kK * kLmC;  // floats per wave: D slab, then am slab
   static constexpr int kSums = kS * kLmOutPitch;         // floats of a wave's partial sums
   static constexpr size_t kLdsBytes =
@@ -899,7 +913,7 @@ __device__ __forceinline__ void simple_bwd_lm_slab_body(
   constexpr int kLmS = kS, kLmK = kK, kLmPitch = Shape::kPitch, kLmSlab = Shape::kSlab;
   constexpr int kLmItems = Shape::kItems;
   using namespace dgemm;
-  extern __shared__ float lm_lds[];
+  extern __shared__ __align__(16) float lm_lds[];
   const int S1 = S + 1;
   const int c_tiles = (C + kLmC - 1) / kLmC, s_tiles = (S1 + kLmS - 1) / kLmS;
   int b, tile;
@@ -1003,11 +1017,8 @@ __device__ __forceinline__ void simple_bwd_lm_slab_body(
     for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
   for (; chunk < chunks; chunk += kLmWaves) {
 #pragma unroll
-    for (int j = 0; j < kLoadsA; ++j) {
-      float *d = as + (sub_a + kRowsA * j) * kLmPitch + kq_a;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) d[i] = sa[j][i];
-    }
+    for (int j = 0; j < kLoadsA; ++j)
+      *reinterpret_cast<floatx4 *>(as + (sub_a + kRowsA * j) * kLmPitch + kq_a) = sa[j];
 #pragma unroll
     for (int j = 0; j < kLoadsB; ++j) {
       floatx4 e;
@@ -1016,17 +1027,26 @@ __device__ __forceinline__ void simple_bwd_lm_slab_body(
       *reinterpret_cast<floatx4 *>(bs + (sub + 8 * j) * kLmC + kq) = e;
     }
     if (chunk + kLmWaves < chunks) fetch((chunk + kLmWaves) * kLmK);
-    const float *ap = as + r32 * kLmPitch + half;
-    const float *bp = bs + half * kLmC + r32;
+    // MFMA i of the slab multiplies frames i (lanes 0..31) and i + kK / 2 (lanes 32..63) -- the
+    // order in which a slab's frames are summed is free -- so that a lane takes its D row's
+    // share of the slab with 16-byte reads
+    constexpr int kHalfK = kLmK / 2;
+    const float *ap = as + r32 * kLmPitch + kHalfK * half;
+    const float *bp = bs + kHalfK * half * kLmC + r32;
+    float bv[kHalfK];
 #pragma unroll
-    for (int i = 0; i < kLmK / 2; ++i) {
-      const float bv = bp[2 * i * kLmC];
+    for (int i = 0; i < kHalfK; ++i) bv[i] = bp[i * kLmC];
 #pragma unroll
-      for (int j = 0; j < kLmS / 32; ++j)
-        if (j < live_tiles)
-          acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[j * 32 * kLmPitch + 2 * i], bv, acc[j],
-                                                        0, 0, 0);
-    }
+    for (int j = 0; j < kLmS / 32; ++j)
+      if (j < live_tiles) {
+#pragma unroll
+        for (int i4 = 0; i4 < kHalfK / 4; ++i4) {
+          const floatx4 a = *reinterpret_cast<const floatx4 *>(ap + j * 32 * kLmPitch + 4 * i4);
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], bv[4 * i4 + i], acc[j], 0, 0, 0);
+        }
+      }
   }
 
   // the partial sums meet: [wave][kS][33] in the slab space
@@ -1115,7 +1135,7 @@ __device__ __forceinline__ void simple_bwd_am_panel_body(
     float *__restrict__ am_grad, const int64_t *__restrict__ window, int B, int S, int T, int C,
     int ldd, int term, int rnnt_type, int rows_cap, int part_shift) {
   using namespace dgemm;
-  extern __shared__ float am_lds[];
+  extern __shared__ __align__(16) float am_lds[];
   int *sym_s = reinterpret_cast<int *>(am_lds);   // [rows_cap] symbols of the pass (-1: none)
   float *lmx_s = am_lds + rows_cap;               // [rows_cap] lm_max of the pass
   float *shift_s = lmx_s + rows_cap;              // [kAmT] am_max of the tile's frames
