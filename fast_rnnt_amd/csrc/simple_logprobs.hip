@@ -582,8 +582,9 @@ __global__ void __launch_bounds__(kPanThreads)
   // t_end itself only for the -inf that closes the regular lattice): a tile past t_end has
   // nothing to do -- except the tiles of frame 0, which also store the row maxima of lm
   // and the lattice's last column -- and 32-row tiles past s_end are not multiplied.
-  const Limits lim = limits_of(window, b, S, T);
-  if (t_tile > lim.t_end && t_tile > 0) return;
+  // (The window's words are looked at only after the first slab has been requested, so that
+  // the two round trips to memory overlap; a tile that turns out to have nothing to do has
+  // then requested a slab in vain, range-checked like all the others.)
   const float *lmb = lm + (long)b * S1 * C;
   const float *amb = am + (long)b * T * C;
   const int64_t *symb = symbols + (long)b * S;
@@ -658,8 +659,13 @@ __global__ void __launch_bounds__(kPanThreads)
   // per product.  The running maxima are kept beside the shifts, and when the waves
   // meet their partial sums are brought to the true maxima, exp(shift - max) <= 1.
   constexpr float kMargin = 30.f;
+  // (One slab in flight per wave is enough: with a second one the 96-row form was 1 us
+  // slower at B = 32, S = 80, T = 250, C = 500 -- the loop is bound by what it issues, not
+  // by the round trips.)
   floatx4 slab[kLoads];
   if (wave < chunks) fetch(slab, wave * kPanK);
+  const Limits lim = limits_of(window, b, S, T);
+  if (t_tile > lim.t_end && t_tile > 0) return;
 
   // ---- epilogue inputs, requested behind the first slab (the symbols they depend on
   // were requested before it) so that their latency hides under the loop:
