@@ -165,3 +165,69 @@ def test_random_logprob_builders_with_arbitrary_gradients(gpu_device):
         for x, y in zip(got, want):
             assert _close(x, y, 1e-9), it
     assert ran >= 100
+
+
+def test_random_simple_losses_float32(gpu_device):
+    """The float32 kernels of rnnt_loss_simple (the benchmarked path) on seeded random shapes:
+    every output is judged against the float64 oracle and may be off by what the reference's
+    own float32 arithmetic (the oracle in float32) is off, times three, plus a floor of a few
+    ulps -- the occupation gradients are ill-conditioned in px / py
+    (tests/test_oracle_conditioning.py), so a fixed bound would say nothing."""
+    dev = gpu_device
+    rng = random.Random(7)
+    ran = 0
+    for it in range(60):
+        kind = rng.choice(["regular", "modified", "constrained"])
+        B = rng.randint(1, 6)
+        S = rng.choice([rng.randint(1, 40), rng.randint(60, 100), rng.randint(120, 140)])
+        C = rng.choice([3, 17, 64, 100, 257, 500, 515, 1030])
+        T = rng.randint(max(S, 2) if kind != "regular" else 1, 260)
+        red = rng.choice(["none", "mean", "sum"])
+        dp = rng.choice([0.0, 0.0, 0.01])
+        g = torch.Generator().manual_seed(41000 + it)
+        spread = rng.choice([1.0, 1.0, 3.0])
+        am = torch.randn(B, T, C, generator=g) * spread
+        lm = torch.randn(B, S + 1, C, generator=g) * spread
+        sym = torch.randint(0, C, (B, S), generator=g)
+        term = rng.randint(0, C - 1)
+        bnd = None
+        if rng.random() < 0.8:
+            Sb = torch.randint(1, S + 1, (B,), generator=g)
+            Tb = torch.randint(1 if kind == "regular" else S, T + 1, (B,), generator=g)
+            z = torch.zeros(B, dtype=torch.int64)
+            bnd = torch.stack([z, z, Sb, Tb], 1)
+            if rng.random() < 0.3:
+                bnd[:, 0] = torch.minimum(torch.randint(0, 3, (B,), generator=g), Sb)
+                bnd[:, 1] = torch.minimum(torch.randint(0, 3, (B,), generator=g), Tb)
+        w8 = torch.randn(B, generator=g)
+        print(f"float32 case {it}: {kind} B={B} S={S} T={T} C={C} {red} penalty={dp} "
+              f"spread={spread} boundary={None if bnd is None else bnd.tolist()}", flush=True)
+        sys.stdout.flush()
+
+        def run(fn, lm_, am_, to):
+            a, l = to(am_).requires_grad_(True), to(lm_).requires_grad_(True)
+            loss, (gx, gy) = fn(l, a, to(sym), term, boundary=None if bnd is None else to(bnd),
+                                rnnt_type=kind, reduction=red, delay_penalty=dp,
+                                return_grad=True)
+            occ = gx.detach().clone(), gy.detach().clone()
+            ((loss * to(w8.to(loss.dtype))).sum() if red == "none" else loss).backward()
+            return [loss.detach(), occ[0], occ[1], a.grad, l.grad]
+
+        try:
+            truth = run(O.loss_simple, lm.double(), am.double(), lambda x: x.clone())
+            ref32 = run(O.loss_simple, lm, am, lambda x: x.clone())
+        except (AssertionError, RuntimeError) as err:
+            print("   refused by the oracle:", type(err).__name__, flush=True)
+            continue
+        got = run(F.rnnt_loss_simple, lm, am, lambda x: x.to(dev))
+        if not bool(torch.isfinite(truth[0]).all()):
+            continue  # an utterance without a path: nothing to compare gradients on
+        ran += 1
+        for name, x, r, t in zip(("loss", "px_grad", "py_grad", "am.grad", "lm.grad"), got, ref32,
+                                 truth):
+            x = x.cpu().double()
+            scale = max(1.0, t.abs().max().item())
+            err = (x - t).abs().max().item()
+            allowed = 3 * (r.double() - t).abs().max().item() + 8 * 1.2e-7 * scale
+            assert err <= allowed, (it, name, err, allowed)
+    assert ran >= 45
