@@ -20,6 +20,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <array>
+#include <cstring>
 #include <mutex>
 #include <stdexcept>
 #include <string>
